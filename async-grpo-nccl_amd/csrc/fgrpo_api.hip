@@ -1,0 +1,727 @@
+// C ABI of the fused logprob + GRPO path: argument checking, workspace layout
+// and kernel launches.  Declarations and the reference interfaces they replace
+// are in include/fgrpo.h.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+#include <string>
+
+#include "../../include/fgrpo.h"
+#include "tail_kernels.h"
+
+using namespace fgrpo;
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                  \
+  do {                                                                                 \
+    hipError_t e_ = (expr);                                                            \
+    if (e_ != hipSuccess) return fail(FGRPO_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+inline long long round_up(long long x, long long m) { return (x + m - 1) / m * m; }
+inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+// ---- tile configurations ---------------------------------------------------------
+// id 0: 256x256x64, 4 wavefronts of 128x128, one work-group per CU
+// id 1: 256x128x64, 4 wavefronts of 128x64
+// id 2: 256x128x32, 4 wavefronts of 128x64, two work-groups per CU
+// id 3: 256x256x32, 8 wavefronts of 128x64 (two per SIMD)
+// id 4: 128x128x64, 4 wavefronts of 64x64, two work-groups per CU (small problems)
+typedef TileCfg<256, 256, 64, 2, 2, 1> Cfg0;
+typedef TileCfg<256, 128, 64, 2, 2, 1> Cfg1;
+typedef TileCfg<256, 128, 32, 2, 2, 2> Cfg2;
+typedef TileCfg<256, 256, 32, 2, 4, 2> Cfg3;
+typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg4;
+constexpr int kNumCfg = 5;
+
+struct CfgInfo {
+  int bm, bn, bk, nt, lds, wgs_per_cu;
+};
+template <class C>
+constexpr CfgInfo info_of(int wgs) {
+  return CfgInfo{C::BM, C::BN, C::BK, C::NT, C::LDS_BYTES, wgs};
+}
+const CfgInfo kCfg[kNumCfg] = {info_of<Cfg0>(1), info_of<Cfg1>(1), info_of<Cfg2>(2), info_of<Cfg3>(1), info_of<Cfg4>(2)};
+
+struct Tuning {
+  int fwd_variant = 0;
+  int ds_variant = 0;
+  int gemm_variant = 0;
+  int fwd_nsplit = 0;   // 0 = heuristic
+  int fwd_group_t = 8;
+  int ds_group_v = 8;
+  int gemm_group_m = 8;
+  int panel_cols = 32768;  // default vocabulary panel width of the backward
+  int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
+} g_tune;
+
+int* tuning_slot(const char* key) {
+  if (!key) return nullptr;
+  if (!strcmp(key, "fwd_variant")) return &g_tune.fwd_variant;
+  if (!strcmp(key, "ds_variant")) return &g_tune.ds_variant;
+  if (!strcmp(key, "gemm_variant")) return &g_tune.gemm_variant;
+  if (!strcmp(key, "fwd_nsplit")) return &g_tune.fwd_nsplit;
+  if (!strcmp(key, "fwd_group_t")) return &g_tune.fwd_group_t;
+  if (!strcmp(key, "ds_group_v")) return &g_tune.ds_group_v;
+  if (!strcmp(key, "gemm_group_m")) return &g_tune.gemm_group_m;
+  if (!strcmp(key, "panel_cols")) return &g_tune.panel_cols;
+  if (!strcmp(key, "small_variant")) return &g_tune.small_variant;
+  return nullptr;
+}
+
+int num_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
+// Kernels with more than 64 KiB of dynamic LDS need the limit raised once per
+// device and function.
+template <class C, class P>
+int raise_lds(void (*kern)(const P), int bytes) {
+  static bool done[64] = {false};
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev >= 0 && dev < 64 && done[dev]) return 0;
+  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  if (dev >= 0 && dev < 64) done[dev] = true;
+  return 0;
+}
+
+template <class C, class P>
+int launch_tile_kernel(void (*kern)(const P), const P& p, int nblocks, hipStream_t st) {
+  if (nblocks <= 0) return 0;
+  int rc = raise_lds<C, P>(kern, C::LDS_BYTES);
+  if (rc) return rc;
+  hipLaunchKernelGGL(kern, dim3(nblocks), dim3(C::NT), C::LDS_BYTES, st, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int check_operands(const GemmOperands& g, int bk) {
+  if (g.nseg < 1 || g.nseg > 3) return fail(FGRPO_ERR_BAD_ARG, "gemm: nseg=%d", g.nseg);
+  if (g.M <= 0 || g.N <= 0) return fail(FGRPO_ERR_BAD_ARG, "gemm: M=%d N=%d", g.M, g.N);
+  if (g.lda % 8 || g.ldb % 8) return fail(FGRPO_ERR_ALIGN, "gemm: lda=%lld ldb=%lld not multiples of 8", g.lda, g.ldb);
+  for (int s = 0; s < g.nseg; ++s) {
+    if (!g.seg[s].A || !g.seg[s].B) return fail(FGRPO_ERR_BAD_ARG, "gemm: null operand in segment %d", s);
+    if (!aligned16(g.seg[s].A) || !aligned16(g.seg[s].B)) return fail(FGRPO_ERR_ALIGN, "gemm: operand of segment %d not 16-byte aligned", s);
+    if (g.seg[s].K <= 0 || g.seg[s].K % bk) return fail(FGRPO_ERR_UNSUPPORTED, "gemm: K=%d of segment %d not a positive multiple of %d", g.seg[s].K, s, bk);
+    if (g.seg[s].K > g.lda || g.seg[s].K > g.ldb) return fail(FGRPO_ERR_BAD_ARG, "gemm: K=%d exceeds a leading dimension", g.seg[s].K);
+  }
+  // a tile's rows must be addressable with 32-bit byte offsets
+  if (256LL * g.lda * 2 >= (1LL << 32) || 256LL * g.ldb * 2 >= (1LL << 32))
+    return fail(FGRPO_ERR_UNSUPPORTED, "gemm: leading dimension too large");
+  return 0;
+}
+
+int launch_convert(const void* src, int src_is_f32, long long ld_src, int R, int Cn, int Rpad, int Cpad, bf16_t* hi,
+                   bf16_t* lo, long long ld_dst, int transpose, hipStream_t st) {
+  ConvertParams p{src, src_is_f32, ld_src, R, Cn, Rpad, Cpad, hi, lo, ld_dst, transpose};
+  dim3 grid((unsigned)((Cpad + 63) / 64), (unsigned)((Rpad + 63) / 64));
+  if (transpose ? (Rpad > ld_dst) : (Cpad > ld_dst)) return fail(FGRPO_ERR_BAD_ARG, "convert: padded extent exceeds ld");
+  hipLaunchKernelGGL(convert_pad_kernel, grid, dim3(256), 0, st, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// ---- workspace carving -------------------------------------------------------------
+struct Carver {
+  char* base;
+  size_t off = 0;
+  explicit Carver(void* b) : base((char*)b) {}
+  template <class T>
+  T* take(size_t count) {
+    off = (size_t)round_up((long long)off, 256);
+    T* p = base ? (T*)(base + off) : nullptr;
+    off += count * sizeof(T);
+    return p;
+  }
+  size_t total() const { return (size_t)round_up((long long)off, 256); }
+};
+
+int pick_variant(int requested, long long M, long long N) {
+  int v = requested;
+  if (v < 0 || v >= kNumCfg) v = 0;
+  // small problems: a big tile would leave most CUs idle
+  const long long tiles = ((M + kCfg[v].bm - 1) / kCfg[v].bm) * ((N + kCfg[v].bn - 1) / kCfg[v].bn);
+  if (tiles < num_cus() / 2 && g_tune.small_variant >= 0 && g_tune.small_variant < kNumCfg) v = g_tune.small_variant;
+  return v;
+}
+
+// ---- forward plan -------------------------------------------------------------------
+struct FwdPlan {
+  int variant, tiles_v, tiles_t, nsplit;
+  int Hp;            // padded contraction length
+  bool copy_ops;     // operands are staged (fp32 split or padding) instead of used in place
+  bf16_t *w_hi, *w_lo, *h_hi, *h_lo;
+  float* bias32;
+  float4* part;
+  float* xt;
+  size_t bytes;
+};
+
+int choose_nsplit(int tiles_t, int tiles_v, int slots) {
+  if (g_tune.fwd_nsplit > 0) return g_tune.fwd_nsplit < tiles_v ? g_tune.fwd_nsplit : tiles_v;
+  int best = 1;
+  long long best_cost = -1;
+  const int cap = tiles_v < 64 ? tiles_v : 64;
+  for (int s = 1; s <= cap; ++s) {
+    const long long blocks = (long long)tiles_t * s;
+    const long long rounds = (blocks + slots - 1) / slots;
+    const long long per = (tiles_v + s - 1) / s;
+    const long long cost = rounds * per;
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = s;
+    }
+  }
+  return best;
+}
+
+void plan_fwd(FwdPlan& pl, void* ws, int T, int H, int V, int dtype, bool has_bias) {
+  pl.variant = pick_variant(g_tune.fwd_variant, V, T);
+  const CfgInfo& c = kCfg[pl.variant];
+  pl.tiles_v = (V + c.bm - 1) / c.bm;
+  pl.tiles_t = (T + c.bn - 1) / c.bn;
+  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu);
+  pl.Hp = (int)round_up(H, 64);
+  pl.copy_ops = (dtype == FGRPO_F32) || (H % 64 != 0);
+  Carver cv(ws);
+  pl.w_hi = pl.w_lo = pl.h_hi = pl.h_lo = nullptr;
+  if (pl.copy_ops) {
+    pl.w_hi = cv.take<bf16_t>((size_t)V * pl.Hp);
+    pl.h_hi = cv.take<bf16_t>((size_t)T * pl.Hp);
+    if (dtype == FGRPO_F32) {
+      pl.w_lo = cv.take<bf16_t>((size_t)V * pl.Hp);
+      pl.h_lo = cv.take<bf16_t>((size_t)T * pl.Hp);
+    }
+  }
+  pl.bias32 = has_bias ? cv.take<float>((size_t)V) : nullptr;
+  pl.part = cv.take<float4>((size_t)pl.nsplit * T);
+  pl.xt = cv.take<float>((size_t)T);
+  pl.bytes = cv.total();
+}
+
+// Fill the operands of the logits contraction: A = weight side, B = hidden side.
+int stage_logit_operands(GemmOperands& g, const void* hidden, const void* weight, int T, int H, int V, int dtype,
+                         bool copy_ops, int Hp, bf16_t* w_hi, bf16_t* w_lo, bf16_t* h_hi, bf16_t* h_lo, hipStream_t st) {
+  g.M = V;
+  g.N = T;
+  if (!copy_ops) {
+    g.nseg = 1;
+    g.seg[0] = GemmSeg{(const bf16_t*)weight, (const bf16_t*)hidden, H};
+    g.lda = g.ldb = H;
+    return 0;
+  }
+  const int f32 = (dtype == FGRPO_F32);
+  int rc = launch_convert(weight, f32, H, V, H, V, Hp, w_hi, f32 ? w_lo : nullptr, Hp, 0, st);
+  if (rc) return rc;
+  rc = launch_convert(hidden, f32, H, T, H, T, Hp, h_hi, f32 ? h_lo : nullptr, Hp, 0, st);
+  if (rc) return rc;
+  g.lda = g.ldb = Hp;
+  if (f32) {
+    g.nseg = 3;
+    g.seg[0] = GemmSeg{w_hi, h_hi, Hp};
+    g.seg[1] = GemmSeg{w_hi, h_lo, Hp};
+    g.seg[2] = GemmSeg{w_lo, h_hi, Hp};
+  } else {
+    g.nseg = 1;
+    g.seg[0] = GemmSeg{w_hi, h_hi, Hp};
+  }
+  return 0;
+}
+
+template <class C>
+int launch_fwd(const FwdParams& p, hipStream_t st) {
+  return launch_tile_kernel<C>(lmhead_fwd_kernel<C>, p, p.tiles_t * p.nsplit, st);
+}
+template <class C>
+int launch_ds(const DsParams& p, hipStream_t st) {
+  return launch_tile_kernel<C>(lmhead_ds_kernel<C, false>, p, p.tiles_t * p.tiles_v, st);
+}
+// fp32 inputs: dS is written as bf16 hi + lo halves; only the small tile carries that epilogue
+int launch_ds_split(const DsParams& p, hipStream_t st) {
+  return launch_tile_kernel<Cfg4>(lmhead_ds_kernel<Cfg4, true>, p, p.tiles_t * p.tiles_v, st);
+}
+template <class C>
+int launch_store(const StoreParams& p, hipStream_t st) {
+  return launch_tile_kernel<C>(gemm_store_kernel<C>, p, p.tiles_m * p.tiles_n, st);
+}
+
+#define DISPATCH_VARIANT(variant, fn, ...)                \
+  switch (variant) {                                      \
+    case 0: rc = fn<Cfg0>(__VA_ARGS__); break;            \
+    case 1: rc = fn<Cfg1>(__VA_ARGS__); break;            \
+    case 2: rc = fn<Cfg2>(__VA_ARGS__); break;            \
+    case 3: rc = fn<Cfg3>(__VA_ARGS__); break;            \
+    default: rc = fn<Cfg4>(__VA_ARGS__); break;           \
+  }
+
+int run_store_gemm(StoreParams p, int variant, hipStream_t st) {
+  variant = pick_variant(variant, p.g.M, p.g.N);
+  const CfgInfo& c = kCfg[variant];
+  int rc = check_operands(p.g, c.bk);
+  if (rc) return rc;
+  p.tiles_m = (p.g.M + c.bm - 1) / c.bm;
+  p.tiles_n = (p.g.N + c.bn - 1) / c.bn;
+  p.group_m = g_tune.gemm_group_m > 0 ? g_tune.gemm_group_m : 1;
+  DISPATCH_VARIANT(variant, launch_store, p, st);
+  return rc;
+}
+
+// ---- backward plan ------------------------------------------------------------------
+struct BwdPlan {
+  int variant;            // of the dS kernel
+  int bm, bn;
+  int Hp, Tpad, Vpad;     // Tpad, Vpad: multiples of 256
+  int panel, npanels;     // vocabulary rows per panel (multiple of 256)
+  int tiles_t;
+  bool copy_ops, f32;
+  bf16_t *w_hi, *w_lo, *h_hi, *h_lo;          // straight operands (staged only when copy_ops)
+  bf16_t *wT_hi, *wT_lo, *hT_hi, *hT_lo;      // transposed copies [H x Vpad], [H x Tpad]
+  bf16_t *tv_hi, *tv_lo, *vt_hi, *vt_lo;      // dS panels
+  float* bias32;
+  float* dh_acc;                              // [T x H] fp32 when more than one panel
+  size_t bytes;
+};
+
+void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long hint, bool has_bias, bool want_dh,
+              bool want_dw) {
+  pl.f32 = (dtype == FGRPO_F32);
+  pl.variant = pl.f32 ? 4 : pick_variant(g_tune.ds_variant, V, T);
+  pl.bm = kCfg[pl.variant].bm;
+  pl.bn = kCfg[pl.variant].bn;
+  pl.Hp = (int)round_up(H, 64);
+  pl.Tpad = (int)round_up(T, 256);
+  pl.Vpad = (int)round_up(V, 256);
+  pl.tiles_t = (T + pl.bn - 1) / pl.bn;
+  long long cols = g_tune.panel_cols;
+  if (hint > 0) cols = hint / (T > 0 ? T : 1);
+  if (cols < 256) cols = 256;
+  int np = (int)((V + cols - 1) / cols);
+  if (np < 1) np = 1;
+  pl.panel = (int)round_up((V + np - 1) / np, 256);
+  pl.npanels = (V + pl.panel - 1) / pl.panel;
+  pl.copy_ops = pl.f32 || (H % 64 != 0);
+  Carver cv(ws);
+  pl.w_hi = pl.w_lo = pl.h_hi = pl.h_lo = nullptr;
+  if (pl.copy_ops) {
+    pl.w_hi = cv.take<bf16_t>((size_t)V * pl.Hp);
+    pl.h_hi = cv.take<bf16_t>((size_t)T * pl.Hp);
+    if (pl.f32) {
+      pl.w_lo = cv.take<bf16_t>((size_t)V * pl.Hp);
+      pl.h_lo = cv.take<bf16_t>((size_t)T * pl.Hp);
+    }
+  }
+  pl.wT_hi = pl.wT_lo = pl.hT_hi = pl.hT_lo = nullptr;
+  if (want_dh) {
+    pl.wT_hi = cv.take<bf16_t>((size_t)H * pl.Vpad);
+    if (pl.f32) pl.wT_lo = cv.take<bf16_t>((size_t)H * pl.Vpad);
+  }
+  if (want_dw) {
+    pl.hT_hi = cv.take<bf16_t>((size_t)H * pl.Tpad);
+    if (pl.f32) pl.hT_lo = cv.take<bf16_t>((size_t)H * pl.Tpad);
+  }
+  const size_t pe = (size_t)pl.Tpad * pl.panel;
+  pl.tv_hi = cv.take<bf16_t>(pe);
+  pl.vt_hi = cv.take<bf16_t>(pe);
+  pl.tv_lo = pl.vt_lo = nullptr;
+  if (pl.f32) {
+    pl.tv_lo = cv.take<bf16_t>(pe);
+    pl.vt_lo = cv.take<bf16_t>(pe);
+  }
+  pl.bias32 = has_bias ? cv.take<float>((size_t)V) : nullptr;
+  pl.dh_acc = (want_dh && pl.npanels > 1 && !pl.f32) ? cv.take<float>((size_t)T * H) : nullptr;
+  pl.bytes = cv.total();
+}
+
+}  // namespace
+
+// =====================================================================================
+extern "C" {
+
+int fgrpo_version(void) { return 100; }
+const char* fgrpo_last_error(void) { return g_err.c_str(); }
+
+int fgrpo_set_tuning(const char* key, int value) {
+  int* s = tuning_slot(key);
+  if (!s) return fail(FGRPO_ERR_BAD_ARG, "unknown tuning key '%s'", key ? key : "(null)");
+  *s = value;
+  return 0;
+}
+int fgrpo_get_tuning(const char* key) {
+  int* s = tuning_slot(key);
+  if (!s) return fail(FGRPO_ERR_BAD_ARG, "unknown tuning key '%s'", key ? key : "(null)");
+  return *s;
+}
+
+size_t fgrpo_logprob_fwd_workspace(int T, int H, int V, int dtype) {
+  if (T <= 0 || H <= 0 || V <= 0) return 0;
+  FwdPlan pl;
+  plan_fwd(pl, nullptr, T, H, V, dtype, true);
+  return pl.bytes;
+}
+
+int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
+                      int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
+                      size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!hidden || !weight || !labels || !lp_out) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: null argument");
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: T=%d H=%d V=%d", T, H, V);
+  if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: dtype=%d", dtype);
+  if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: inv_temperature must be positive");
+  if (!ws || !aligned16(ws)) return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd: workspace null or misaligned");
+  if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "logprob_fwd: hidden/weight must be 16-byte aligned");
+  FwdPlan pl;
+  plan_fwd(pl, ws, T, H, V, dtype, bias != nullptr);
+  if (pl.bytes > ws_bytes) return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd: workspace %zu < %zu bytes", ws_bytes, pl.bytes);
+
+  FwdParams p;
+  memset(&p, 0, sizeof(p));
+  int rc = stage_logit_operands(p.g, hidden, weight, T, H, V, dtype, pl.copy_ops, pl.Hp, pl.w_hi, pl.w_lo, pl.h_hi,
+                                pl.h_lo, st);
+  if (rc) return rc;
+  rc = check_operands(p.g, kCfg[pl.variant].bk);
+  if (rc) return rc;
+  if (bias) {
+    hipLaunchKernelGGL(to_f32_kernel, dim3((V + 255) / 256), dim3(256), 0, st, bias, dtype == FGRPO_F32, pl.bias32, V);
+    HIP_TRY(hipGetLastError());
+  }
+  p.bias = bias ? pl.bias32 : nullptr;
+  p.labels = (const long long*)labels;
+  p.inv_temp = inv_temp;
+  p.tiles_v = pl.tiles_v;
+  p.tiles_t = pl.tiles_t;
+  p.nsplit = pl.nsplit;
+  p.group_t = g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1;
+  p.part = pl.part;
+  p.xt = pl.xt;
+  DISPATCH_VARIANT(pl.variant, launch_fwd, p, st);
+  if (rc) return rc;
+
+  CombineParams c{pl.part, pl.xt, (const long long*)labels, T, V, pl.nsplit, lp_out, ent_out, lse_out};
+  hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((T + 255) / 256), dim3(256), 0, st, c);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+size_t fgrpo_lmhead_bwd_workspace(int T, int H, int V, int dtype, long long hint) {
+  if (T <= 0 || H <= 0 || V <= 0) return 0;
+  BwdPlan pl;
+  plan_bwd(pl, nullptr, T, H, V, dtype, hint, true, true, true);
+  return pl.bytes;
+}
+
+int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, const int64_t* labels, const float* lse,
+                     const float* g, const float* gout_dev, float inv_temp, int T, int H, int V, int dtype,
+                     void* dH_out, void* dW_out, void* dbias_out, long long hint, void* ws, size_t ws_bytes,
+                     void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!hidden || !weight || !labels || !lse || !g) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd: null argument");
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd: T=%d H=%d V=%d", T, H, V);
+  if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd: dtype=%d", dtype);
+  if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd: inv_temperature must be positive");
+  if (!dH_out && !dW_out && !dbias_out) return 0;
+  if (!ws || !aligned16(ws)) return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd: workspace null or misaligned");
+  if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd: dbias requested without a bias");
+  if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "lmhead_bwd: hidden/weight must be 16-byte aligned");
+  const bool want_dh = dH_out != nullptr, want_dw = dW_out != nullptr;
+  BwdPlan pl;
+  plan_bwd(pl, ws, T, H, V, dtype, hint, bias != nullptr, want_dh, want_dw);
+  if (pl.bytes > ws_bytes) return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd: workspace %zu < %zu bytes", ws_bytes, pl.bytes);
+  const int f32 = pl.f32;
+
+  DsParams d;
+  memset(&d, 0, sizeof(d));
+  int rc = stage_logit_operands(d.g, hidden, weight, T, H, V, dtype, pl.copy_ops, pl.Hp, pl.w_hi, pl.w_lo, pl.h_hi,
+                                pl.h_lo, st);
+  if (rc) return rc;
+  rc = check_operands(d.g, kCfg[pl.variant].bk);
+  if (rc) return rc;
+  if (bias) {
+    hipLaunchKernelGGL(to_f32_kernel, dim3((V + 255) / 256), dim3(256), 0, st, bias, f32, pl.bias32, V);
+    HIP_TRY(hipGetLastError());
+  }
+  // contraction-major copies for the two gradient GEMMs
+  if (want_dh) {
+    rc = launch_convert(weight, f32, H, V, H, pl.Vpad, H, pl.wT_hi, pl.wT_lo, pl.Vpad, 1, st);
+    if (rc) return rc;
+  }
+  if (want_dw) {
+    rc = launch_convert(hidden, f32, H, T, H, pl.Tpad, H, pl.hT_hi, pl.hT_lo, pl.Tpad, 1, st);
+    if (rc) return rc;
+  }
+  d.bias = bias ? pl.bias32 : nullptr;
+  d.labels = (const long long*)labels;
+  d.lse = lse;
+  d.gtok = g;
+  d.gout = gout_dev;
+  d.inv_temp = inv_temp;
+  d.tiles_t = pl.tiles_t;
+  d.group_v = g_tune.ds_group_v > 0 ? g_tune.ds_group_v : 1;
+  d.tv_hi = pl.tv_hi;
+  d.tv_lo = pl.tv_lo;
+  d.vt_hi = pl.vt_hi;
+  d.vt_lo = pl.vt_lo;
+  d.ld_tv = pl.panel;
+  d.ld_vt = pl.Tpad;
+
+  for (int pi = 0; pi < pl.npanels; ++pi) {
+    const int v0 = pi * pl.panel;
+    const int rows = (V - v0) < pl.panel ? (V - v0) : pl.panel;
+    d.v0 = v0;
+    d.tiles_v = (rows + pl.bm - 1) / pl.bm;
+    const int kv = d.tiles_v * pl.bm;        // written panel width
+    const int kt = pl.tiles_t * pl.bn;       // written token extent
+    if (f32) {
+      rc = launch_ds_split(d, st);
+    } else {
+      DISPATCH_VARIANT(pl.variant, launch_ds, d, st);
+    }
+    if (rc) return rc;
+
+    if (want_dh) {  // dH[T x H] (+)= dS_tv[T x kv] * W^T[H x kv]^T
+      StoreParams s;
+      memset(&s, 0, sizeof(s));
+      s.g.M = T;
+      s.g.N = H;
+      s.g.lda = pl.panel;
+      s.g.ldb = pl.Vpad;
+      if (f32) {
+        s.g.nseg = 3;
+        s.g.seg[0] = GemmSeg{pl.tv_hi, pl.wT_hi + v0, kv};
+        s.g.seg[1] = GemmSeg{pl.tv_hi, pl.wT_lo + v0, kv};
+        s.g.seg[2] = GemmSeg{pl.tv_lo, pl.wT_hi + v0, kv};
+      } else {
+        s.g.nseg = 1;
+        s.g.seg[0] = GemmSeg{pl.tv_hi, pl.wT_hi + v0, kv};
+      }
+      s.ldc = H;
+      s.alpha = 1.f;
+      const bool first = (pi == 0), last = (pi == pl.npanels - 1);
+      if (f32) {  // accumulate in the fp32 output itself
+        s.c_in = first ? nullptr : (const float*)dH_out;
+        s.c_out_f32 = (float*)dH_out;
+      } else if (pl.npanels == 1) {
+        s.c_out_bf16 = (bf16_t*)dH_out;
+      } else {
+        s.c_in = first ? nullptr : pl.dh_acc;
+        if (last)
+          s.c_out_bf16 = (bf16_t*)dH_out;
+        else
+          s.c_out_f32 = pl.dh_acc;
+      }
+      rc = run_store_gemm(s, g_tune.gemm_variant, st);
+      if (rc) return rc;
+    }
+    if (want_dw) {  // dW[v0 : v0+rows, H] = dS_vt[rows x kt] * hidden^T[H x kt]^T
+      StoreParams s;
+      memset(&s, 0, sizeof(s));
+      s.g.M = rows;
+      s.g.N = H;
+      s.g.lda = pl.Tpad;
+      s.g.ldb = pl.Tpad;
+      if (f32) {
+        s.g.nseg = 3;
+        s.g.seg[0] = GemmSeg{pl.vt_hi, pl.hT_hi, kt};
+        s.g.seg[1] = GemmSeg{pl.vt_hi, pl.hT_lo, kt};
+        s.g.seg[2] = GemmSeg{pl.vt_lo, pl.hT_hi, kt};
+      } else {
+        s.g.nseg = 1;
+        s.g.seg[0] = GemmSeg{pl.vt_hi, pl.hT_hi, kt};
+      }
+      s.ldc = H;
+      s.alpha = 1.f;
+      if (f32)
+        s.c_out_f32 = (float*)dW_out + (size_t)v0 * H;
+      else
+        s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
+      rc = run_store_gemm(s, g_tune.gemm_variant, st);
+      if (rc) return rc;
+    }
+    if (dbias_out) {
+      float* o32 = f32 ? (float*)dbias_out + v0 : nullptr;
+      bf16_t* o16 = f32 ? nullptr : (bf16_t*)dbias_out + v0;
+      hipLaunchKernelGGL(panel_row_sum_kernel, dim3((rows + 3) / 4), dim3(256), 0, st, pl.vt_hi, pl.vt_lo,
+                         (long long)pl.Tpad, rows, T, o32, o16);
+      HIP_TRY(hipGetLastError());
+    }
+  }
+  return 0;
+}
+
+size_t fgrpo_loss_fwd_workspace(int T, int nseq) {
+  if (T <= 0) return 0;
+  Carver cv(nullptr);
+  cv.take<double>(2 * (size_t)((T + kLossThreads - 1) / kLossThreads));
+  cv.take<float>((size_t)T);
+  cv.take<int>((size_t)(nseq > 0 ? nseq : 1));
+  return cv.total();
+}
+
+int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, const float* adv, const int64_t* labels,
+                   const int32_t* cu, int nseq, int T, float clip_low, float clip_high, float clip_c, float kl_beta,
+                   int agg_mode, double denom_override, float* loss_out, float* g_out, float* log_ratio, float* clip1,
+                   float* unclipped, float* clipped, float* scal_out, void* ws, size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!lp || !adv || !labels || !loss_out || !g_out) return fail(FGRPO_ERR_BAD_ARG, "loss_fwd: null argument");
+  if (T <= 0) return fail(FGRPO_ERR_BAD_ARG, "loss_fwd: T=%d", T);
+  if (agg_mode != FGRPO_AGG_TOKEN_MEAN && agg_mode != FGRPO_AGG_SAMPLE_MEAN)
+    return fail(FGRPO_ERR_BAD_ARG, "loss_fwd: agg_mode=%d", agg_mode);
+  if (agg_mode == FGRPO_AGG_SAMPLE_MEAN && (!cu || nseq <= 0))
+    return fail(FGRPO_ERR_BAD_ARG, "loss_fwd: sample_mean needs cu_seqlens");
+  if (!ws || !aligned16(ws) || ws_bytes < fgrpo_loss_fwd_workspace(T, nseq))
+    return fail(FGRPO_ERR_WORKSPACE, "loss_fwd: workspace too small");
+  const int nblocks = (T + kLossThreads - 1) / kLossThreads;
+  Carver cv(ws);
+  LossParams p;
+  memset(&p, 0, sizeof(p));
+  p.partial = cv.take<double>(2 * (size_t)nblocks);
+  float* tokw = cv.take<float>((size_t)T);
+  int* segc = cv.take<int>((size_t)(nseq > 0 ? nseq : 1));
+  p.lp = lp;
+  p.old_lp = old_lp;
+  p.ref_lp = ref_lp;
+  p.adv = adv;
+  p.labels = (const long long*)labels;
+  p.T = T;
+  p.clip_low = clip_low;
+  p.clip_high = clip_high;
+  p.clip_c = clip_c;
+  p.kl_beta = kl_beta;
+  p.agg_mode = agg_mode;
+  p.denom_override = denom_override;
+  p.g = g_out;
+  p.log_ratio = log_ratio;
+  p.clip1 = clip1;
+  p.unclipped = unclipped;
+  p.clipped = clipped;
+  p.loss = loss_out;
+  p.scal = scal_out;
+  if (agg_mode == FGRPO_AGG_SAMPLE_MEAN) {
+    // tokens outside every segment keep weight 0
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((T + 255) / 256), dim3(256), 0, st, tokw, 0.f, T);
+    HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(segment_valid_weight_kernel, dim3((nseq + 3) / 4), dim3(256), 0, st, p.labels, cu, nseq, segc,
+                       tokw);
+    HIP_TRY(hipGetLastError());
+    p.tokw = tokw;
+    p.seg_cnt = segc;
+    p.nseq = nseq;
+  }
+  hipLaunchKernelGGL(grpo_loss_tokens_kernel, dim3(nblocks), dim3(kLossThreads), 0, st, p);
+  HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(grpo_loss_finalize_kernel, dim3(nblocks), dim3(kLossThreads), 0, st, p, nblocks);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_metrics(const int64_t* idx, int n, int T, const float* log_ratio, const float* entropy,
+                  const float* old_entropy, const float* adv, const float* unclipped, const float* clipped,
+                  float clip_low, float clip_high, double* stats_out, void* stream) {
+  if (!stats_out || n < 0 || T <= 0) return fail(FGRPO_ERR_BAD_ARG, "metrics: bad argument");
+  if (n > 0 && (!idx || !log_ratio || !adv || !unclipped || !clipped)) return fail(FGRPO_ERR_BAD_ARG, "metrics: null argument");
+  MetricParams p{(const long long*)idx, n, T, log_ratio, entropy, old_entropy, adv, unclipped, clipped, clip_low, clip_high, stats_out};
+  hipLaunchKernelGGL(grpo_metrics_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_group_advantages(const void* rewards, int rewards_f64, const int32_t* goff, int ngroups, double eps,
+                           float* out_f32, double* out_f64, void* stream) {
+  if (!rewards || !goff || ngroups <= 0 || (!out_f32 && !out_f64)) return fail(FGRPO_ERR_BAD_ARG, "group_advantages: bad argument");
+  hipLaunchKernelGGL(group_advantage_kernel, dim3((ngroups + 3) / 4), dim3(256), 0, (hipStream_t)stream, rewards,
+                     rewards_f64, goff, ngroups, eps, out_f32, out_f64);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_segment_broadcast(const void* values, int values_f64, const int32_t* cu, int nseq, float* out, void* stream) {
+  if (!values || !cu || !out || nseq <= 0) return fail(FGRPO_ERR_BAD_ARG, "segment_broadcast: bad argument");
+  hipLaunchKernelGGL(segment_broadcast_kernel, dim3((nseq + 3) / 4), dim3(256), 0, (hipStream_t)stream, values,
+                     values_f64, cu, nseq, out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_segment_reduce(const float* x, const int64_t* labels, const int32_t* cu, int nseq, float* sum_out,
+                         float* mean_out, int32_t* count_out, void* stream) {
+  if (!x || !cu || nseq <= 0) return fail(FGRPO_ERR_BAD_ARG, "segment_reduce: bad argument");
+  hipLaunchKernelGGL(segment_reduce_kernel, dim3((nseq + 3) / 4), dim3(256), 0, (hipStream_t)stream, x,
+                     (const long long*)labels, cu, nseq, sum_out, mean_out, count_out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_logits_logprob_entropy(const void* logits, int dtype, long long ld, int N, int V, const int64_t* labels,
+                                 long long ignore_index, int use_ignore, float* lp, float* ent, float* lse,
+                                 void* stream) {
+  if (!logits || N <= 0 || V <= 0 || ld < V) return fail(FGRPO_ERR_BAD_ARG, "logits_logprob_entropy: bad argument");
+  if (lp && !labels) return fail(FGRPO_ERR_BAD_ARG, "logits_logprob_entropy: lp requested without labels");
+  if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "logits_logprob_entropy: dtype=%d", dtype);
+  RowParams p{logits, dtype == FGRPO_F32, ld, N, V, (const long long*)labels, ignore_index, use_ignore, lp, ent, lse};
+  hipLaunchKernelGGL(logits_row_stats_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_logits_logprob_bwd(const void* logits, int dtype, long long ld, int N, int V, const int64_t* labels,
+                             long long ignore_index, int use_ignore, const float* g, const float* lse, void* dlogits,
+                             void* stream) {
+  if (!logits || !labels || !g || !lse || !dlogits || N <= 0 || V <= 0 || ld < V)
+    return fail(FGRPO_ERR_BAD_ARG, "logits_logprob_bwd: bad argument");
+  if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "logits_logprob_bwd: dtype=%d", dtype);
+  RowBwdParams p{{logits, dtype == FGRPO_F32, ld, N, V, (const long long*)labels, ignore_index, use_ignore, nullptr, nullptr, nullptr},
+                 g, lse, dlogits};
+  hipLaunchKernelGGL(logits_row_bwd_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_gemm_nt(const void* A, const void* B, int M, int N, int K, long long lda, long long ldb, const float* c_in,
+                  float* c_out_f32, void* c_out_bf16, long long ldc, float alpha, int variant, void* stream) {
+  if (!A || !B || (!c_out_f32 == !c_out_bf16)) return fail(FGRPO_ERR_BAD_ARG, "gemm_nt: need A, B and exactly one output");
+  if (ldc < N) return fail(FGRPO_ERR_BAD_ARG, "gemm_nt: ldc < N");
+  StoreParams s;
+  memset(&s, 0, sizeof(s));
+  s.g.M = M;
+  s.g.N = N;
+  s.g.lda = lda;
+  s.g.ldb = ldb;
+  s.g.nseg = 1;
+  s.g.seg[0] = GemmSeg{(const bf16_t*)A, (const bf16_t*)B, K};
+  s.c_in = c_in;
+  s.c_out_f32 = c_out_f32;
+  s.c_out_bf16 = (bf16_t*)c_out_bf16;
+  s.ldc = ldc;
+  s.alpha = alpha;
+  if (variant < 0 || variant >= kNumCfg) return fail(FGRPO_ERR_BAD_ARG, "gemm_nt: variant=%d", variant);
+  // the hook runs exactly the requested variant
+  const int keep = g_tune.small_variant;
+  g_tune.small_variant = -1;
+  int rc = run_store_gemm(s, variant, (hipStream_t)stream);
+  g_tune.small_variant = keep;
+  return rc;
+}
+
+}  // extern "C"

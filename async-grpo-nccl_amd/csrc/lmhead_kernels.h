@@ -1,0 +1,479 @@
+// LM-head kernels built on the NT GEMM main loop: vocabulary statistics
+// (forward), dLogits panels (backward recompute) and plain GEMM with a store
+// epilogue (dHidden, dW).  In the two LM-head kernels the MFMA "M" index is the
+// vocabulary and "N" is the token, so one lane owns a single token per 32x32
+// block and 16 vocabulary entries of it: the soft-max statistics reduce inside
+// the lane and need one cross-lane step (lanes l and l^32) at the very end.
+#pragma once
+#include "gemm_core.h"
+
+namespace fgrpo {
+
+constexpr float kNegBig = -1.0e30f;           // stand-in for -inf that keeps 0*x finite
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rn(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+// (m1,s1,x1) (+) (m2,s2,x2) for sums of exp(v - m) and exp(v - m) * v.
+__device__ __forceinline__ void lse_merge(float& m, float& s, float& sx, float m2, float s2, float sx2) {
+  const float mn = m > m2 ? m : m2;
+  const float a1 = fast_exp2((m - mn) * kLog2e), a2 = fast_exp2((m2 - mn) * kLog2e);
+  s = s * a1 + s2 * a2;
+  sx = sx * a1 + sx2 * a2;
+  m = mn;
+}
+
+// ---------------------------------------------------------------------------
+// Forward: per token running (max, sum exp, sum exp*x) over a range of
+// vocabulary tiles + the target logit.
+// ---------------------------------------------------------------------------
+struct FwdParams {
+  GemmOperands g;            // A = W [V x K] (M = V), B = hidden [T x K] (N = T)
+  const float* bias;         // [V] fp32 or null
+  const long long* labels;   // shifted labels [T]; -100 = ignored
+  float inv_temp;
+  int tiles_v, tiles_t, nsplit, group_t;
+  float4* part;              // [nsplit][T] : (m, s, sx, unused)
+  float* xt;                 // [T] target logit (written only where a valid label exists)
+};
+
+template <class C>
+__global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+  const int V = p.g.M, T = p.g.N;
+
+  // block -> (token tile, vocabulary split); neighbours on one XCD share both
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int per_group = p.group_t * p.nsplit;
+  const int grp = lid / per_group;
+  const int first_t = grp * p.group_t;
+  const int gsz = (p.tiles_t - first_t) < p.group_t ? (p.tiles_t - first_t) : p.group_t;
+  const int w = lid - grp * per_group;
+  const int tt = first_t + w % gsz;
+  const int split = w / gsz;
+  const int vt_begin = (int)((long long)split * p.tiles_v / p.nsplit);
+  const int vt_end = (int)((long long)(split + 1) * p.tiles_v / p.nsplit);
+  const int col0 = tt * C::BN;
+
+  float m_run[C::TN], s_run[C::TN], sx_run[C::TN];
+  int y[C::TN];
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) {
+    m_run[j] = kNegBig;
+    s_run[j] = 0.f;
+    sx_run[j] = 0.f;
+    const int n = col0 + acc_col<C>(wn, j, lane);
+    long long lab = (n < T) ? p.labels[n] : -1;
+    y[j] = (lab >= 0 && lab < V) ? (int)lab : -1;
+  }
+
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    const int row0 = vt * C::BM;
+    f32x16_t acc[C::TM][C::TN];
+    zero_acc<C>(acc);
+    gemm_mainloop<C>(p.g, row0, col0, smem, acc);
+
+    const bool edge = row0 + C::BM > V;
+    if (p.bias != nullptr || edge) {
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int v = row0 + acc_row<C>(wm, i, r, lane);
+          const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
+#pragma unroll
+          for (int j = 0; j < C::TN; ++j) {
+            const float x = (acc[i][j][r] + b) * p.inv_temp;
+            acc[i][j][r] = (v < V) ? x : kNegBig;
+          }
+        }
+    } else {
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] *= p.inv_temp;
+    }
+
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      float mt = kNegBig;
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mt = fmaxf(mt, acc[i][j][r]);
+      const float mn = fmaxf(m_run[j], mt);
+      const float alpha = fast_exp2((m_run[j] - mn) * kLog2e);
+      const float mb = mn * kLog2e;
+      float s = s_run[j] * alpha, sx = sx_run[j] * alpha;
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float x = acc[i][j][r];
+          const float e = fast_exp2(__builtin_fmaf(x, kLog2e, -mb));
+          s += e;
+          sx = __builtin_fmaf(e, x, sx);
+        }
+      m_run[j] = mn;
+      s_run[j] = s;
+      sx_run[j] = sx;
+      // target logit: rows of this lane are lane_row0 + i*32 + 8*(r/4) + (r%4)
+      const int yrel = y[j] - row0 - wm * C::WTM - 4 * (lane >> 5);
+      if (y[j] >= 0 && yrel >= 0 && yrel < C::WTM) {
+        float xv = 0.f;
+        bool hit = false;
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const bool h = (yrel == i * 32 + 8 * (r >> 2) + (r & 3));
+            xv = h ? acc[i][j][r] : xv;
+            hit = hit || h;
+          }
+        if (hit) p.xt[col0 + acc_col<C>(wn, j, lane)] = xv;
+      }
+    }
+  }
+
+  // lanes l and l^32 hold the same tokens (different vocabulary rows)
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) {
+    const float m2 = __shfl_xor(m_run[j], 32), s2 = __shfl_xor(s_run[j], 32), x2 = __shfl_xor(sx_run[j], 32);
+    lse_merge(m_run[j], s_run[j], sx_run[j], m2, s2, x2);
+  }
+  // wavefronts stacked along the vocabulary (same wn, different wm) meet in LDS
+  float* red = (float*)smem;  // [WM][BN][3]
+  if (lane < 32) {
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      float* d = red + ((wm * C::BN) + wn * C::WTN + j * 32 + lane) * 3;
+      d[0] = m_run[j];
+      d[1] = s_run[j];
+      d[2] = sx_run[j];
+    }
+  }
+  __syncthreads();
+  for (int c = tid; c < C::BN; c += C::NT) {
+    float m = red[c * 3], s = red[c * 3 + 1], sx = red[c * 3 + 2];
+    for (int q = 1; q < C::WM; ++q) {
+      const float* d = red + (q * C::BN + c) * 3;
+      lse_merge(m, s, sx, d[0], d[1], d[2]);
+    }
+    const int n = col0 + c;
+    if (n < T) p.part[(long long)split * T + n] = make_float4(m, s, sx, 0.f);
+  }
+}
+
+// One thread per token: merge the vocabulary splits, emit logprob / entropy / lse.
+struct CombineParams {
+  const float4* part;
+  const float* xt;
+  const long long* labels;
+  int T, V, nsplit;
+  float* lp;    // [T]
+  float* ent;   // [T] or null
+  float* lse;   // [T] or null
+};
+
+__global__ void lmhead_fwd_combine_kernel(const CombineParams p) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= p.T) return;
+  float4 a = p.part[n];
+  float m = a.x, s = a.y, sx = a.z;
+  for (int k = 1; k < p.nsplit; ++k) {
+    const float4 b = p.part[(long long)k * p.T + n];
+    lse_merge(m, s, sx, b.x, b.y, b.z);
+  }
+  const float lse = m + logf(s);
+  if (p.lse) p.lse[n] = lse;
+  const long long lab = p.labels[n];
+  const bool valid = (lab != -100);
+  float lp = 0.f, ent = 0.f;
+  if (valid) {
+    // a label outside [0, V) has no target logit: report NaN rather than a silent number
+    lp = (lab >= 0 && lab < p.V) ? (p.xt[n] - lse) : __uint_as_float(0x7fc00000u);
+    ent = lse - sx / s;
+  }
+  p.lp[n] = lp;
+  if (p.ent) p.ent[n] = ent;
+}
+
+// ---------------------------------------------------------------------------
+// Backward recompute: dLogits for one vocabulary panel, written as bf16 in
+// both [token][vocab] and [vocab][token] order (the contraction index of the
+// GEMM that consumes each copy is its contiguous index).
+//   dS[t, v] = c_t * (1[v == y_t] - exp(x_tv - lse_t)),  c_t = g_t * gout / temperature
+// Every element of both padded panel buffers is written (zeros outside T x V).
+// ---------------------------------------------------------------------------
+struct DsParams {
+  GemmOperands g;            // A = W [V x K] (M = V), B = hidden [T x K] (N = T)
+  const float* bias;
+  const long long* labels;
+  const float* lse;          // [T]
+  const float* gtok;         // [T] d loss / d logprob
+  const float* gout;         // device scalar (upstream gradient) or null
+  float inv_temp;
+  int v0;                    // first vocabulary row of the panel (multiple of BM)
+  int tiles_v, tiles_t, group_v;
+  bf16_t* tv_hi;             // [tiles_t*BN][ld_tv]
+  bf16_t* tv_lo;             // low half for the fp32 path, or null
+  long long ld_tv;
+  bf16_t* vt_hi;             // [tiles_v*BM][ld_vt]
+  bf16_t* vt_lo;
+  long long ld_vt;
+};
+
+template <class C, bool SPLIT>
+__global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+  const int V = p.g.M, T = p.g.N;
+
+  // grouped raster: group_v vocabulary tiles share the token sweep
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int per_group = p.group_v * p.tiles_t;
+  const int grp = lid / per_group;
+  const int first_v = grp * p.group_v;
+  const int gsz = (p.tiles_v - first_v) < p.group_v ? (p.tiles_v - first_v) : p.group_v;
+  const int w = lid - grp * per_group;
+  const int tv = first_v + w % gsz;
+  const int tt = w / gsz;
+  const int prow0 = tv * C::BM;        // row inside the panel
+  const int row0 = p.v0 + prow0;       // vocabulary row
+  const int col0 = tt * C::BN;
+
+  f32x16_t acc[C::TM][C::TN];
+  zero_acc<C>(acc);
+  gemm_mainloop<C>(p.g, row0, col0, smem, acc);
+
+  if (p.bias != nullptr) {
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int v = row0 + acc_row<C>(wm, i, r, lane);
+        const float b = (v < V) ? p.bias[v] : 0.f;
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) acc[i][j][r] += b;
+      }
+  }
+  // rows of this lane inside the wavefront sub-tile that are real vocabulary entries
+  const int vrem = V - (row0 + wm * C::WTM + 4 * (lane >> 5));  // rr < vrem  <=>  v < V
+  const float go = (p.gout ? *p.gout : 1.f) * p.inv_temp;
+  const float xs = p.inv_temp * kLog2e;
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) {
+    const int n = col0 + acc_col<C>(wn, j, lane);
+    const bool tok_ok = n < T;
+    const float lse2 = tok_ok ? p.lse[n] * kLog2e : 0.f;
+    const long long lab = tok_ok ? p.labels[n] : -100;
+    const float c = (lab != -100) ? p.gtok[n] * go : 0.f;  // ignored tokens carry no gradient
+    // target row relative to this lane's first row; out of range when not in this sub-tile
+    const int yrel = (lab >= 0 && lab < V) ? (int)(lab - row0) - wm * C::WTM - 4 * (lane >> 5) : -1;
+    bf16_t* tv_hi = p.tv_hi + (long long)n * p.ld_tv + prow0 + wm * C::WTM + 4 * (lane >> 5);
+    bf16_t* tv_lo = SPLIT ? p.tv_lo + (long long)n * p.ld_tv + prow0 + wm * C::WTM + 4 * (lane >> 5) : nullptr;
+    bf16_t* vt_hi = p.vt_hi + (long long)(prow0 + wm * C::WTM + 4 * (lane >> 5)) * p.ld_vt + n;
+    bf16_t* vt_lo = SPLIT ? p.vt_lo + (long long)(prow0 + wm * C::WTM + 4 * (lane >> 5)) * p.ld_vt + n : nullptr;
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        uint16_t h[4], l[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int rr = i * 32 + 8 * q + e;  // row relative to the lane's first row
+          float pr = fast_exp2(__builtin_fmaf(acc[i][j][q * 4 + e], xs, -lse2));
+          pr = (rr < vrem) ? pr : 0.f;
+          float ds = -c * pr;
+          ds = (rr == yrel) ? ds + c : ds;
+          h[e] = f32_to_bf16_rn(ds);
+          if (SPLIT) l[e] = f32_to_bf16_rn(ds - bf16_to_f32(h[e]));
+        }
+        const int rr0 = i * 32 + 8 * q;
+        // [token][vocab]: four consecutive vocabulary entries = one 8-byte store
+        uint2 pk;
+        pk.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+        pk.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+        *(uint2*)(tv_hi + rr0) = pk;
+        if (SPLIT) {
+          pk.x = (uint32_t)l[0] | ((uint32_t)l[1] << 16);
+          pk.y = (uint32_t)l[2] | ((uint32_t)l[3] << 16);
+          *(uint2*)(tv_lo + rr0) = pk;
+        }
+        // [vocab][token]: lanes hold consecutive tokens
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vt_hi[(long long)(rr0 + e) * p.ld_vt] = h[e];
+          if (SPLIT) vt_lo[(long long)(rr0 + e) * p.ld_vt] = l[e];
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Plain GEMM with store epilogue: C[m,n] = alpha * sum_k A[m,k] B[n,k] (+ C_in)
+// ---------------------------------------------------------------------------
+struct StoreParams {
+  GemmOperands g;
+  const float* c_in;     // optional fp32 addend, same ldc
+  float* c_out_f32;      // exactly one of c_out_f32 / c_out_bf16 is set
+  bf16_t* c_out_bf16;
+  long long ldc;
+  float alpha;
+  const float* alpha_dev;  // optional device scalar multiplied into alpha
+  int tiles_m, tiles_n, group_m;
+};
+
+// Output is either fp32 or bf16 (never both); rows/cols past M/N are skipped.
+template <class C, bool HAS_IN, bool OUT_BF16>
+__device__ __forceinline__ void store_tile(const StoreParams& p, f32x16_t (&acc)[C::TM][C::TN], float alpha, int row0,
+                                           int col0, int wm, int wn, int lane) {
+  const int mrem = p.g.M - (row0 + wm * C::WTM + 4 * (lane >> 5));  // rr < mrem <=> row valid
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) {
+    const int n = col0 + acc_col<C>(wn, j, lane);
+    if (n < p.g.N) {
+      const long long o0 = (long long)(row0 + wm * C::WTM + 4 * (lane >> 5)) * p.ldc + n;
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rr = i * 32 + 8 * (r >> 2) + (r & 3);
+          if (rr < mrem) {
+            const long long o = o0 + (long long)rr * p.ldc;
+            float v = acc[i][j][r] * alpha;
+            if (HAS_IN) v += p.c_in[o];
+            if (OUT_BF16)
+              p.c_out_bf16[o] = f32_to_bf16_rn(v);
+            else
+              p.c_out_f32[o] = v;
+          }
+        }
+    }
+  }
+}
+
+template <class C>
+__global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StoreParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int per_group = p.group_m * p.tiles_n;
+  const int grp = lid / per_group;
+  const int first_m = grp * p.group_m;
+  const int gsz = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
+  const int w = lid - grp * per_group;
+  const int tm = first_m + w % gsz;
+  const int tn = w / gsz;
+  const int row0 = tm * C::BM, col0 = tn * C::BN;
+
+  f32x16_t acc[C::TM][C::TN];
+  zero_acc<C>(acc);
+  gemm_mainloop<C>(p.g, row0, col0, smem, acc);
+
+  const float alpha = p.alpha * (p.alpha_dev ? *p.alpha_dev : 1.f);
+  const int mode = (p.c_in ? 1 : 0) | (p.c_out_bf16 ? 2 : 0);
+  switch (mode) {
+    case 0: store_tile<C, false, false>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+    case 1: store_tile<C, true, false>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+    case 2: store_tile<C, false, true>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+    default: store_tile<C, true, true>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Operand preparation: copy / transpose a [R x Cn] matrix (fp32 or bf16) into a
+// zero-padded bf16 buffer, optionally also emitting the bf16 low half of an fp32
+// source (x ~= hi + lo).  Destination is [Rpad x ld] (or [Cpad x ld] transposed).
+// ---------------------------------------------------------------------------
+struct ConvertParams {
+  const void* src;
+  int src_is_f32;
+  long long ld_src;
+  int R, Cn;          // logical source shape
+  int Rpad, Cpad;     // padded extents written
+  bf16_t* hi;
+  bf16_t* lo;         // or null
+  long long ld_dst;
+  int transpose;
+};
+
+__global__ __launch_bounds__(256) void convert_pad_kernel(const ConvertParams p) {
+  __shared__ float th[64][65];
+  __shared__ float tl[64][65];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  for (int rr = ty; rr < 64; rr += 4) {
+    const int r = r0 + rr, c = c0 + tx;
+    float v = 0.f;
+    if (r < p.R && c < p.Cn) {
+      const long long o = (long long)r * p.ld_src + c;
+      v = p.src_is_f32 ? ((const float*)p.src)[o] : bf16_to_f32(((const bf16_t*)p.src)[o]);
+    }
+    const float h = bf16_to_f32(f32_to_bf16_rn(v));
+    th[rr][tx] = h;
+    tl[rr][tx] = v - h;
+  }
+  __syncthreads();
+  if (!p.transpose) {
+    for (int rr = ty; rr < 64; rr += 4) {
+      const int r = r0 + rr, c = c0 + tx;
+      if (r < p.Rpad && c < p.Cpad) {
+        const long long o = (long long)r * p.ld_dst + c;
+        p.hi[o] = f32_to_bf16_rn(th[rr][tx]);
+        if (p.lo) p.lo[o] = f32_to_bf16_rn(tl[rr][tx]);
+      }
+    }
+  } else {
+    for (int cc = ty; cc < 64; cc += 4) {
+      const int c = c0 + cc, r = r0 + tx;
+      if (c < p.Cpad && r < p.Rpad) {
+        const long long o = (long long)c * p.ld_dst + r;
+        p.hi[o] = f32_to_bf16_rn(th[tx][cc]);
+        if (p.lo) p.lo[o] = f32_to_bf16_rn(tl[tx][cc]);
+      }
+    }
+  }
+}
+
+__global__ void to_f32_kernel(const void* src, int src_is_f32, float* dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src_is_f32 ? ((const float*)src)[i] : bf16_to_f32(((const bf16_t*)src)[i]);
+}
+
+// bias gradient: db[v] = sum_t dS[v][t] over one [vocab][token] panel
+__global__ void panel_row_sum_kernel(const bf16_t* vt_hi, const bf16_t* vt_lo, long long ld, int rows, int cols,
+                                     float* out_f32, bf16_t* out_bf16) {
+  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  float s = 0.f;
+  for (int c = lane; c < cols; c += 64) {
+    s += bf16_to_f32(vt_hi[(long long)row * ld + c]);
+    if (vt_lo) s += bf16_to_f32(vt_lo[(long long)row * ld + c]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if (lane == 0) {
+    if (out_f32) out_f32[row] = s;
+    if (out_bf16) out_bf16[row] = f32_to_bf16_rn(s);
+  }
+}
+
+}  // namespace fgrpo

@@ -1,0 +1,419 @@
+// Per-token GRPO objective, segmented reductions over cu_seqlens, per-group
+// reward statistics, diagnostics, and the row soft-max kernels that serve
+// callers holding materialised logits.  All of these are HBM-bound streaming
+// kernels (tens of bytes per token); reductions are two-stage with a fixed
+// order so that two runs on the same input are bit-identical.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "lmhead_kernels.h"
+
+namespace fgrpo {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+__global__ void fill_f32_kernel(float* dst, float v, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = v;
+}
+
+// ---------------------------------------------------------------------------
+// Segment (sample) statistics over cu_seqlens: one wavefront per segment.
+// ---------------------------------------------------------------------------
+// cnt[s] = number of valid (label != -100) tokens of segment s; tokw[t] = 1/cnt
+// of the token's segment (0 when the segment has no valid token).
+__global__ void segment_valid_weight_kernel(const long long* labels, const int* cu, int nseq, int* cnt, float* tokw) {
+  const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (s >= nseq) return;
+  const int b = cu[s], e = cu[s + 1];
+  int c = 0;
+  for (int t = b + lane; t < e; t += 64) c += (labels[t] != -100);
+  c = wave_sum_i(c);
+  if (lane == 0) cnt[s] = c;
+  const float w = c > 0 ? 1.0f / (float)c : 0.f;
+  for (int t = b + lane; t < e; t += 64) tokw[t] = w;
+}
+
+// out[t] = values[s] for every token of segment s
+__global__ void segment_broadcast_kernel(const void* values, int values_f64, const int* cu, int nseq, float* out) {
+  const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (s >= nseq) return;
+  const float v = values_f64 ? (float)((const double*)values)[s] : ((const float*)values)[s];
+  for (int t = cu[s] + lane; t < cu[s + 1]; t += 64) out[t] = v;
+}
+
+// sum[s], and mean[s] = sum / count over the (optionally masked) tokens of segment s
+__global__ void segment_reduce_kernel(const float* x, const long long* labels, const int* cu, int nseq, float* sum,
+                                      float* mean, int* count) {
+  const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (s >= nseq) return;
+  float a = 0.f;
+  int c = 0;
+  for (int t = cu[s] + lane; t < cu[s + 1]; t += 64) {
+    const bool ok = labels ? (labels[t] != -100) : true;
+    a += ok ? x[t] : 0.f;
+    c += ok;
+  }
+  a = wave_sum(a);
+  c = wave_sum_i(c);
+  if (lane == 0) {
+    if (sum) sum[s] = a;
+    if (mean) mean[s] = c > 0 ? a / (float)c : 0.f;
+    if (count) count[s] = c;
+  }
+}
+
+// adv[i] = (r[i] - mean_g) / (std_pop_g + eps) per group, double arithmetic
+__global__ void group_advantage_kernel(const void* rewards, int rewards_f64, const int* goff, int ngroups, double eps,
+                                       float* out_f32, double* out_f64) {
+  const int g = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (g >= ngroups) return;
+  const int b = goff[g], e = goff[g + 1];
+  auto rd = [&](int i) -> double {
+    return rewards_f64 ? ((const double*)rewards)[i] : (double)((const float*)rewards)[i];
+  };
+  double s = 0.0;
+  for (int i = b + lane; i < e; i += 64) s += rd(i);
+  s = wave_sum_d(s);
+  const int n = e - b;
+  const double mean = n > 0 ? s / (double)n : 0.0;
+  double q = 0.0;
+  for (int i = b + lane; i < e; i += 64) {
+    const double d = rd(i) - mean;
+    q += d * d;
+  }
+  q = wave_sum_d(q);
+  const double sd = n > 0 ? sqrt(q / (double)n) : 0.0;
+  const double inv = 1.0 / (sd + eps);
+  for (int i = b + lane; i < e; i += 64) {
+    const double a = (rd(i) - mean) * inv;
+    if (out_f32) out_f32[i] = (float)a;
+    if (out_f64) out_f64[i] = a;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// GRPO per-token objective (dual clip, optional k3 KL to a reference policy)
+// ---------------------------------------------------------------------------
+struct LossParams {
+  const float* lp;           // [T] policy logprob (0 on masked tokens)
+  const float* old_lp;       // [T] or null (=> ratio 1)
+  const float* ref_lp;       // [T] or null
+  const float* adv;          // [T]
+  const long long* labels;   // shifted labels [T]
+  const float* tokw;         // [T] per-token weight (sample_mean) or null (token_mean)
+  const int* seg_cnt;        // [nseq] valid tokens per segment (sample_mean) or null
+  int nseq;
+  int T;
+  float clip_low, clip_high, clip_c, kl_beta;
+  int agg_mode;              // 0 token_mean, 1 sample_mean
+  double denom_override;     // > 0: use as normaliser (number of samples / tokens)
+  float* g;                  // [T] d loss / d lp
+  float* log_ratio;          // [T]
+  float* clip1;              // [T]
+  float* unclipped;          // [T]
+  float* clipped;            // [T]
+  double* partial;           // [2 * nblocks] : sum, count
+  float* loss;               // scalar
+  float* scal;               // [4] : normaliser, valid count, nonempty segments, raw sum
+};
+
+constexpr int kLossThreads = 256;
+
+__global__ __launch_bounds__(kLossThreads) void grpo_loss_tokens_kernel(const LossParams p) {
+  __shared__ double sh[2][kLossThreads / 64];
+  const int t = blockIdx.x * kLossThreads + threadIdx.x;
+  float contrib = 0.f;
+  int cnt = 0;
+  if (t < p.T) {
+    const bool valid = p.labels[t] != -100;
+    const float lp = p.lp[t];
+    const float old = p.old_lp ? p.old_lp[t] : lp;
+    const float a = p.adv[t];
+    const float lr = lp - old;
+    const float r = expf(lr);
+    const float lo = 1.0f - p.clip_low, hi = 1.0f + p.clip_high;
+    const float l1 = -a * r;
+    const float rc = fminf(fmaxf(r, lo), hi);
+    const float l2 = -a * rc;
+    const float c1 = fmaxf(l1, l2);
+    const float c2 = fminf(c1, -a * p.clip_c);
+    float tok = (a < 0.f) ? c2 : c1;
+    const bool live = (a > 0.f && r <= hi) || (a < 0.f && r >= lo && r <= p.clip_c);
+    float dtok = live ? -a * r : 0.f;
+    if (p.ref_lp && p.kl_beta != 0.f) {
+      const float d = p.ref_lp[t] - lp;
+      const float ed = expf(d);
+      tok += p.kl_beta * (ed - d - 1.0f);
+      dtok += p.kl_beta * (1.0f - ed);
+    }
+    const float w = valid ? (p.tokw ? p.tokw[t] : 1.0f) : 0.f;
+    p.g[t] = w * dtok;
+    if (p.log_ratio) p.log_ratio[t] = lr;
+    if (p.clip1) p.clip1[t] = c1;
+    if (p.unclipped) p.unclipped[t] = l1;
+    if (p.clipped) p.clipped[t] = l2;
+    contrib = valid ? w * tok : 0.f;
+    cnt = valid;
+  }
+  double s = wave_sum_d((double)contrib);
+  int c = wave_sum_i(cnt);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if (lane == 0) {
+    sh[0][wv] = s;
+    sh[1][wv] = (double)c;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double a = 0.0, b = 0.0;
+    for (int i = 0; i < kLossThreads / 64; ++i) {
+      a += sh[0][i];
+      b += sh[1][i];
+    }
+    p.partial[2 * blockIdx.x] = a;
+    p.partial[2 * blockIdx.x + 1] = b;
+  }
+}
+
+// Every block re-derives the totals from the block partials in the same order,
+// then scales its slice of g by the normaliser; block 0 publishes the scalars.
+__global__ __launch_bounds__(kLossThreads) void grpo_loss_finalize_kernel(const LossParams p, int nparts) {
+  __shared__ double tot[3];
+  if (threadIdx.x < 64) {
+    double a = 0.0, b = 0.0, ne = 0.0;
+    for (int i = threadIdx.x; i < nparts; i += 64) {
+      a += p.partial[2 * i];
+      b += p.partial[2 * i + 1];
+    }
+    if (p.seg_cnt)
+      for (int i = threadIdx.x; i < p.nseq; i += 64) ne += (p.seg_cnt[i] > 0) ? 1.0 : 0.0;
+    a = wave_sum_d(a);
+    b = wave_sum_d(b);
+    ne = wave_sum_d(ne);
+    if (threadIdx.x == 0) {
+      tot[0] = a;
+      tot[1] = b;
+      tot[2] = ne;
+    }
+  }
+  __syncthreads();
+  double den = (p.agg_mode == 0) ? tot[1] : tot[2];
+  if (p.denom_override > 0.0) den = p.denom_override;
+  if (den < 1.0) den = 1.0;
+  const float norm = (float)(1.0 / den);
+  const int t = blockIdx.x * kLossThreads + threadIdx.x;
+  if (t < p.T) p.g[t] *= norm;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *p.loss = (float)(tot[0] / den);
+    if (p.scal) {
+      p.scal[0] = norm;
+      p.scal[1] = (float)tot[1];
+      p.scal[2] = (float)tot[2];
+      p.scal[3] = (float)tot[0];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Diagnostics over the output-token index list, one launch, one result vector.
+// ---------------------------------------------------------------------------
+constexpr int kNumStats = 16;
+struct MetricParams {
+  const long long* idx;      // [n] positions
+  int n;
+  int T;
+  const float* log_ratio;    // [T]
+  const float* entropy;      // [T] or null
+  const float* old_entropy;  // [T] or null
+  const float* adv;          // [T]
+  const float* unclipped;    // [T]
+  const float* clipped;      // [T]
+  float clip_low, clip_high;
+  double* stats;             // [kNumStats]
+};
+
+__global__ __launch_bounds__(1024) void grpo_metrics_kernel(const MetricParams p) {
+  __shared__ double sh[kNumStats][16];
+  double a[kNumStats];
+#pragma unroll
+  for (int k = 0; k < kNumStats; ++k) a[k] = 0.0;
+  for (int i = threadIdx.x; i < p.n; i += 1024) {
+    long long t = p.idx[i];
+    if (t < 0) t += p.T;  // python-style negative index
+    if (t < 0 || t >= p.T) {
+      a[15] += 1.0;  // out-of-range indices are counted, never dereferenced
+      continue;
+    }
+    const float lr = p.log_ratio[t];
+    const float r = expf(lr);
+    const float ad = p.adv[t];
+    a[0] += 1.0;
+    a[1] += fabsf(lr);
+    a[2] += lr;
+    a[3] += (double)lr * lr;
+    a[4] += (r - 1.0f - lr);
+    a[5] += (r > 1.0f + p.clip_high) ? 1.0 : 0.0;
+    a[6] += (r < 1.0f - p.clip_low) ? 1.0 : 0.0;
+    a[7] += p.entropy ? p.entropy[t] : 0.f;
+    a[8] += p.old_entropy ? p.old_entropy[t] : 0.f;
+    a[9] += ad;
+    a[10] += (double)ad * ad;
+    a[11] += (ad > 0.f) ? 1.0 : 0.0;
+    a[12] += (ad == 0.f) ? 1.0 : 0.0;
+    a[13] += (p.clipped[t] > p.unclipped[t]) ? 1.0 : 0.0;
+  }
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < kNumStats; ++k) {
+    const double v = wave_sum_d(a[k]);
+    if (lane == 0) sh[k][wv] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < kNumStats) {
+    double v = 0.0;
+    for (int w = 0; w < 16; ++w) v += sh[threadIdx.x][w];
+    p.stats[threadIdx.x] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Row soft-max statistics on materialised logits [N x V] (bf16 or fp32):
+// logprob of the label, entropy, lse; one work-group per row, one pass.
+// ---------------------------------------------------------------------------
+struct RowParams {
+  const void* logits;
+  int is_f32;
+  long long ld;
+  int N, V;
+  const long long* labels;   // [N] or null; -100 (or `ignore`) = ignored
+  long long ignore;
+  int use_ignore;
+  float* lp;                 // [N] or null
+  float* ent;                // [N] or null
+  float* lse;                // [N] or null
+};
+
+__device__ __forceinline__ float row_load(const RowParams& p, long long row, int v) {
+  const long long o = row * p.ld + v;
+  return p.is_f32 ? ((const float*)p.logits)[o] : bf16_to_f32(((const bf16_t*)p.logits)[o]);
+}
+
+__global__ __launch_bounds__(256) void logits_row_stats_kernel(const RowParams p) {
+  __shared__ float sh[3][4];
+  const long long row = blockIdx.x;
+  float m = kNegBig, s = 0.f, sx = 0.f;
+  const bool vec = (p.ld % 8 == 0) && ((((uintptr_t)p.logits) & 15) == 0);
+  if (!p.is_f32 && vec) {
+    const uint4* base = (const uint4*)((const bf16_t*)p.logits + row * p.ld);
+    const int nv = p.V / 8;
+    for (int c = threadIdx.x; c < nv; c += 256) {
+      const uint4 q = base[c];
+      const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+      float x[8];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        x[2 * k] = __uint_as_float(u[k] << 16);
+        x[2 * k + 1] = __uint_as_float(u[k] & 0xffff0000u);
+      }
+      float mt = x[0];
+#pragma unroll
+      for (int k = 1; k < 8; ++k) mt = fmaxf(mt, x[k]);
+      const float mn = fmaxf(m, mt);
+      const float al = fast_exp2((m - mn) * kLog2e);
+      s *= al;
+      sx *= al;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float e = fast_exp2((x[k] - mn) * kLog2e);
+        s += e;
+        sx = __builtin_fmaf(e, x[k], sx);
+      }
+      m = mn;
+    }
+    for (int v = nv * 8 + threadIdx.x; v < p.V; v += 256) {
+      const float x = row_load(p, row, v);
+      lse_merge(m, s, sx, x, 1.f, x);
+    }
+  } else {
+    for (int v = threadIdx.x; v < p.V; v += 256) {
+      const float x = row_load(p, row, v);
+      lse_merge(m, s, sx, x, 1.f, x);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float m2 = __shfl_xor(m, o), s2 = __shfl_xor(s, o), x2 = __shfl_xor(sx, o);
+    lse_merge(m, s, sx, m2, s2, x2);
+  }
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if (lane == 0) {
+    sh[0][wv] = m;
+    sh[1][wv] = s;
+    sh[2][wv] = sx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) lse_merge(m, s, sx, sh[0][w], sh[1][w], sh[2][w]);
+    const float lse = m + logf(s);
+    if (p.lse) p.lse[row] = lse;
+    if (p.ent) p.ent[row] = lse - sx / s;
+    if (p.lp) {
+      long long lab = p.labels[row];
+      const bool ign = p.use_ignore && lab == p.ignore;
+      float out;
+      if (ign)
+        out = 0.f;
+      else if (lab >= 0 && lab < p.V)
+        out = row_load(p, row, (int)lab) - lse;
+      else
+        out = __uint_as_float(0x7fc00000u);
+      p.lp[row] = out;
+    }
+  }
+}
+
+// dlogits[n, v] = g[n] * (1[v == y_n] - exp(x - lse[n])); ignored rows give 0
+struct RowBwdParams {
+  RowParams f;
+  const float* g;       // [N] upstream gradient of lp
+  const float* lse;     // [N]
+  void* dlogits;        // same dtype/ld as logits
+};
+
+__global__ __launch_bounds__(256) void logits_row_bwd_kernel(const RowBwdParams p) {
+  const long long row = blockIdx.x;
+  const long long lab = p.f.labels[row];
+  const bool ign = p.f.use_ignore && lab == p.f.ignore;
+  const float g = ign ? 0.f : p.g[row];
+  const float l2 = p.lse[row] * kLog2e;
+  for (int v = threadIdx.x; v < p.f.V; v += 256) {
+    const float x = row_load(p.f, row, v);
+    float d = -g * fast_exp2(__builtin_fmaf(x, kLog2e, -l2));
+    if (v == lab) d += g;
+    const long long o = row * p.f.ld + v;
+    if (p.f.is_f32)
+      ((float*)p.dlogits)[o] = d;
+    else
+      ((bf16_t*)p.dlogits)[o] = f32_to_bf16_rn(d);
+  }
+}
+
+}  // namespace fgrpo

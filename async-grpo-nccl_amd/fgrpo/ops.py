@@ -1,0 +1,397 @@
+"""Torch-facing wrappers of the C ABI: allocate outputs and workspaces with
+torch (device memory and streams are torch's), hand raw pointers to the HIP
+library, and wire the forward/backward pair into autograd.
+
+Nothing here computes: every number comes out of ``libfgrpo.so``.  CPU tensors
+are rejected - there is no eager fallback."""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+IGNORE_INDEX = -100
+
+
+# --------------------------------------------------------------------------- helpers
+def _require_cuda(*tensors) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("fgrpo: tensors must live on the GPU (the HIP path has no CPU fallback)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError("fgrpo: all tensors must be on the same device")
+    if dev is None:
+        raise RuntimeError("fgrpo: no tensor given")
+    return dev
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return _lib.BF16
+    if dtype == torch.float32:
+        return _lib.F32
+    raise RuntimeError(f"fgrpo: unsupported dtype {dtype} (bf16 and fp32 only)")
+
+
+def _f32(t: Optional[torch.Tensor], n: int, name: str) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    t = t.detach().reshape(-1)
+    if t.numel() != n:
+        raise RuntimeError(f"fgrpo: {name} has {t.numel()} elements, expected {n}")
+    return t.to(torch.float32).contiguous()
+
+
+def _aligned(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned (a sliced view can start anywhere)."""
+    t = t.detach().contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
+def _ws(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def shift_labels(labels: torch.Tensor) -> torch.Tensor:
+    """labels [..., L] -> next-token targets, -100 in the last column."""
+    return torch.nn.functional.pad(labels, (0, 1), value=IGNORE_INDEX)[..., 1:].contiguous()
+
+
+# --------------------------------------------------------------------------- raw ops
+def lmhead_logprob_fwd(hidden: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                       labels_shifted: torch.Tensor, temperature: float = 1.0,
+                       want_entropy: bool = True, want_lse: bool = True):
+    """hidden [T,H], weight [V,H] (same dtype, bf16 or fp32), labels_shifted [T] int64
+    -> (lp [T] fp32, entropy [T] fp32 | None, lse [T] fp32 | None)."""
+    dev = _require_cuda(hidden, weight, bias, labels_shifted)
+    lib = _lib.load()
+    if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
+        raise RuntimeError(f"fgrpo: hidden {tuple(hidden.shape)} / weight {tuple(weight.shape)} mismatch")
+    if hidden.dtype != weight.dtype:
+        raise RuntimeError("fgrpo: hidden and weight must share a dtype")
+    T, H = hidden.shape
+    V = weight.shape[0]
+    code = _code(weight.dtype)
+    hidden = _aligned(hidden)
+    weight = _aligned(weight)
+    if bias is not None:
+        bias = bias.detach().to(weight.dtype).contiguous()
+        if bias.numel() != V:
+            raise RuntimeError("fgrpo: bias must have V elements")
+    labels_shifted = labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    if labels_shifted.numel() != T:
+        raise RuntimeError("fgrpo: labels must have one entry per token")
+    lp = torch.empty(T, dtype=torch.float32, device=dev)
+    ent = torch.empty(T, dtype=torch.float32, device=dev) if want_entropy else None
+    lse = torch.empty(T, dtype=torch.float32, device=dev) if want_lse else None
+    if T == 0:
+        return lp, ent, lse
+    nbytes = lib.fgrpo_logprob_fwd_workspace(T, H, V, code)
+    ws = _ws(nbytes, dev)
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_logprob_fwd(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted),
+                                   1.0 / float(temperature), T, H, V, code,
+                                   _ptr(lp), _ptr(ent), _ptr(lse), _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "logprob_fwd")
+    return lp, ent, lse
+
+
+def lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torch.Tensor],
+               temperature: float, need_dh: bool, need_dw: bool, need_db: bool,
+               panel_elems_hint: int = 0):
+    """Gradients of the projection+log-softmax+gather given g = d loss / d lp [T].
+    Returns (dH [T,H] | None, dW [V,H] | None, dbias [V] | None) in the input dtype."""
+    dev = _require_cuda(hidden, weight, labels_shifted, lse, g)
+    lib = _lib.load()
+    T, H = hidden.shape
+    V = weight.shape[0]
+    code = _code(weight.dtype)
+    hidden = _aligned(hidden)
+    weight = _aligned(weight)
+    if bias is not None:
+        bias = bias.detach().to(weight.dtype).contiguous()
+    labels_shifted = labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    lse = _f32(lse, T, "lse")
+    g = _f32(g, T, "g")
+    if gout is not None:
+        gout = gout.detach().reshape(-1)[:1].to(device=dev, dtype=torch.float32).contiguous()
+    dH = torch.empty_like(hidden) if need_dh else None
+    dW = torch.empty_like(weight) if need_dw else None
+    db = torch.empty(V, dtype=weight.dtype, device=dev) if (need_db and bias is not None) else None
+    if T == 0 or not (need_dh or need_dw or db is not None):
+        if dW is not None:
+            dW.zero_()
+        if db is not None:
+            db.zero_()
+        return dH, dW, db
+    nbytes = lib.fgrpo_lmhead_bwd_workspace(T, H, V, code, int(panel_elems_hint))
+    ws = _ws(nbytes, dev)
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_lmhead_bwd(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted), _ptr(lse), _ptr(g),
+                                  _ptr(gout), 1.0 / float(temperature), T, H, V, code,
+                                  _ptr(dH), _ptr(dW), _ptr(db), int(panel_elems_hint),
+                                  _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "lmhead_bwd")
+    return dH, dW, db
+
+
+def grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens=None,
+                  clip_low=0.2, clip_high=0.4, clip_ratio_c=1e32, kl_beta=0.0,
+                  loss_agg_mode="token_mean", denom_override: float = 0.0, want_diag: bool = True):
+    """Per-token dual-clip objective on device.
+    Returns (loss [] fp32, g [T], log_ratio, clip1, unclipped, clipped, scal [4])."""
+    dev = _require_cuda(lp, adv, labels_shifted)
+    lib = _lib.load()
+    T = lp.numel()
+    lp = _f32(lp, T, "lp")
+    old_lp = _f32(old_lp, T, "old_logprobs")
+    ref_lp = _f32(ref_lp, T, "ref_logprobs")
+    adv = _f32(adv, T, "advantages")
+    labels_shifted = labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    if loss_agg_mode == "token_mean":
+        agg = _lib.AGG_TOKEN_MEAN
+    elif loss_agg_mode == "sample_mean":
+        agg = _lib.AGG_SAMPLE_MEAN
+        if cu_seqlens is None:
+            raise RuntimeError("fgrpo: loss_agg_mode='sample_mean' needs cu_seqlens")
+    else:
+        raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+    nseq = 0
+    if cu_seqlens is not None:
+        cu_seqlens = cu_seqlens.to(device=dev, dtype=torch.int32).contiguous()
+        nseq = cu_seqlens.numel() - 1
+    mk = lambda: torch.empty(T, dtype=torch.float32, device=dev)
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    g = mk()
+    lr, c1, l1, l2 = (mk(), mk(), mk(), mk()) if want_diag else (None, None, None, None)
+    scal = torch.empty(4, dtype=torch.float32, device=dev)
+    if T == 0:
+        loss.zero_()
+        scal.zero_()
+        return loss, g, lr, c1, l1, l2, scal
+    ws = _ws(lib.fgrpo_loss_fwd_workspace(T, nseq), dev)
+    clamp = lambda x: float(max(min(float(x), 3.0e38), -3.0e38))
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_loss_fwd(_ptr(lp), _ptr(old_lp), _ptr(ref_lp), _ptr(adv), _ptr(labels_shifted),
+                                _ptr(cu_seqlens), nseq, T, clamp(clip_low), clamp(clip_high), clamp(clip_ratio_c),
+                                clamp(kl_beta), agg, float(denom_override),
+                                _ptr(loss), _ptr(g), _ptr(lr), _ptr(c1), _ptr(l1), _ptr(l2), _ptr(scal),
+                                _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "loss_fwd")
+    return loss, g, lr, c1, l1, l2, scal
+
+
+def grpo_metrics(output_indices, log_ratio, entropy, old_entropy, adv, unclipped, clipped,
+                 clip_low: float, clip_high: float) -> torch.Tensor:
+    """One launch, one [16] float64 device vector (layout in include/fgrpo.h)."""
+    dev = _require_cuda(log_ratio, adv)
+    lib = _lib.load()
+    T = log_ratio.numel()
+    idx = output_indices.to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
+    stats = torch.zeros(_lib.NUM_STATS, dtype=torch.float64, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_metrics(_ptr(idx), idx.numel(), T, _ptr(_f32(log_ratio, T, "log_ratio")),
+                               _ptr(_f32(entropy, T, "entropy")), _ptr(_f32(old_entropy, T, "old_entropy")),
+                               _ptr(_f32(adv, T, "advantages")), _ptr(_f32(unclipped, T, "unclipped")),
+                               _ptr(_f32(clipped, T, "clipped")), float(clip_low), float(clip_high),
+                               _ptr(stats), _stream())
+    _lib.check(rc, "metrics")
+    return stats
+
+
+def group_advantages(rewards: torch.Tensor, group_offsets: torch.Tensor, eps: float = 1e-4,
+                     out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """(r - mean) / (population std + eps) per group; rewards fp32/fp64 on device."""
+    dev = _require_cuda(rewards)
+    lib = _lib.load()
+    if rewards.dtype not in (torch.float32, torch.float64):
+        rewards = rewards.to(torch.float64)
+    rewards = rewards.reshape(-1).contiguous()
+    goff = group_offsets.to(device=dev, dtype=torch.int32).contiguous()
+    out = torch.empty(rewards.numel(), dtype=out_dtype, device=dev)
+    if rewards.numel() == 0:
+        return out
+    o32 = _ptr(out) if out_dtype == torch.float32 else None
+    o64 = _ptr(out) if out_dtype == torch.float64 else None
+    if o32 is None and o64 is None:
+        raise RuntimeError("fgrpo: out_dtype must be float32 or float64")
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_group_advantages(_ptr(rewards), int(rewards.dtype == torch.float64), _ptr(goff),
+                                        goff.numel() - 1, float(eps), o32, o64, _stream())
+    _lib.check(rc, "group_advantages")
+    return out
+
+
+def segment_broadcast(values: torch.Tensor, cu_seqlens: torch.Tensor, total: int) -> torch.Tensor:
+    """out[t] = values[segment(t)], fp32 [total]."""
+    dev = _require_cuda(values)
+    lib = _lib.load()
+    if values.dtype not in (torch.float32, torch.float64):
+        values = values.to(torch.float32)
+    values = values.reshape(-1).contiguous()
+    cu = cu_seqlens.to(device=dev, dtype=torch.int32).contiguous()
+    out = torch.zeros(total, dtype=torch.float32, device=dev)
+    if values.numel() == 0:
+        return out
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_segment_broadcast(_ptr(values), int(values.dtype == torch.float64), _ptr(cu), cu.numel() - 1,
+                                         _ptr(out), _stream())
+    _lib.check(rc, "segment_broadcast")
+    return out
+
+
+def segment_reduce(x: torch.Tensor, cu_seqlens: torch.Tensor, labels_shifted: Optional[torch.Tensor] = None):
+    """Per-segment (sum, mean, count) of a per-token fp32 array, masked by labels != -100 when given."""
+    dev = _require_cuda(x)
+    lib = _lib.load()
+    x = x.detach().reshape(-1).to(torch.float32).contiguous()
+    cu = cu_seqlens.to(device=dev, dtype=torch.int32).contiguous()
+    n = cu.numel() - 1
+    s = torch.empty(n, dtype=torch.float32, device=dev)
+    m = torch.empty(n, dtype=torch.float32, device=dev)
+    c = torch.empty(n, dtype=torch.int32, device=dev)
+    lab = None if labels_shifted is None else labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    if n > 0:
+        with torch.cuda.device(dev):
+            rc = lib.fgrpo_segment_reduce(_ptr(x), _ptr(lab), _ptr(cu), n, _ptr(s), _ptr(m), _ptr(c), _stream())
+        _lib.check(rc, "segment_reduce")
+    return s, m, c
+
+
+def logits_logprob_entropy(logits: torch.Tensor, labels: Optional[torch.Tensor], ignore_index: Optional[int],
+                           want_lp=True, want_ent=True, want_lse=True):
+    """Row soft-max statistics of materialised logits [N,V] (bf16/fp32, row stride allowed)."""
+    dev = _require_cuda(logits)
+    lib = _lib.load()
+    code = _code(logits.dtype)
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise RuntimeError("fgrpo: logits must be [N,V] with unit column stride")
+    N, V = logits.shape
+    mk = lambda: torch.empty(N, dtype=torch.float32, device=dev)
+    lp, ent, lse = (mk() if want_lp else None), (mk() if want_ent else None), (mk() if want_lse else None)
+    if N == 0:
+        return lp, ent, lse
+    lab = None if labels is None else labels.reshape(-1).to(torch.int64).contiguous()
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_logits_logprob_entropy(_ptr(logits), code, logits.stride(0), N, V, _ptr(lab),
+                                              int(ignore_index if ignore_index is not None else 0),
+                                              int(ignore_index is not None), _ptr(lp), _ptr(ent), _ptr(lse), _stream())
+    _lib.check(rc, "logits_logprob_entropy")
+    return lp, ent, lse
+
+
+def logits_logprob_bwd(logits, labels, ignore_index, g, lse) -> torch.Tensor:
+    dev = _require_cuda(logits)
+    lib = _lib.load()
+    N, V = logits.shape
+    out = torch.empty((N, V), dtype=logits.dtype, device=dev)
+    if N == 0:
+        return out
+    lab = labels.reshape(-1).to(torch.int64).contiguous()
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_logits_logprob_bwd(_ptr(logits), _code(logits.dtype), logits.stride(0), N, V, _ptr(lab),
+                                          int(ignore_index if ignore_index is not None else 0),
+                                          int(ignore_index is not None), _ptr(_f32(g, N, "g")), _ptr(_f32(lse, N, "lse")),
+                                          _ptr(out), _stream())
+    _lib.check(rc, "logits_logprob_bwd")
+    return out
+
+
+def gemm_nt(A: torch.Tensor, B: torch.Tensor, out_dtype=torch.float32, c_in: Optional[torch.Tensor] = None,
+            alpha: float = 1.0, variant: int = 0) -> torch.Tensor:
+    """Test hook: C = alpha * A @ B.T (+ c_in); A [M,K], B [N,K] bf16, K % 64 == 0."""
+    dev = _require_cuda(A, B)
+    lib = _lib.load()
+    M, K = A.shape
+    N = B.shape[0]
+    A = A.contiguous()
+    B = B.contiguous()
+    out = torch.empty((M, N), dtype=out_dtype, device=dev)
+    o32 = _ptr(out) if out_dtype == torch.float32 else None
+    o16 = _ptr(out) if out_dtype == torch.bfloat16 else None
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_gemm_nt(_ptr(A), _ptr(B), M, N, K, K, K, _ptr(c_in), o32, o16, N, float(alpha), int(variant),
+                               _stream())
+    _lib.check(rc, "gemm_nt")
+    return out
+
+
+# --------------------------------------------------------------------------- autograd
+class _LMHeadLogprob(torch.autograd.Function):
+    """(hidden, weight, bias, labels_shifted) -> (lp, entropy); entropy carries no gradient."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, bias, labels_shifted, temperature, panel_hint):
+        lp, ent, lse = lmhead_logprob_fwd(hidden, weight, bias, labels_shifted, temperature)
+        ctx.save_for_backward(hidden, weight, bias if bias is not None else hidden.new_empty(0), labels_shifted, lse)
+        ctx.has_bias = bias is not None
+        ctx.temperature = temperature
+        ctx.panel_hint = panel_hint
+        ctx.mark_non_differentiable(ent)
+        return lp, ent
+
+    @staticmethod
+    def backward(ctx, g_lp, _g_ent):
+        hidden, weight, bias, labels_shifted, lse = ctx.saved_tensors
+        bias = bias if ctx.has_bias else None
+        dH, dW, db = lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g_lp, None, ctx.temperature,
+                                ctx.needs_input_grad[0], ctx.needs_input_grad[1],
+                                ctx.has_bias and ctx.needs_input_grad[2], ctx.panel_hint)
+        return dH, dW, db, None, None, None
+
+
+class _FusedGRPOLoss(torch.autograd.Function):
+    """Projection -> logprob -> dual-clip objective in one autograd node.  The
+    backward receives the scalar upstream gradient as a device pointer."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens, temperature,
+                clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode, denom_override, panel_hint):
+        lp, ent, lse = lmhead_logprob_fwd(hidden, weight, bias, labels_shifted, temperature)
+        loss, g, lr, c1, l1, l2, scal = grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
+                                                      clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
+                                                      denom_override)
+        ctx.save_for_backward(hidden, weight, bias if bias is not None else hidden.new_empty(0), labels_shifted,
+                              lse, g)
+        ctx.has_bias = bias is not None
+        ctx.temperature = temperature
+        ctx.panel_hint = panel_hint
+        ctx.mark_non_differentiable(ent, lr, c1, l1, l2, lp)
+        return loss, ent, lr, c1, l1, l2, lp
+
+    @staticmethod
+    def backward(ctx, g_loss, *_unused):
+        hidden, weight, bias, labels_shifted, lse, g = ctx.saved_tensors
+        bias = bias if ctx.has_bias else None
+        dH, dW, db = lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, g_loss, ctx.temperature,
+                                ctx.needs_input_grad[0], ctx.needs_input_grad[1],
+                                ctx.has_bias and ctx.needs_input_grad[2], ctx.panel_hint)
+        return (dH, dW, db) + (None,) * 13
+
+
+def lmhead_logprob(hidden, weight, bias, labels_shifted, temperature=1.0, panel_hint=0) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint))
+
+
+def fused_grpo_loss(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp=None, cu_seqlens=None,
+                    temperature=1.0, clip_low=0.2, clip_high=0.4, clip_ratio_c=1e32, kl_beta=0.0,
+                    loss_agg_mode="token_mean", denom_override=0.0, panel_hint=0):
+    """(loss, entropy, log_ratio, clip1, unclipped, clipped, lp); only loss carries a gradient."""
+    return _FusedGRPOLoss.apply(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens,
+                                float(temperature), float(clip_low), float(clip_high), float(clip_ratio_c),
+                                float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint))

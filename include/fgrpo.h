@@ -1,0 +1,150 @@
+/* fgrpo: C ABI of the MI355X (gfx950) fused logprob + GRPO hot path.
+ *
+ * Plain pointers and sizes only; every pointer named *_dev / every array is
+ * DEVICE memory unless the comment says host.  Every call is asynchronous on
+ * `stream` (a hipStream_t passed as void*), allocates nothing and keeps no
+ * state between calls except tuning knobs.  Return value: 0 on success, a
+ * negative FGRPO_ERR_* otherwise; fgrpo_last_error() gives the message of the
+ * calling thread's last failure.
+ *
+ * Each entry point names the reference interface it replaces
+ * (paths relative to the reference repository engineerA314/async-grpo-nccl).
+ */
+#ifndef FGRPO_H
+#define FGRPO_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FGRPO_OK 0
+#define FGRPO_ERR_BAD_ARG (-1)     /* null pointer, non-positive size, bad enum */
+#define FGRPO_ERR_UNSUPPORTED (-2) /* shape/dtype outside what the kernels handle */
+#define FGRPO_ERR_WORKSPACE (-3)   /* workspace missing, misaligned or too small */
+#define FGRPO_ERR_HIP (-4)         /* a HIP runtime call failed */
+#define FGRPO_ERR_ALIGN (-5)       /* operand base not 16-byte aligned */
+
+#define FGRPO_BF16 0
+#define FGRPO_F32 1
+
+#define FGRPO_AGG_TOKEN_MEAN 0
+#define FGRPO_AGG_SAMPLE_MEAN 1
+
+#define FGRPO_NUM_STATS 16
+
+int fgrpo_version(void);
+const char* fgrpo_last_error(void);
+
+/* Tuning knobs (kernel variant ids, vocabulary splits, raster groups).  Unknown
+ * keys return FGRPO_ERR_BAD_ARG.  Not part of the reference interface. */
+int fgrpo_set_tuning(const char* key, int value);
+int fgrpo_get_tuning(const char* key);
+
+/* ---- LM-head projection -> log-softmax -> target gather (+ entropy) --------
+ * Replaces the body of fused_log_probs_and_entropy_fn (grpo_loss.py:211-250)
+ * and the chunk loop of grpo_loss_and_entropy_ce_fn (grpo_loss.py:286-313):
+ *   x_t = (W h_t + b) * inv_temperature
+ *   lp_t  = [y_t != -100] * (x_t[y_t] - logsumexp x_t)
+ *   ent_t = [y_t != -100] * (logsumexp x_t - sum softmax(x_t) x_t)
+ * hidden [T x H], weight [V x H] row-major in `dtype`; bias [V] in `dtype` or
+ * NULL; labels_shifted [T] int64 (already shifted by one, -100 = ignored).
+ * lp_out/ent_out/lse_out: fp32 [T]; ent_out and lse_out may be NULL.
+ * The [T x V] logits never exist in memory. */
+size_t fgrpo_logprob_fwd_workspace(int T, int H, int V, int dtype);
+int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias,
+                      const int64_t* labels_shifted, float inv_temperature,
+                      int T, int H, int V, int dtype,
+                      float* lp_out, float* ent_out, float* lse_out,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- backward of the above (what autograd derives from grpo_loss.py:290-296
+ * through torch.matmul / gather / logsumexp):
+ *   dX_t = g_t * gout * inv_temperature * (onehot(y_t) - softmax(x_t))
+ *   dH = dX W ; dW = dX^T H ; dbias = sum_t dX_t
+ * Logits are recomputed per tile; only one vocabulary panel of dX (bf16) lives
+ * in the workspace at a time.  g [T] fp32 = d loss / d lp; gout_dev = device
+ * scalar with the upstream gradient of the loss (NULL = 1); lse [T] from the
+ * forward.  dH_out [T x H], dW_out [V x H], dbias_out [V] in `dtype`; each may
+ * be NULL.  panel_elems_hint: upper bound on T*panel_width (<=0 = default). */
+size_t fgrpo_lmhead_bwd_workspace(int T, int H, int V, int dtype, long long panel_elems_hint);
+int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
+                     const int64_t* labels_shifted, const float* lse, const float* g,
+                     const float* gout_dev, float inv_temperature,
+                     int T, int H, int V, int dtype,
+                     void* dH_out, void* dW_out, void* dbias_out,
+                     long long panel_elems_hint,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- per-token GRPO objective -------------------------------------------------
+ * Replaces the tail of grpo_loss_and_entropy_ce_fn (grpo_loss.py:318-348):
+ * ratio, dual clip, masked mean.  old_lp NULL => ratio 1 (grpo_loss.py:318-319).
+ * Extensions not in the reference: ref_lp/kl_beta (k3 KL penalty per token) and
+ * agg_mode SAMPLE_MEAN over cu_seqlens [nseq+1] int32 (mean over samples of the
+ * per-sample token mean); denom_override > 0 replaces the normaliser.
+ * Outputs (fp32): loss_out scalar; g_out [T] = d loss / d lp; log_ratio, clip1,
+ * unclipped, clipped [T] (each may be NULL); scal_out [4] (may be NULL) =
+ * {1/normaliser, valid tokens, non-empty samples, unnormalised sum}. */
+size_t fgrpo_loss_fwd_workspace(int T, int nseq);
+int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, const float* adv,
+                   const int64_t* labels_shifted, const int32_t* cu_seqlens, int nseq, int T,
+                   float clip_low, float clip_high, float clip_ratio_c, float kl_beta,
+                   int agg_mode, double denom_override,
+                   float* loss_out, float* g_out, float* log_ratio, float* clip1,
+                   float* unclipped, float* clipped, float* scal_out,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- diagnostics on the output-token positions ---------------------------------
+ * Replaces the ~20 .item() reductions of compute_dual_clip_grpo_loss
+ * (grpo_loss.py:408-498) with one launch.  idx [n] int64 positions into the
+ * [T] arrays.  stats_out: FGRPO_NUM_STATS doubles =
+ * {n, sum|lr|, sum lr, sum lr^2, sum(r-1-lr), #(r>1+hi), #(r<1-lo), sum ent,
+ *  sum old_ent, sum adv, sum adv^2, #(adv>0), #(adv==0), #(clipped>unclipped),
+ *  0, #out-of-range idx}. */
+int fgrpo_metrics(const int64_t* idx, int n, int T, const float* log_ratio, const float* entropy,
+                  const float* old_entropy, const float* adv, const float* unclipped,
+                  const float* clipped, float clip_low, float clip_high,
+                  double* stats_out, void* stream);
+
+/* ---- group-normalised advantages ------------------------------------------------
+ * Replaces vllm_worker.py:788-796 (and normalize_rewards, :77-92):
+ * (r - mean) / (population std + eps) per group; group_offsets [ngroups+1] int32.
+ * rewards fp32 or fp64 (rewards_f64 != 0); out_f32 / out_f64 may be NULL. */
+int fgrpo_group_advantages(const void* rewards, int rewards_f64, const int32_t* group_offsets,
+                           int ngroups, double eps, float* out_f32, double* out_f64, void* stream);
+
+/* ---- segmented helpers over cu_seqlens [nseq+1] int32 ---------------------------
+ * fgrpo_segment_broadcast replaces broadcast_values (sample_processing_utils.py:69-105):
+ * out[t] = values[s(t)].  fgrpo_segment_reduce gives per-sample sums / means /
+ * counts of a per-token array, masked by labels != -100 when labels is given. */
+int fgrpo_segment_broadcast(const void* values, int values_f64, const int32_t* cu_seqlens, int nseq,
+                            float* out, void* stream);
+int fgrpo_segment_reduce(const float* x, const int64_t* labels, const int32_t* cu_seqlens, int nseq,
+                         float* sum_out, float* mean_out, int32_t* count_out, void* stream);
+
+/* ---- row soft-max on materialised logits ----------------------------------------
+ * Replaces logprobs_from_logits (grpo_loss.py:146-173) and entropy_from_logits
+ * (grpo_loss.py:203-208) for callers that already hold logits [N x V] (ld =
+ * row stride in elements).  labels may be NULL when lp is NULL.  use_ignore = 0
+ * disables the ignore_index test.  The backward writes
+ * dlogits = g (onehot - softmax) in the logits' dtype. */
+int fgrpo_logits_logprob_entropy(const void* logits, int dtype, long long ld, int N, int V,
+                                 const int64_t* labels, long long ignore_index, int use_ignore,
+                                 float* lp, float* ent, float* lse, void* stream);
+int fgrpo_logits_logprob_bwd(const void* logits, int dtype, long long ld, int N, int V,
+                             const int64_t* labels, long long ignore_index, int use_ignore,
+                             const float* g, const float* lse, void* dlogits, void* stream);
+
+/* ---- test hook: the GEMM core on its own -----------------------------------------
+ * C[m,n] = alpha * sum_k A[m,k] B[n,k] (+ c_in); A [M x K], B [N x K] bf16,
+ * K a multiple of 64.  No counterpart in the reference. */
+int fgrpo_gemm_nt(const void* A, const void* B, int M, int N, int K, long long lda, long long ldb,
+                  const float* c_in, float* c_out_f32, void* c_out_bf16, long long ldc, float alpha,
+                  int variant, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FGRPO_H */
