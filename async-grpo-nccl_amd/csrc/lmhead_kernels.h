@@ -115,7 +115,9 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
         for (int r = 0; r < 16; ++r) mt = fmaxf(mt, acc[i][j][r]);
       const float mn = fmaxf(m_run[j], mt);
       const float alpha = fast_exp2((m_run[j] - mn) * kLog2e);
-      const float mb = mn * kLog2e;
+      // a slot that has seen only masked rows keeps (m, s, sx) = (kNegBig, 0, 0):
+      // x*log2e - mb would otherwise be the rounding residue of two 1e30-sized terms
+      const float mb = (mn > 0.5f * kNegBig) ? mn * kLog2e : 0.f;
       float s = s_run[j] * alpha, sx = sx_run[j] * alpha;
 #pragma unroll
       for (int i = 0; i < C::TM; ++i)
