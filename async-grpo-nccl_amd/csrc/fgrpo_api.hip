@@ -673,6 +673,24 @@ int fgrpo_segment_reduce(const float* x, const int64_t* labels, const int32_t* c
   return 0;
 }
 
+int fgrpo_output_indices(const int32_t* tok_off, const int32_t* in_len, const int32_t* out_off, int nsamples,
+                         int64_t* out, void* stream) {
+  if (!tok_off || !in_len || !out_off || !out || nsamples <= 0) return fail(FGRPO_ERR_BAD_ARG, "output_indices: bad argument");
+  hipLaunchKernelGGL(output_indices_kernel, dim3((nsamples + 3) / 4), dim3(256), 0, (hipStream_t)stream, tok_off, in_len,
+                     out_off, nsamples, (long long*)out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_segment_starts(const int64_t* position_ids, int T, int32_t* cu_out, int max_out, int32_t* count_out,
+                         void* stream) {
+  if (!position_ids || !cu_out || !count_out || T <= 0 || max_out <= 0) return fail(FGRPO_ERR_BAD_ARG, "segment_starts: bad argument");
+  hipLaunchKernelGGL(segment_starts_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const long long*)position_ids,
+                     T, cu_out, max_out, count_out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 int fgrpo_logits_logprob_entropy(const void* logits, int dtype, long long ld, int N, int V, const int64_t* labels,
                                  long long ignore_index, int use_ignore, float* lp, float* ent, float* lse,
                                  void* stream) {

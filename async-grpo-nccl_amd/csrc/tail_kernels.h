@@ -80,6 +80,56 @@ __global__ void segment_reduce_kernel(const float* x, const long long* labels, c
   }
 }
 
+// Positions of the logits that score each sample's generated tokens: sample i,
+// packed at token offset tok_off[i], contributes
+//   tok_off[i] + in_len[i] - 1 + j   for j in [0, out_len[i])
+// written at out_off[i] + j.  One wavefront per sample.
+__global__ void output_indices_kernel(const int* tok_off, const int* in_len, const int* out_off, int nsamples,
+                                      long long* out) {
+  const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (s >= nsamples) return;
+  const int n = out_off[s + 1] - out_off[s];
+  const long long first = (long long)tok_off[s] + in_len[s] - 1;
+  for (int j = lane; j < n; j += 64) out[out_off[s] + j] = first + j;
+}
+
+// cu_seqlens from position ids: ordered list of the indices t with pos[t] == 0,
+// followed by T.  A single work-group walks the array in order; within a chunk
+// the rank of a hit is a ballot prefix, so the output order is the token order.
+// out has room for max_out entries; *count receives the number of boundaries
+// found + 1 (even when it exceeds max_out, in which case the tail is dropped).
+__global__ __launch_bounds__(1024) void segment_starts_kernel(const long long* pos, int T, int* out, int max_out,
+                                                              int* count) {
+  __shared__ int wave_cnt[16];
+  __shared__ int base;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if (threadIdx.x == 0) base = 0;
+  __syncthreads();
+  for (int t0 = 0; t0 < T; t0 += 1024) {
+    const int t = t0 + threadIdx.x;
+    const bool hit = (t < T) && (pos[t] == 0);
+    const unsigned long long b = __ballot(hit);
+    const int rank = __popcll(b & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_cnt[wv] = __popcll(b);
+    __syncthreads();
+    int off = base;
+    for (int w = 0; w < wv; ++w) off += wave_cnt[w];
+    if (hit && off + rank < max_out) out[off + rank] = t;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int tot = 0;
+      for (int w = 0; w < 16; ++w) tot += wave_cnt[w];
+      base += tot;
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    if (base < max_out) out[base] = T;
+    *count = base + 1;
+  }
+}
+
 // adv[i] = (r[i] - mean_g) / (std_pop_g + eps) per group, double arithmetic
 __global__ void group_advantage_kernel(const void* rewards, int rewards_f64, const int* goff, int ngroups, double eps,
                                        float* out_f32, double* out_f64) {

@@ -34,6 +34,8 @@ SIGNATURES = {
     "fgrpo_group_advantages": (_i, [_vp, _i, _vp, _i, _d, _vp, _vp, _vp]),
     "fgrpo_segment_broadcast": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "fgrpo_segment_reduce": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp]),
+    "fgrpo_output_indices": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
+    "fgrpo_segment_starts": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "fgrpo_logits_logprob_entropy": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _vp]),
     "fgrpo_logits_logprob_bwd": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _vp]),
     "fgrpo_gemm_nt": (_i, [_vp, _vp, _i, _i, _i, _ll, _ll, _vp, _vp, _vp, _ll, _f, _i, _vp]),

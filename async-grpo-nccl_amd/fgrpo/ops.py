@@ -273,6 +273,51 @@ def segment_reduce(x: torch.Tensor, cu_seqlens: torch.Tensor, labels_shifted: Op
     return s, m, c
 
 
+def output_indices(input_lens, output_lens, device) -> torch.Tensor:
+    """int64 positions of the logits scoring every generated token (see fgrpo_output_indices)."""
+    lib = _lib.load()
+    il = torch.as_tensor(input_lens, dtype=torch.int64).reshape(-1)
+    ol = torch.as_tensor(output_lens, dtype=torch.int64).reshape(-1)
+    n = il.numel()
+    tok_off = torch.zeros(n, dtype=torch.int64)
+    out_off = torch.zeros(n + 1, dtype=torch.int64)
+    if n:
+        tok_off[1:] = torch.cumsum(il + ol, 0)[:-1]
+        out_off[1:] = torch.cumsum(ol, 0)
+    total = int(out_off[-1])
+    out = torch.empty(total, dtype=torch.int64, device=device)
+    if n == 0 or total == 0:
+        return out
+    if int((il + ol).sum()) >= 2 ** 31:
+        raise RuntimeError("fgrpo: packed batch longer than 2^31 tokens")
+    pack = torch.cat([tok_off.to(torch.int32), il.to(torch.int32), out_off.to(torch.int32)]).to(device)
+    with torch.cuda.device(device):
+        rc = lib.fgrpo_output_indices(pack.data_ptr(), pack.data_ptr() + 4 * n, pack.data_ptr() + 8 * n, n,
+                                      _ptr(out), _stream())
+    _lib.check(rc, "output_indices")
+    return out
+
+
+def cu_seqlens_from_position_ids(position_ids: torch.Tensor, max_segments: Optional[int] = None) -> torch.Tensor:
+    """int32 [n+1]: indices where position_ids == 0, then T (one host sync for n)."""
+    dev = _require_cuda(position_ids)
+    lib = _lib.load()
+    pos = position_ids.reshape(-1).to(torch.int64).contiguous()
+    T = pos.numel()
+    cap = (max_segments if max_segments is not None else T) + 1
+    out = torch.empty(cap, dtype=torch.int32, device=dev)
+    cnt = torch.zeros(1, dtype=torch.int32, device=dev)
+    if T == 0:
+        return torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_segment_starts(_ptr(pos), T, _ptr(out), cap, _ptr(cnt), _stream())
+    _lib.check(rc, "segment_starts")
+    n = int(cnt.item())
+    if n > cap:
+        raise RuntimeError(f"fgrpo: {n - 1} segments exceed max_segments={cap - 1}")
+    return out[:n]
+
+
 def logits_logprob_entropy(logits: torch.Tensor, labels: Optional[torch.Tensor], ignore_index: Optional[int],
                            want_lp=True, want_ent=True, want_lse=True):
     """Row soft-max statistics of materialised logits [N,V] (bf16/fp32, row stride allowed)."""

@@ -1,0 +1,171 @@
+"""Drop-in for the batch-shaping functions of the reference module
+``sample_processing_utils.py``: a list of sample dicts becomes padding-free
+``1 x T`` device tensors plus the per-token broadcasts the trainer consumes.
+
+The reference expands per-sample scalars on the CPU with numba loops and copies
+the expanded arrays to the GPU (sample_processing_utils.py:29-105, :159-223).
+Here only per-sample arrays and the token lists cross PCIe; the expansion
+(``output_indices``, advantage and length broadcasts) runs in HIP kernels over
+``cu_seqlens``.  ``device`` must be a GPU: there is no CPU path.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import numpy as np
+import torch
+
+from fgrpo import ops
+
+
+def _lens(batched_questions):
+    il = np.fromiter((s["input_len"] for s in batched_questions), dtype=np.int64, count=len(batched_questions))
+    ol = np.fromiter((s["output_len"] for s in batched_questions), dtype=np.int64, count=len(batched_questions))
+    return il, ol
+
+
+def get_output_logits_indices_numba(input_lens, output_lens):
+    """Host reference form kept for callers that want a numpy array
+    (reference: sample_processing_utils.py:29-67), vectorised: sample i starting
+    at offset o_i yields o_i + Lin_i - 1 + [0, Lout_i)."""
+    il = np.asarray(input_lens, dtype=np.int64)
+    ol = np.asarray(output_lens, dtype=np.int64)
+    start = np.concatenate(([0], np.cumsum(il + ol)[:-1])) + il - 1 if il.size else np.zeros(0, np.int64)
+    first = np.repeat(start, ol)
+    within = np.arange(int(ol.sum()), dtype=np.int64) - np.repeat(np.cumsum(ol) - ol, ol)
+    return (first + within).astype(np.int64)
+
+
+def broadcast_values(values, output_lens):
+    """float64 repeat of per-sample scalars (reference: sample_processing_utils.py:69-105)."""
+    return np.repeat(np.asarray(values, dtype=np.float64), np.asarray(output_lens, dtype=np.int64))
+
+
+def get_output_logits_indices(batched_questions, device):
+    """(output_indices on device, output_lens) - reference: sample_processing_utils.py:107-112."""
+    il, ol = _lens(batched_questions)
+    return ops.output_indices(il, ol, device), ol
+
+
+def get_input_for_logprobs(batched_questions, output_indices, device):
+    """Concatenated ids / position ids / labels as [1, T] int64 device tensors
+    (reference: sample_processing_utils.py:114-125).  One pinned staging buffer,
+    one copy."""
+    n_tok = sum(len(s["sample_ids"]) for s in batched_questions)
+    host = torch.empty((3, n_tok), dtype=torch.long).pin_memory() if n_tok else torch.empty((3, 0), dtype=torch.long)
+    off = 0
+    for s in batched_questions:
+        k = len(s["sample_ids"])
+        host[0, off:off + k] = torch.as_tensor(s["sample_ids"], dtype=torch.long)
+        host[1, off:off + k] = torch.as_tensor(s["sample_position_ids"], dtype=torch.long)
+        host[2, off:off + k] = torch.as_tensor(s["labels"], dtype=torch.long)
+        off += k
+    dev = host.to(device, non_blocking=True)
+    return dev[0:1], dev[1:2], dev[2:3]
+
+
+def make_dummy_batch(batched_questions, device):
+    """All-masked 4-token placeholder that keeps lock-step ranks busy without
+    touching the metrics (reference: sample_processing_utils.py:127-157)."""
+    ids = [11, 12, 13, 14]
+    z = lambda: torch.tensor(0.0, device=device, dtype=torch.float32)
+    n = len(ids)
+    return {
+        "batch_ids": torch.tensor([ids], dtype=torch.long, device=device),
+        "batch_position_ids": torch.arange(n, device=device).unsqueeze(0),
+        "output_indices": torch.empty((0,), dtype=torch.long, device=device),
+        "advantages": torch.zeros(n, device=device, dtype=torch.float32),
+        "reference_output_logprobs": torch.zeros(n, device=device, dtype=torch.float32),
+        "output_lens_broadcasted": torch.zeros(n, device=device, dtype=torch.float32),
+        "num_output_tokens_non_masked": z(),
+        "num_output_tokens": z(),
+        "num_samples": z(),
+        "max_reward_in_group": z(),
+        "total_modified_reward": z(),
+        "total_non_modified_reward": z(),
+        "num_modified_samples": z(),
+        "delimiter_not_found": z(),
+        "samples": batched_questions,
+        "labels": torch.full((1, n), -100, dtype=torch.long, device=device),
+        "total_reward_rank": z(),
+        "truncated_sample": z(),
+        "advantage_is_zero": z(),
+    }
+
+
+def post_process_batch(batched_questions, device, constant_length_samples=None):
+    """Pack samples for the trainer; same keys, dtypes and shapes as the
+    reference (sample_processing_utils.py:159-223)."""
+    if len(batched_questions) == 1 and batched_questions[0].get('dummy', False):
+        return make_dummy_batch(batched_questions, device)
+
+    il, ol = _lens(batched_questions)
+    sample_lens = il + ol
+    total = int(sample_lens.sum())
+    cu = torch.from_numpy(np.concatenate(([0], np.cumsum(sample_lens))).astype(np.int32)).to(device)
+    output_indices = ops.output_indices(il, ol, device)
+
+    per_sample = torch.tensor([[float(s["advantage"]) for s in batched_questions], ol.astype(np.float64).tolist()],
+                              dtype=torch.float64).to(device)
+    advantages = ops.segment_broadcast(per_sample[0], cu, total)
+    if constant_length_samples is None:
+        output_lens_broadcasted = ops.segment_broadcast(per_sample[1], cu, total)
+    else:
+        output_lens_broadcasted = torch.full((total,), float(constant_length_samples), device=device, dtype=torch.float32)
+
+    lp_host = [torch.as_tensor(s["sample_logprobs"], dtype=torch.float32).reshape(-1) for s in batched_questions]
+    reference_output_logprobs = torch.cat(lp_host).to(device)
+    ent_host = []
+    for s, lp in zip(batched_questions, lp_host):
+        e = s.get("sample_entropies", None)
+        ent_host.append(torch.zeros(lp.numel()) if e is None else torch.as_tensor(e, dtype=torch.float32).reshape(-1))
+    reference_output_entropies = torch.cat(ent_host).to(device) if ent_host else torch.zeros_like(reference_output_logprobs)
+
+    batch_ids, batch_position_ids, labels = get_input_for_logprobs(batched_questions, output_indices, device)
+
+    modified = [q for q in batched_questions if q['modified_reward'] is not None]
+    plain = [q for q in batched_questions if q['modified_reward'] is None]
+    f32 = lambda x: torch.tensor(float(x), device=device, dtype=torch.float32)
+    out = {
+        "batch_ids": batch_ids.contiguous(),
+        "batch_position_ids": batch_position_ids.contiguous(),
+        "output_indices": output_indices.contiguous(),
+        "advantages": advantages.contiguous(),
+        "reference_output_logprobs": reference_output_logprobs.contiguous(),
+        "reference_output_entropies": reference_output_entropies.contiguous(),
+        "output_lens_broadcasted": output_lens_broadcasted.contiguous(),
+        "num_output_tokens_non_masked": (labels != -100).sum().to(torch.float32),
+        "num_output_tokens": f32(ol.sum()),
+        "num_samples": f32(len(batched_questions)),
+        "max_reward_in_group": f32(0.0),
+        "total_modified_reward": f32(sum(s['modified_reward'] for s in modified)) if modified else f32(0.0),
+        "total_non_modified_reward": f32(sum(s['reward'] for s in plain)) if plain else f32(0.0),
+        "num_modified_samples": f32(len(modified)),
+        "delimiter_not_found": f32(sum(s['delimiter_not_found'] for s in modified)) if modified else f32(0.0),
+        "samples": batched_questions,
+        "labels": labels.contiguous(),
+        "total_reward_rank": f32(sum(s['reward'] for s in batched_questions)),
+        "truncated_sample": f32(sum(s['truncated_sample'] for s in batched_questions)),
+        "advantage_is_zero": f32(0.0),
+        # not in the reference: segment boundaries, so that the loss can aggregate per sample
+        "cu_seqlens": cu,
+    }
+    try:
+        out["uids"] = torch.tensor([int(s.get("__uid__", -1)) for s in batched_questions], device=device)
+    except Exception:
+        pass
+    return out
+
+
+def normalize_rewards(rewards, eps: float = 1e-4, group_size: Optional[int] = None):
+    """Group-normalised advantages on the GPU: (r - mean) / (population std + eps)
+    (reference: vllm_worker.py:77-92 and :788-796).  ``rewards`` is one group, or
+    several groups of ``group_size`` laid end to end; returns float64 numpy."""
+    r = torch.as_tensor(np.asarray(rewards, dtype=np.float64))
+    n = r.numel()
+    gs = n if group_size is None else int(group_size)
+    if gs <= 0 or n % gs:
+        raise ValueError("normalize_rewards: group_size must divide the number of rewards")
+    goff = torch.arange(0, n + 1, gs, dtype=torch.int32)
+    out = ops.group_advantages(r.cuda(), goff.cuda(), eps, torch.float64)
+    return out.cpu().numpy()

@@ -1,0 +1,85 @@
+"""Single-GPU harnesses mirroring the two worker methods that drive the hot path
+in the reference: ``TrainerGPUWorker.compute_gradients``
+(gpu_process_worker.py:963-1050) and
+``LogProbGPUWorker.compute_log_probs_from_samples``
+(gpu_process_worker.py:1662-1709).  Ray, FSDP and the weight sync around them
+are not reproduced; the model is any module patched by
+``grpo_loss.make_grpo_forward``."""
+from __future__ import annotations
+
+from types import SimpleNamespace
+from typing import List
+
+import torch
+
+from grpo_loss import compute_dual_clip_grpo_loss
+from sample_processing_utils import post_process_batch
+
+
+class TrainerHarness:
+    """Forward + backward of one micro-batch with the reference's loss scaling."""
+
+    def __init__(self, model, config=None, device="cuda:0", fsdp_world_size: int = 1):
+        self.actor_module_fsdp = model
+        self.config = config or SimpleNamespace(clip_low=0.2, clip_high=0.28, clip_ratio_c=3.0,
+                                                train_minibatch_sample_size=0, entropy_coeff=0.0)
+        self.device = torch.device(device)
+        self.fsdp_world_size = fsdp_world_size
+        self._mb_count_since_last_step = 0
+
+    def compute_gradients(self, worker_batch: list, total_non_masked_tokens: int = 0) -> dict:
+        self.actor_module_fsdp.train()
+        batch = post_process_batch(worker_batch, self.device)
+        # single GPU: an all-masked batch contributes nothing (gpu_process_worker.py:979-985)
+        if self.fsdp_world_size == 1 and float(batch["num_output_tokens_non_masked"].item()) == 0:
+            return {"loss": 0.0, "pg_clip": 0, "kl_div": 0.0, "entropy": 0.0}
+        cfg = self.config
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            loss, metrics = compute_dual_clip_grpo_loss(
+                self.actor_module_fsdp, batch, cfg.clip_low, cfg.clip_high, cfg.clip_ratio_c,
+                compute_entropy=bool(getattr(cfg, "compute_entropy", True)),
+                apply_entropy_bonus=bool(getattr(cfg, "apply_entropy_bonus", True)),
+                entropy_coeff=float(getattr(cfg, "entropy_coeff", 0.0)))
+        # n_real / (minibatch_target // world) before backward (gpu_process_worker.py:1006-1025)
+        n_real = sum(1 for s in worker_batch if not s.get("dummy", False))
+        target = int(getattr(cfg, "train_minibatch_sample_size", 0) or 0)
+        if self.fsdp_world_size > 0:
+            target = max(1, target // self.fsdp_world_size) if target else 0
+        if target > 0 and n_real != target:
+            loss = loss * (float(n_real) / float(target))
+        loss.backward()
+        self._mb_count_since_last_step += 1
+        return metrics
+
+
+class LogProbHarness:
+    """No-grad per-sample logprobs and entropies of packed samples."""
+
+    def __init__(self, model, device="cuda:0"):
+        self.actor_module_fsdp = model
+        self.device = torch.device(device)
+
+    @torch.no_grad()
+    def compute_log_probs_from_samples(self, samples: list) -> List[dict]:
+        self.actor_module_fsdp.eval()
+        lens = [len(s["sample_ids"]) for s in samples]
+        total = sum(lens)
+        host = torch.empty((3, total), dtype=torch.long)
+        off = 0
+        for s, k in zip(samples, lens):
+            host[0, off:off + k] = torch.as_tensor(s["sample_ids"], dtype=torch.long)
+            host[1, off:off + k] = torch.arange(k)
+            host[2, off:off + k] = torch.as_tensor(s.get("labels", [-100] * k), dtype=torch.long)
+            off += k
+        dev = host.to(self.device)
+        out = self.actor_module_fsdp(input_ids=dev[0:1], attention_mask=None, position_ids=dev[1:2], labels=dev[2:3])
+        # one device->host copy for the whole batch, then split on the host
+        lp = out.loss.detach().float().cpu()
+        ent = getattr(out, "entropy", None)
+        ent = ent.detach().float().cpu() if ent is not None else None
+        res, off = [], 0
+        for k in lens:
+            res.append({"logprobs": lp[off:off + k].tolist(),
+                        "entropies": ent[off:off + k].tolist() if ent is not None else None})
+            off += k
+        return res

@@ -1,0 +1,170 @@
+"""Benchmark of the fused logprob + GRPO forward/backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1]
+
+A step is one pass of the hot path (LM-head projection -> log-softmax -> target
+gather -> dual-clip GRPO objective -> backward to dHidden and dW) over one packed
+micro-batch of synthetic data already resident in HBM.  Prints ONE JSON line:
+packed tokens/s, the MFMA roofline fraction of the dominant kernel (measured with
+HIP events on the launch stream) and the CPU oracle timed on the host cores."""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (os.path.join(ROOT, "async-grpo-nccl_amd"), ROOT):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+
+# HBM bytes per launch of the forward kernel at cfg1 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (scaled by a copy kernel of known size); None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {"cfg1": None}
+
+
+def cpu_baseline(name: str, cfg_chunk, seed: int):
+    """The oracle (a port of the reference's eager path) on the host cores, on a
+    bounded slice: one chunk of tokens at the full H and V, forward + backward,
+    bf16-rounded inputs with fp32 math.  Work is linear in tokens."""
+    import torch
+    from oracle import grpo_oracle as O
+    from fgrpo.synthetic import CONFIGS
+    cfg = CONFIGS[name]
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    H, V = cfg["H"], cfg["V"]
+    g = torch.Generator().manual_seed(seed)
+    W = (torch.randn(V, H, generator=g) * cfg["w_std"]).bfloat16().float()
+
+    def run(n_tok):
+        hs = (torch.randn(1, n_tok, H, generator=g) / H ** 0.5).bfloat16().float().requires_grad_(not cfg["forward_only"])
+        Wl = W.clone().requires_grad_(not cfg["forward_only"])
+        labels = torch.randint(0, V, (1, n_tok), generator=g)
+        adv = torch.randn(n_tok, generator=g)
+        old = torch.full((n_tok,), -12.0)
+        t0 = time.perf_counter()
+        if cfg["forward_only"]:
+            with torch.no_grad():
+                O.fused_log_probs_and_entropy(Wl, None, hs, labels, 1.0)
+        else:
+            out = O.grpo_loss_and_entropy(Wl, None, hs, labels, 1.0, old, adv, cfg["clip_low"], cfg["clip_high"], cfg["clip_ratio_c"])
+            out[0].backward()
+        return time.perf_counter() - t0
+
+    probe = 128
+    t_probe = run(probe)
+    # aim at ~15 s of CPU work, at most the configuration's own chunk size
+    n = int(max(probe, min(cfg_chunk or 4096, probe * 15.0 / max(t_probe, 1e-3))))
+    n = max(probe, (n // 128) * 128)
+    times = [run(n) for _ in range(2)]
+    t = min(times)
+    return {"value": n / t, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{n} tokens (one chunk) at full H={H}, V={V}, fwd{'' if cfg['forward_only'] else '+bwd'}, "
+                      f"fp32 math on bf16-rounded inputs, best of 2; tokens/s is linear in tokens"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="cfg1")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the path shards by micro-batch, one per GPU); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import grpo_loss as G
+    from fgrpo import ops
+    from fgrpo.synthetic import make_workload
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = make_workload(args.config, seed=args.seed, device=dev)
+    p = w.params
+    T, H, V = w.T, w.H, w.V
+    fwd_only = p["forward_only"]
+    labels = w.labels
+    shifted = ops.shift_labels(labels).reshape(-1)
+
+    # inputs of the objective: advantages from the group kernel, old/ref = current logprob + noise
+    adv_s = ops.group_advantages(w.rewards, w.group_offsets, p["adv_eps"])
+    adv = ops.segment_broadcast(adv_s, w.cu_seqlens, T)
+    with torch.no_grad():
+        lp0, _, _ = ops.lmhead_logprob_fwd(w.hidden.reshape(T, H), w.weight, None, shifted)
+    old = lp0 + w.noise_old
+    ref = lp0 + w.noise_ref
+    hidden = w.hidden.clone().requires_grad_(not fwd_only)
+    weight = w.weight.clone().requires_grad_(not fwd_only)
+
+    def step():
+        if fwd_only:
+            with torch.no_grad():
+                return G.fused_log_probs_and_entropy_fn(weight, None, hidden, labels)
+        hidden.grad = None
+        weight.grad = None
+        out = G.grpo_loss_and_entropy_ce_fn(weight, None, hidden, labels, 1.0, old, adv, p["clip_low"], p["clip_high"],
+                                            p["clip_ratio_c"], loss_chunksize=p["chunk"], ref_logprobs=ref,
+                                            kl_beta=p["kl_beta"], loss_agg_mode="sample_mean", cu_seqlens=w.cu_seqlens)
+        out[0].backward()
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+    tok_s = T / (ms / 1e3)
+
+    # dominant kernel: the forward statistics kernel (one launch = all T tokens x all V rows).
+    # HIP events on the stream the kernel is launched on (torch's current stream).
+    hs2 = w.hidden.reshape(T, H)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n_k = max(3, min(args.steps, 10))
+    with torch.no_grad():
+        ops.lmhead_logprob_fwd(hs2, w.weight, None, shifted)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(n_k):
+            ops.lmhead_logprob_fwd(hs2, w.weight, None, shifted)
+        e1.record()
+    torch.cuda.synchronize()
+    k_ms = e0.elapsed_time(e1) / n_k
+    flops_launch = 2.0 * T * H * V
+    achieved = flops_launch / (k_ms * 1e-3) / 1e12
+    alg_flops_step = (2.0 if fwd_only else 6.0) * T * H * V
+
+    line = {
+        "metric": "packed tokens/sec fused logprob+GRPO fwd/bwd (Qwen2.5-1.5B shape); MFMA % peak",
+        "value": tok_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "fp32", "data": "synthetic",
+        "config": {"workload": f"{args.config}: T={T} packed tokens, H={H}, V={V}, "
+                               f"{'forward only' if fwd_only else 'forward+backward (dHidden, dW)'}, "
+                               f"{w.n_samples} samples, chunk hint {p['chunk']}",
+                   "tokens": T, "hidden": H, "vocab": V, "samples": w.n_samples},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
+                     "kernel": "lmhead_fwd_kernel (+ per-token combine)", "kernel_ms": k_ms,
+                     "algorithmic_flops_per_launch": flops_launch},
+        "path_mfma_frac": alg_flops_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        "path_algorithmic_tflops": alg_flops_step / (ms * 1e-3) / 1e12,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.config, p["chunk"], args.seed)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -124,6 +124,21 @@ int fgrpo_segment_broadcast(const void* values, int values_f64, const int32_t* c
 int fgrpo_segment_reduce(const float* x, const int64_t* labels, const int32_t* cu_seqlens, int nseq,
                          float* sum_out, float* mean_out, int32_t* count_out, void* stream);
 
+/* ---- batch shaping --------------------------------------------------------------
+ * fgrpo_output_indices replaces get_output_logits_indices_numba
+ * (sample_processing_utils.py:29-67): sample i, packed at token offset
+ * tok_off[i] with prompt length in_len[i], contributes the positions
+ * tok_off[i]+in_len[i]-1+j, j in [0, out_off[i+1]-out_off[i]), written at
+ * out[out_off[i]+j].  tok_off, in_len [nsamples], out_off [nsamples+1] int32.
+ * fgrpo_segment_starts replaces the cu_seqlens derivation of
+ * gpu_process_worker.py:239-252: cu_out = ordered indices t with
+ * position_ids[t]==0, then T; *count_out = entries produced (boundaries + 1),
+ * at most max_out of them are stored. */
+int fgrpo_output_indices(const int32_t* tok_off, const int32_t* in_len, const int32_t* out_off,
+                         int nsamples, int64_t* out, void* stream);
+int fgrpo_segment_starts(const int64_t* position_ids, int T, int32_t* cu_out, int max_out,
+                         int32_t* count_out, void* stream);
+
 /* ---- row soft-max on materialised logits ----------------------------------------
  * Replaces logprobs_from_logits (grpo_loss.py:146-173) and entropy_from_logits
  * (grpo_loss.py:203-208) for callers that already hold logits [N x V] (ld =

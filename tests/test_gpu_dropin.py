@@ -1,0 +1,227 @@
+"""GPU tests of the drop-in Python surface (grpo_loss.py, sample_processing_utils.py,
+workers.py of this package) against the CPU oracle: the patched model forward in both
+modes, the metrics dictionary, batch packing, the worker harnesses, and the small
+segmented / per-group kernels."""
+import math
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import grpo_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+class TinyBody(torch.nn.Module):
+    """Stand-in for the transformer body: embedding + one linear layer."""
+
+    def __init__(self, V, H):
+        super().__init__()
+        self.embed_tokens = torch.nn.Embedding(V, H)
+        self.proj = torch.nn.Linear(H, H, bias=False)
+
+    def forward(self, input_ids=None, position_ids=None, **kw):
+        h = self.proj(self.embed_tokens(input_ids)) + 0.01 * position_ids.unsqueeze(-1).to(self.proj.weight.dtype)
+        return (h,)
+
+
+class TinyLM(torch.nn.Module):
+    def __init__(self, V=512, H=64, tied=True):
+        super().__init__()
+        self.model = TinyBody(V, H)
+        self.lm_head = torch.nn.Linear(H, V, bias=False)
+        if tied:
+            self.lm_head.weight = self.model.embed_tokens.weight
+        self.config = SimpleNamespace(output_attentions=False, output_hidden_states=False, use_return_dict=True)
+
+    def forward(self, *a, **k):
+        raise RuntimeError("unpatched forward")
+
+
+def make_samples(n=6, V=512, seed=0):
+    rng = np.random.default_rng(seed)
+    samples = []
+    for i in range(n):
+        li, lo = int(rng.integers(2, 9)), int(rng.integers(3, 20))
+        ids = rng.integers(0, V, li + lo).tolist()
+        samples.append(dict(sample_ids=ids, sample_position_ids=list(range(li + lo)), labels=O.make_labels(ids, li, lo),
+                            input_len=li, output_len=lo, advantage=float(rng.normal()),
+                            sample_logprobs=(-rng.random(li + lo) * 0.2 - math.log(V)).tolist(),
+                            sample_entropies=(rng.random(li + lo) + 5).tolist() if i % 2 == 0 else None,
+                            reward=float(i % 2), modified_reward=None, delimiter_not_found=False,
+                            truncated_sample=bool(i % 3 == 0), __uid__=100 + i))
+    return samples
+
+
+def test_post_process_batch_matches_oracle(dev):
+    import sample_processing_utils as spu
+    samples = make_samples()
+    got = spu.post_process_batch(samples, dev)
+    want = O.pack_samples(samples)
+    for k, v in want.items():
+        assert k in got, k
+        g = got[k].cpu()
+        assert g.dtype == v.dtype and g.shape == v.shape, k
+        assert torch.equal(g, v), k
+    assert got["uids"].tolist() == [100 + i for i in range(len(samples))]
+    cu = got["cu_seqlens"].cpu()
+    assert torch.equal(cu, O.cu_seqlens_from_position_ids(want["batch_position_ids"]))
+    const = spu.post_process_batch(samples, dev, constant_length_samples=7)
+    assert (const["output_lens_broadcasted"] == 7).all()
+    dummy = spu.post_process_batch([{"dummy": True}], dev)
+    assert dummy["labels"].eq(-100).all() and dummy["output_indices"].numel() == 0
+
+
+def test_segment_kernels(dev):
+    from fgrpo import ops
+    pos = torch.cat([torch.arange(n) for n in (5, 1, 300, 64, 1000, 2)])[None].to(dev)
+    cu = ops.cu_seqlens_from_position_ids(pos)
+    assert torch.equal(cu.cpu(), O.cu_seqlens_from_position_ids(pos.cpu())) and cu.dtype == torch.int32
+    vals = torch.randn(6, dtype=torch.float64)
+    out = ops.segment_broadcast(vals.to(dev), cu, pos.numel())
+    assert torch.equal(out.cpu(), torch.from_numpy(O.broadcast_values(vals.numpy(), [5, 1, 300, 64, 1000, 2])).float())
+    x = torch.randn(pos.numel())
+    lab = torch.randint(0, 9, (pos.numel(),))
+    lab[::3] = -100
+    s, m, c = ops.segment_reduce(x.to(dev), cu, lab.to(dev))
+    off = 0
+    for i, n in enumerate((5, 1, 300, 64, 1000, 2)):
+        ok = lab[off:off + n] != -100
+        assert c[i].item() == int(ok.sum())
+        assert abs(s[i].item() - x[off:off + n][ok].sum().item()) < 1e-3
+        if ok.any():
+            assert abs(m[i].item() - x[off:off + n][ok].mean().item()) < 1e-4
+        off += n
+    il, ol = [3, 1, 4, 2], [2, 5, 1, 0]
+    assert ops.output_indices(il, ol, dev).cpu().tolist() == O.output_logits_indices(il, ol).tolist()
+
+
+def test_group_advantages(dev):
+    from fgrpo import ops
+    import sample_processing_utils as spu
+    rng = np.random.default_rng(0)
+    r = (rng.random(8 * 13) < 0.3).astype(np.float64)
+    r[8:16] = 1.0                                   # an all-equal group
+    goff = torch.arange(0, 8 * 13 + 1, 8, dtype=torch.int32)
+    want = np.concatenate([O.group_advantages(r[i:i + 8]) for i in range(0, len(r), 8)])
+    got = ops.group_advantages(torch.from_numpy(r).to(dev), goff.to(dev), 1e-4, torch.float64).cpu().numpy()
+    assert np.allclose(got, want, rtol=1e-12, atol=1e-12) and np.all(got[8:16] == 0)
+    got32 = ops.group_advantages(torch.from_numpy(r).float().to(dev), goff.to(dev), 1e-6).cpu().numpy()
+    want6 = np.concatenate([O.group_advantages(r[i:i + 8], 1e-6) for i in range(0, len(r), 8)])
+    assert np.allclose(got32, want6, rtol=1e-5, atol=1e-5)
+    assert np.allclose(spu.normalize_rewards(r[:8]), O.group_advantages(r[:8]), atol=1e-12)
+    ragged = torch.tensor([0, 3, 4, 104], dtype=torch.int32)
+    got_r = ops.group_advantages(torch.from_numpy(r).to(dev), ragged.to(dev), 1e-4, torch.float64).cpu().numpy()
+    want_r = np.concatenate([O.group_advantages(r[a:b]) for a, b in ((0, 3), (3, 4), (4, 104))])
+    assert np.allclose(got_r, want_r, atol=1e-12)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_row_kernels_on_materialised_logits(dev, dtype):
+    import grpo_loss as G
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(2, 37, 1003, generator=g) * 3).to(dtype)
+    y = torch.randint(0, 1003, (2, 37), generator=g)
+    y[0, :4] = -100
+    xg = x.to(dev).requires_grad_(True)
+    lp = G.logprobs_from_logits(xg, y.to(dev))
+    want = O.logprobs_from_logits(x.float(), y)
+    tol = 1e-5 if dtype == torch.float32 else 0.07          # bf16 output rounding of values near -12
+    assert lp.dtype == dtype and lp.shape == y.shape
+    assert (lp.float().cpu() - want).abs().max() <= tol
+    lp32 = G.logprobs_from_logits_flash_attn(xg, y.to(dev))
+    assert lp32.dtype == torch.float32 and (lp32.cpu() - want).abs().max() <= 1e-5
+    ent = G.entropy_from_logits(x.to(dev))
+    assert (ent.float().cpu() - O.entropy_from_logits(x.float())).abs().max() <= (1e-5 if dtype == torch.float32 else 0.04)
+    w = torch.randn(2, 37, generator=g)
+    (lp32 * w.to(dev)).sum().backward()
+    xo = x.float().requires_grad_(True)
+    (O.logprobs_from_logits(xo, y) * w).sum().backward()
+    rel = (xg.grad.float().cpu() - xo.grad).norm() / xo.grad.norm()
+    assert rel <= (1e-5 if dtype == torch.float32 else 5e-3)
+    assert xg.grad[0, :4].abs().max() == 0
+    # ignore_index=None: every label is gathered
+    lpn = G.logprobs_from_logits(x.to(dev), y.clamp(min=0).to(dev), ignore_index=None)
+    assert (lpn.float().cpu() - O.logprobs_from_logits(x.float(), y.clamp(min=0), None)).abs().max() <= tol
+
+
+def _patched(dev, mode, dtype=torch.float32, chunk=None, temperature=1.0):
+    import grpo_loss as G
+    torch.manual_seed(0)
+    m = TinyLM().to(dev).to(dtype)
+    return G.make_grpo_forward(m, temperature=temperature, mode=mode, loss_chunksize=chunk), G
+
+
+def _oracle_hidden(model, batch):
+    with torch.no_grad():
+        return model.model(input_ids=batch["batch_ids"], position_ids=batch["batch_position_ids"])[0].float().cpu()
+
+
+def test_eval_forward_and_logprob_worker(dev):
+    from workers import LogProbHarness
+    model, G = _patched(dev, "eval", temperature=0.9)
+    samples = make_samples(5)
+    res = LogProbHarness(model, dev).compute_log_probs_from_samples(samples)
+    assert len(res) == 5
+    ids = torch.tensor(sum((s["sample_ids"] for s in samples), []))[None]
+    pos = torch.cat([torch.arange(len(s["sample_ids"])) for s in samples])[None]
+    labels = torch.tensor(sum((s["labels"] for s in samples), []))[None]
+    hid = _oracle_hidden(model, dict(batch_ids=ids.to(dev), batch_position_ids=pos.to(dev)))
+    lp, ent = O.fused_log_probs_and_entropy(model.lm_head.weight.detach().float().cpu(), None, hid, labels, 0.9)
+    want = O.split_logprobs_per_sample(lp, ent, [len(s["sample_ids"]) for s in samples])
+    for a, b in zip(res, want):
+        assert np.allclose(a["logprobs"], b["logprobs"], atol=1e-4)
+        assert np.allclose(a["entropies"], b["entropies"], atol=1e-4)
+    with pytest.raises(ValueError):
+        G.make_grpo_forward(TinyLM().to(dev), mode="bogus").forward(input_ids=ids.to(dev), position_ids=pos.to(dev), labels=labels.to(dev))
+
+
+@pytest.mark.parametrize("entropy_coeff", [0.0, 0.01])
+def test_training_forward_metrics_and_backward(dev, entropy_coeff):
+    import sample_processing_utils as spu
+    model, G = _patched(dev, "training", chunk=16)
+    samples = make_samples(7, seed=3)
+    batch = spu.post_process_batch(samples, dev)
+    loss, metrics = G.compute_dual_clip_grpo_loss(model, batch, 0.2, 0.28, 3.0, entropy_coeff=entropy_coeff)
+    loss.backward()
+    # oracle on the same hidden states, gradients through the same tiny body on the CPU
+    import copy
+    cpu_model = copy.deepcopy(model).cpu().float()
+    cb = O.pack_samples(samples)
+    hid = cpu_model.model(input_ids=cb["batch_ids"], position_ids=cb["batch_position_ids"])[0]
+    out = O.grpo_loss_and_entropy(cpu_model.lm_head.weight, None, hid, cb["labels"], 1.0, cb["reference_output_logprobs"],
+                                  cb["advantages"], 0.2, 0.28, 3.0)
+    want = O.dual_clip_metrics(out[0].item(), out[1], out[2], out[4], out[5], cb["advantages"], cb["output_indices"],
+                               cb["labels"], 0.2, 0.28, old_entropy=cb["reference_output_entropies"],
+                               num_samples=len(samples), entropy_coeff=entropy_coeff)
+    assert set(metrics) == set(want)
+    for k, v in want.items():
+        assert abs(metrics[k] - v) <= 2e-4 * max(1.0, abs(v)), (k, metrics[k], v)
+    want_loss = out[0] - entropy_coeff * out[1][cb["output_indices"]].mean()
+    assert abs(loss.item() - want_loss.item()) <= 2e-4 * max(1.0, abs(want_loss.item()))
+    out[0].backward()
+    ge = model.model.embed_tokens.weight.grad.float().cpu()          # tied: LM-head + embedding gradients summed
+    gw = cpu_model.model.embed_tokens.weight.grad
+    assert torch.nn.functional.cosine_similarity(ge.flatten(), gw.flatten(), dim=0) > 0.9999
+    gp = model.model.proj.weight.grad.float().cpu()
+    assert torch.nn.functional.cosine_similarity(gp.flatten(), cpu_model.model.proj.weight.grad.flatten(), dim=0) > 0.9999
+
+
+def test_trainer_harness_scaling_and_dummy(dev):
+    from workers import TrainerHarness
+    model, G = _patched(dev, "training", dtype=torch.bfloat16)
+    cfg = SimpleNamespace(clip_low=0.2, clip_high=0.28, clip_ratio_c=3.0, train_minibatch_sample_size=16, entropy_coeff=0.0)
+    tr = TrainerHarness(model, cfg, dev)
+    samples = make_samples(4, seed=5)
+    m = tr.compute_gradients(samples, 0)
+    g1 = model.model.proj.weight.grad.clone()
+    assert set(("loss", "kl_div", "entropy", "pg_clip", "approx_kl")) <= set(m)
+    model.zero_grad()
+    cfg.train_minibatch_sample_size = 4            # scale 1 instead of 4/16
+    tr.compute_gradients(samples, 0)
+    g2 = model.model.proj.weight.grad.clone()
+    ratio = (g1.float().norm() / g2.float().norm()).item()
+    assert abs(ratio - 0.25) < 0.02
+    assert tr.compute_gradients([{"dummy": True}], 0) == {"loss": 0.0, "pg_clip": 0, "kl_div": 0.0, "entropy": 0.0}

@@ -1,0 +1,79 @@
+"""Host-side logic that needs no GPU: numpy forms of the batch-shaping helpers
+against the oracle, synthetic workload generators, and the refusal of CPU
+tensors by the product path."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import grpo_oracle as O
+
+
+def test_numpy_index_and_broadcast_helpers_match_oracle():
+    import sample_processing_utils as spu
+    rng = np.random.default_rng(1)
+    for n in (0, 1, 7):
+        il = rng.integers(1, 9, n)
+        ol = rng.integers(0, 9, n)
+        assert np.array_equal(spu.get_output_logits_indices_numba(il, ol), O.output_logits_indices(il, ol))
+        vals = rng.normal(size=n)
+        assert np.array_equal(spu.broadcast_values(vals, il + ol), O.broadcast_values(vals, il + ol))
+
+
+def test_product_path_refuses_cpu_tensors():
+    import grpo_loss as G
+    hs = torch.randn(1, 8, 16)
+    W = torch.randn(32, 16)
+    labels = torch.randint(0, 32, (1, 8))
+    with pytest.raises(RuntimeError, match="GPU"):
+        G.fused_log_probs_and_entropy_fn(W, None, hs, labels)
+    with pytest.raises(RuntimeError, match="GPU"):
+        G.grpo_loss_and_entropy_ce_fn(W, None, hs, labels, advantages=torch.zeros(8))
+    with pytest.raises(RuntimeError, match="GPU"):
+        G.logprobs_from_logits(torch.randn(4, 9), torch.zeros(4, dtype=torch.long))
+
+
+def test_foreign_per_token_fn_is_rejected():
+    import grpo_loss as G
+    with pytest.raises(NotImplementedError):
+        G.fused_log_probs_and_entropy_fn(torch.randn(4, 4), None, torch.randn(1, 2, 4), torch.zeros(1, 2, dtype=torch.long),
+                                         per_token_fn=lambda *a, **k: None)
+
+
+def test_reference_surface_is_present():
+    import grpo_loss as G
+    import inspect
+    for name in ("GRPOOutput", "LogProbsOutput", "make_grpo_forward", "logprobs_from_logits",
+                 "logprobs_from_logits_flash_attn", "entropy_from_logits", "fused_log_probs_and_entropy_fn",
+                 "ce_loss_and_entropy_logsoftmax", "grpo_loss_and_entropy_ce_fn",
+                 "grpo_loss_and_entropy_ce_from_logsoftmax", "compute_dual_clip_grpo_loss", "COMPUTE_ENTROPY_FN",
+                 "DEBUG", "debug_print"):
+        assert hasattr(G, name), name
+    sig = inspect.signature(G.grpo_loss_and_entropy_ce_fn)
+    assert list(sig.parameters) == ["lm_head_weights", "lm_head_bias", "hidden_states", "labels", "temperature",
+                                    "old_logprobs", "advantages", "clip_low", "clip_high", "clip_ratio_c",
+                                    "ce_loss_and_entropy_fn", "per_token_fn", "loss_chunksize", "unused_kwargs"]
+    d = {k: v.default for k, v in sig.parameters.items()}
+    assert (d["temperature"], d["clip_low"], d["clip_high"], d["clip_ratio_c"], d["loss_chunksize"]) == (1.0, 0.2, 0.4, 1e32, None)
+    sig = inspect.signature(G.compute_dual_clip_grpo_loss)
+    assert list(sig.parameters) == ["policy_model", "minibatch", "clip_low", "clip_high", "clip_ratio_c",
+                                    "compute_entropy", "apply_entropy_bonus", "entropy_coeff"]
+    sig = inspect.signature(G.make_grpo_forward)
+    assert list(sig.parameters) == ["model", "temperature", "mode", "use_torch_compile", "loss_chunksize"]
+
+
+def test_synthetic_workloads_have_the_stated_shapes():
+    from fgrpo.synthetic import make_workload, CONFIGS
+    w = make_workload("cfg0")
+    assert w.H == 64 and w.V == 1000 and w.n_samples == 16 and 16 * 16 <= w.T <= 16 * 64
+    assert w.hidden.shape == (1, w.T, 64) and w.weight.shape == (1000, 64) and w.dtype == torch.float32
+    assert int(w.cu_seqlens[-1]) == w.T and w.cu_seqlens.dtype == torch.int32
+    assert (w.labels[0, w.cu_seqlens[:-1].long()] == -100).all()
+    assert (w.labels != -100).sum() == w.T - w.n_samples
+    assert torch.equal(O.cu_seqlens_from_position_ids(w.position_ids), w.cu_seqlens)
+    w2 = make_workload("cfg0")
+    assert torch.equal(w.hidden, w2.hidden) and torch.equal(w.labels, w2.labels)
+    # a shrunken cfg1: same generator code path, exact token count
+    w1 = make_workload("cfg1", overrides=dict(H=64, V=512, tokens=4096))
+    assert w1.T == 4096 and w1.dtype == torch.bfloat16 and int(w1.cu_seqlens[-1]) == 4096
+    assert min(w1.sample_lens) >= 2
+    assert set(CONFIGS) == {"cfg0", "cfg1", "cfg2", "cfg3", "cfg4"}
