@@ -46,7 +46,13 @@ typedef TileCfg<256, 128, 64, 2, 2, 1> Cfg1;
 typedef TileCfg<256, 128, 32, 2, 2, 2> Cfg2;
 typedef TileCfg<256, 256, 32, 2, 4, 2> Cfg3;
 typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg4;
-constexpr int kNumCfg = 5;
+// id 5: 256x256x32, 4 wavefronts, direct-to-LDS loads, 5 LDS stages, look-ahead fragment prefetch
+// id 6: 256x256x64, 4 wavefronts, direct-to-LDS loads, 2 LDS stages
+// id 7: 256x128x32, 4 wavefronts of 128x64, direct-to-LDS, 4 stages, two work-groups per CU
+typedef TileCfg<256, 256, 32, 2, 2, 1, 5, true> Cfg5;
+typedef TileCfg<256, 256, 64, 2, 2, 1, 2, true> Cfg6;
+typedef TileCfg<256, 128, 32, 2, 2, 2, 3, true> Cfg7;
+constexpr int kNumCfg = 8;
 
 struct CfgInfo {
   int bm, bn, bk, nt, lds, wgs_per_cu;
@@ -55,16 +61,17 @@ template <class C>
 constexpr CfgInfo info_of(int wgs) {
   return CfgInfo{C::BM, C::BN, C::BK, C::NT, C::LDS_BYTES, wgs};
 }
-const CfgInfo kCfg[kNumCfg] = {info_of<Cfg0>(1), info_of<Cfg1>(1), info_of<Cfg2>(2), info_of<Cfg3>(1), info_of<Cfg4>(2)};
+const CfgInfo kCfg[kNumCfg] = {info_of<Cfg0>(1), info_of<Cfg1>(1), info_of<Cfg2>(2), info_of<Cfg3>(1), info_of<Cfg4>(2),
+                                info_of<Cfg5>(1), info_of<Cfg6>(1), info_of<Cfg7>(2)};
 
 struct Tuning {
-  int fwd_variant = 0;
-  int ds_variant = 0;
-  int gemm_variant = 0;
+  int fwd_variant = 6;
+  int ds_variant = 6;
+  int gemm_variant = 5;
   int fwd_nsplit = 0;   // 0 = heuristic
   int fwd_group_t = 8;
   int ds_group_v = 8;
-  int gemm_group_m = 8;
+  int gemm_group_m = 4;
   int panel_cols = 32768;  // default vocabulary panel width of the backward
   int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
 } g_tune;
@@ -274,6 +281,9 @@ int launch_store(const StoreParams& p, hipStream_t st) {
     case 1: rc = fn<Cfg1>(__VA_ARGS__); break;            \
     case 2: rc = fn<Cfg2>(__VA_ARGS__); break;            \
     case 3: rc = fn<Cfg3>(__VA_ARGS__); break;            \
+    case 5: rc = fn<Cfg5>(__VA_ARGS__); break;            \
+    case 6: rc = fn<Cfg6>(__VA_ARGS__); break;            \
+    case 7: rc = fn<Cfg7>(__VA_ARGS__); break;            \
     default: rc = fn<Cfg4>(__VA_ARGS__); break;           \
   }
 

@@ -23,6 +23,19 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#ifdef FGRPO_EXP_NO_MFMA  // experiment: keep the data movement, drop the arithmetic
+#define FGRPO_MFMA(a, b, c) (c)
+#else
+#define FGRPO_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
+#endif
+
+#define FGRPO_EXP_FRAG_BASE(st) (st)
+#ifdef FGRPO_EXP_NO_LDSREAD  // experiment: MFMA operands never come from LDS
+#define FGRPO_LDFRAG(ptr) (__builtin_bit_cast(bf16x8_t, u32x4_t{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, (uint32_t)threadIdx.x}))
+#else
+#define FGRPO_LDFRAG(ptr) (*(const bf16x8_t*)(ptr))
+#endif
+
 namespace fgrpo {
 
 typedef uint16_t bf16_t;  // storage type of a bfloat16
@@ -43,24 +56,29 @@ struct GemmOperands {
   int M, N;
 };
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int NST_ = 2, bool DMA_ = false>
 struct TileCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, OCC = OCC_;
-  static constexpr int NT = WM * WN * 64;       // threads per work-group
+  static constexpr bool DMA = DMA_;             // global -> LDS directly (no register staging)
+  static constexpr int NW = WM * WN;            // wavefronts per work-group
+  static constexpr int NT = NW * 64;            // threads per work-group
   static constexpr int WTM = BM / WM;           // wavefront tile rows
   static constexpr int WTN = BN / WN;           // wavefront tile cols
   static constexpr int TM = WTM / 32;           // 32x32 blocks per wavefront, rows
   static constexpr int TN = WTN / 32;           // 32x32 blocks per wavefront, cols
   static constexpr int CPR = BK / 8;            // 16-byte chunks per tile row
-  static constexpr int RPP = NT / CPR;          // tile rows covered by one load pass
-  static constexpr int PA = BM / RPP;           // load passes for A
-  static constexpr int PB = BN / RPP;           // load passes for B
-  static constexpr int ROWB = BK * 2 + 16;      // padded LDS row, bytes
+  static constexpr int RPP = NT / CPR;          // tile rows covered by one load pass of the work-group
+  static constexpr int PA = BM / RPP;           // load passes for A (per thread)
+  static constexpr int PB = BN / RPP;           // load passes for B (per thread)
+  static constexpr int RPI = 64 / CPR;          // tile rows covered by one wavefront-wide 16-byte load
+  static constexpr int ROWB = DMA ? BK * 2 : BK * 2 + 16;  // LDS row bytes (register path pads, DMA path swizzles)
   static constexpr int STAGE = (BM + BN) * ROWB;
-  static constexpr int NSTAGE = 2;
+  static constexpr int NSTAGE = NST_;
   static constexpr int LDS_BYTES = STAGE * NSTAGE;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile/wave shape");
   static_assert(BK % 16 == 0 && NT % CPR == 0 && BM % RPP == 0 && BN % RPP == 0, "loader shape");
+  static_assert(!DMA || (CPR == 4 || CPR == 8), "DMA path supports BK = 32 or 64");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
 // Accumulator element (i, j, r) of lane `lane` in wavefront (wm, wn) sits at
@@ -159,7 +177,7 @@ __device__ __forceinline__ void gemm_mainloop(const GemmOperands& g, int row0, i
         for (int i = 0; i < C::TM; ++i)
 #pragma unroll
           for (int j = 0; j < C::TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            acc[i][j] = FGRPO_MFMA(af[i], bf[j], acc[i][j]);
       }
       if (more) {
         const int nxt = C::STAGE - cur;
@@ -171,6 +189,374 @@ __device__ __forceinline__ void gemm_mainloop(const GemmOperands& g, int row0, i
       __syncthreads();
     }
   }
+}
+
+// ---------------------------------------------------------------------------
+// Direct-to-LDS variant.  global_load_lds_dwordx4 writes lane l's 16 bytes at
+// (wave-uniform LDS base) + 16*l, so one wavefront-wide load fills RPI whole
+// tile rows of BK*2 bytes without padding.  Bank conflicts of the fragment
+// reads are avoided by an XOR swizzle of the 16-byte chunk index with a
+// function of the row, applied on the *global* side (each lane fetches the
+// chunk that belongs at its LDS slot).  NSTAGE LDS buffers keep NSTAGE-1 K
+// steps of loads in flight; completion is tracked with explicit vmcnt waits and
+// one s_barrier per K step.
+// ---------------------------------------------------------------------------
+#ifndef FGRPO_DMA_AUX
+#define FGRPO_DMA_AUX 0   // cache-policy bits of the direct-to-LDS loads
+#endif
+#define FGRPO_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define FGRPO_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// s_waitcnt that waits only for the vector-memory counter to drop to n (n < 64).
+#define FGRPO_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
+// same, and also wait for every outstanding LDS read (lgkmcnt = 0)
+#define FGRPO_WAIT_VMCNT_LGKM0(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (0 << 8) | (((n) >> 4) << 14))
+
+template <class C>
+__device__ __forceinline__ int lds_swizzle(int row) {
+  // Both choices were measured at the full 128 B/clk of the LDS for the MFMA
+  // fragment read pattern (lane l: row l%32, chunk l/32 + 2*kk).
+  if constexpr (C::CPR == 4)
+    return (row >> 1) & 3;                        // 64-byte rows
+  else
+    return row & 7;                               // 128-byte rows
+}
+
+__device__ __forceinline__ void wg_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <class C>
+__device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row0, int col0, char* smem,
+                                                  f32x16_t (&acc)[C::TM][C::TN]) {
+  constexpr int D = C::NSTAGE - 1;              // K steps of loads in flight
+  constexpr int LPT = C::PA + C::PB;            // loads per thread per K step
+  static_assert(D >= 1 && D <= 4 && LPT * (D - 1) < 64, "pipeline depth");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+
+  // loader: instruction i of this wavefront covers tile rows (i*NW + wave)*RPI ..
+  const int lrow = lane / C::CPR, lpc = lane % C::CPR;
+  uint32_t aoff[C::PA], boff[C::PB];
+  const int amax = g.M - 1 - row0, bmax = g.N - 1 - col0;
+#pragma unroll
+  for (int i = 0; i < C::PA; ++i) {
+    const int rt = (i * C::NW + wave) * C::RPI + lrow;            // row inside the tile (decides the swizzle)
+    const int r = rt < amax ? rt : amax;                          // row actually read
+    aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+  }
+#pragma unroll
+  for (int i = 0; i < C::PB; ++i) {
+    const int rt = (i * C::NW + wave) * C::RPI + lrow;
+    const int r = rt < bmax ? rt : bmax;
+    boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+  }
+  const int dst_a = wave * C::RPI * C::ROWB;                      // + i * NW*RPI*ROWB, wave-uniform
+  const int dst_b = C::BM * C::ROWB + dst_a;
+  // fragment reads
+  const int sw = lds_swizzle<C>(lane & 31);
+  const int fr_a = (wm * C::WTM + (lane & 31)) * C::ROWB;
+  const int fr_b = C::BM * C::ROWB + (wn * C::WTN + (lane & 31)) * C::ROWB;
+  int fr_c[C::BK / 16];
+#pragma unroll
+  for (int kk = 0; kk < C::BK / 16; ++kk) fr_c[kk] = ((kk * 2 + (lane >> 5)) ^ sw) * 16;
+
+  int nk_total = 0;
+  for (int s = 0; s < g.nseg; ++s) nk_total += g.seg[s].K / C::BK;
+
+  // issue cursor over (segment, k)
+  int iseg = 0, ileft = g.seg[0].K / C::BK;
+  const char* Ai = (const char*)(g.seg[0].A + (long long)row0 * g.lda);
+  const char* Bi = (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
+  auto issue = [&](int stage) {
+#ifdef FGRPO_EXP_NO_GLOBAL  // experiment: no global traffic at all
+    return;
+#endif
+    char* base = smem + stage * C::STAGE;
+#pragma unroll
+    for (int i = 0; i < C::PA; ++i)
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Ai + aoff[i]),
+                                       FGRPO_LDS_PTR(base + dst_a + i * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
+#pragma unroll
+    for (int i = 0; i < C::PB; ++i)
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[i]),
+                                       FGRPO_LDS_PTR(base + dst_b + i * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
+    Ai += C::BK * 2;
+    Bi += C::BK * 2;
+    if (--ileft == 0 && iseg + 1 < g.nseg) {
+      ++iseg;
+      ileft = g.seg[iseg].K / C::BK;
+      Ai = (const char*)(g.seg[iseg].A + (long long)row0 * g.lda);
+      Bi = (const char*)(g.seg[iseg].B + (long long)col0 * g.ldb);
+    }
+  };
+
+  // One load of the current issue step (idx < PA: operand A, else B); the last one advances the cursor.
+  auto issue_one = [&](int stage, int idx) {
+#ifdef FGRPO_EXP_NO_GLOBAL
+    return;
+#endif
+    char* base = smem + stage * C::STAGE;
+    if (idx < C::PA)
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Ai + aoff[idx]),
+                                       FGRPO_LDS_PTR(base + dst_a + idx * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
+    else
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[idx - C::PA]),
+                                       FGRPO_LDS_PTR(base + dst_b + (idx - C::PA) * C::NW * C::RPI * C::ROWB), 16, 0,
+                                       FGRPO_DMA_AUX);
+    if (idx == LPT - 1) {
+      Ai += C::BK * 2;
+      Bi += C::BK * 2;
+      if (--ileft == 0 && iseg + 1 < g.nseg) {
+        ++iseg;
+        ileft = g.seg[iseg].K / C::BK;
+        Ai = (const char*)(g.seg[iseg].A + (long long)row0 * g.lda);
+        Bi = (const char*)(g.seg[iseg].B + (long long)col0 * g.ldb);
+      }
+    }
+  };
+
+  // loads issued before this call (by the caller's epilogue) must not be mistaken for ours
+  FGRPO_WAIT_VMCNT(0);
+  int issued = 0;
+  for (; issued < D && issued < nk_total; ++issued) issue(issued);
+
+  // With three or more LDS buffers the loads of a step are spread over the MFMAs of the step (one
+  // load after every TN MFMAs), so no wavefront ever sits on a full vector-memory queue; with two
+  // buffers they must go out right after the barrier to have a whole step to land.
+  constexpr bool kSpread = (C::NSTAGE >= 3) && (LPT <= (C::BK / 16) * C::TM);
+  constexpr int KK = C::BK / 16;
+
+  int cur = 0, nxt = D % C::NSTAGE;
+  for (int kt = 0; kt < nk_total; ++kt) {
+    const int rem = nk_total - 1 - kt;          // K steps after this one
+    // wait until this step's loads have landed: at most min(rem, D-1) younger steps may stay in flight
+    if (rem >= D - 1) {
+      FGRPO_WAIT_VMCNT(LPT * (D - 1));
+    } else if (D >= 3 && rem == 2) {
+      FGRPO_WAIT_VMCNT(LPT * 2);
+    } else if (D >= 2 && rem == 1) {
+      FGRPO_WAIT_VMCNT(LPT * 1);
+    } else {
+      FGRPO_WAIT_VMCNT(0);
+    }
+    wg_barrier();   // everyone's part of step kt is in LDS; everyone is done reading step kt-1
+    const bool more = issued < nk_total;
+    if (more) ++issued;
+    if (!kSpread && more) issue(nxt);
+    const char* st = smem + cur * C::STAGE;
+    bf16x8_t af[2][C::TM], bf[2][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) af[0][i] = FGRPO_LDFRAG(st + fr_a + i * 32 * C::ROWB + fr_c[0]);
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) bf[0][j] = FGRPO_LDFRAG(st + fr_b + j * 32 * C::ROWB + fr_c[0]);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) {   // next sub-step's fragments fly while this one multiplies
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+          af[(kk + 1) & 1][i] = FGRPO_LDFRAG(st + fr_a + i * 32 * C::ROWB + fr_c[kk + 1]);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+          bf[(kk + 1) & 1][j] = FGRPO_LDFRAG(st + fr_b + j * 32 * C::ROWB + fr_c[kk + 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
+        if (kSpread && kk * C::TM + i < LPT) {
+          if (more) issue_one(nxt, kk * C::TM + i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    cur = (cur + 1 == C::NSTAGE) ? 0 : cur + 1;
+    nxt = (nxt + 1 == C::NSTAGE) ? 0 : nxt + 1;
+  }
+  wg_barrier();   // LDS may be reused by the caller
+}
+
+// ---------------------------------------------------------------------------
+// Direct-to-LDS main loop with one K step of look-ahead (NSTAGE >= 4).
+// The barrier that opens step kt also guarantees that step kt+1 is complete in
+// LDS, so the first fragments of step kt+1 are read *before* the next barrier,
+// while the last MFMAs of step kt run: no LDS latency is exposed after a
+// barrier.  Per step: fragments double-buffered in registers, the loads of step
+// kt+NSTAGE-1 spread one per TN MFMAs, one vmcnt wait + one s_barrier.
+// ---------------------------------------------------------------------------
+template <class C>
+__device__ __forceinline__ void gemm_mainloop_la(const GemmOperands& g, int row0, int col0, char* smem,
+                                                 f32x16_t (&acc)[C::TM][C::TN]) {
+  constexpr int NST = C::NSTAGE;
+  constexpr int LPT = C::PA + C::PB;            // loads per thread per K step
+  constexpr int KK = C::BK / 16;
+  static_assert(NST >= 4 && NST <= 6, "look-ahead pipeline needs 4..6 LDS buffers");
+  static_assert(LPT <= KK * C::TM, "one load slot per TN MFMAs");
+  static_assert(LPT * (NST - 3) < 64, "vmcnt range");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+
+  const int lrow = lane / C::CPR, lpc = lane % C::CPR;
+  uint32_t aoff[C::PA], boff[C::PB];
+  const int amax = g.M - 1 - row0, bmax = g.N - 1 - col0;
+#pragma unroll
+  for (int i = 0; i < C::PA; ++i) {
+    const int rt = (i * C::NW + wave) * C::RPI + lrow;
+    const int r = rt < amax ? rt : amax;
+    aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+  }
+#pragma unroll
+  for (int i = 0; i < C::PB; ++i) {
+    const int rt = (i * C::NW + wave) * C::RPI + lrow;
+    const int r = rt < bmax ? rt : bmax;
+    boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+  }
+  const int dst_a = wave * C::RPI * C::ROWB;
+  const int dst_b = C::BM * C::ROWB + dst_a;
+  const int sw = lds_swizzle<C>(lane & 31);
+  const int fr_a = (wm * C::WTM + (lane & 31)) * C::ROWB;
+  const int fr_b = C::BM * C::ROWB + (wn * C::WTN + (lane & 31)) * C::ROWB;
+  int fr_c[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) fr_c[kk] = ((kk * 2 + (lane >> 5)) ^ sw) * 16;
+
+  // segment table in registers (no scalar memory traffic inside the loop)
+  const char* segA[3];
+  const char* segB[3];
+  int segN[3];
+  int nk_total = 0;
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    const bool on = s < g.nseg;
+    segA[s] = on ? (const char*)(g.seg[s].A + (long long)row0 * g.lda) : nullptr;
+    segB[s] = on ? (const char*)(g.seg[s].B + (long long)col0 * g.ldb) : nullptr;
+    segN[s] = on ? g.seg[s].K / C::BK : 0;
+    nk_total += segN[s];
+  }
+  int iseg = 0, ileft = segN[0];
+  const char* Ai = segA[0];
+  const char* Bi = segB[0];
+  auto issue_one = [&](int stage, int idx) {
+#ifndef FGRPO_EXP_NO_GLOBAL
+    char* base = smem + stage * C::STAGE;
+    if (idx < C::PA)
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Ai + aoff[idx]),
+                                       FGRPO_LDS_PTR(base + dst_a + idx * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
+    else
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[idx - C::PA]),
+                                       FGRPO_LDS_PTR(base + dst_b + (idx - C::PA) * C::NW * C::RPI * C::ROWB), 16, 0,
+                                       FGRPO_DMA_AUX);
+#endif
+    if (idx == LPT - 1) {
+      Ai += C::BK * 2;
+      Bi += C::BK * 2;
+      if (--ileft == 0) {
+        ++iseg;
+        const bool s1 = (iseg == 1);
+        ileft = s1 ? segN[1] : segN[2];
+        Ai = s1 ? segA[1] : segA[2];
+        Bi = s1 ? segB[1] : segB[2];
+      }
+    }
+  };
+  // At most `tiles` K steps of this thread's loads stay in flight.  The look-ahead fragment reads
+  // issued half a step earlier are certainly back by now; saying so (lgkmcnt 0) lets the compiler
+  // start the next step's MFMAs without waiting for the reads it issues at the top of that step.
+  auto wait_allow = [&](int tiles) {
+    if (tiles >= NST - 3) {
+      FGRPO_WAIT_VMCNT_LGKM0(LPT * (NST - 3));
+    } else if (NST >= 6 && tiles == 2) {
+      FGRPO_WAIT_VMCNT_LGKM0(LPT * 2);
+    } else if (NST >= 5 && tiles == 1) {
+      FGRPO_WAIT_VMCNT_LGKM0(LPT * 1);
+    } else {
+      FGRPO_WAIT_VMCNT_LGKM0(0);
+    }
+  };
+
+  FGRPO_WAIT_VMCNT(0);   // the caller's own loads must not be mistaken for ours
+  int issued = 0;
+  for (; issued < NST - 1 && issued < nk_total; ++issued) {
+#pragma unroll
+    for (int idx = 0; idx < LPT; ++idx) issue_one(issued, idx);
+  }
+  // steps 0 and 1 must be in LDS before the first barrier
+  {
+    int allow = issued - 2;
+    wait_allow(allow < 0 ? 0 : allow);
+  }
+  wg_barrier();
+
+  bf16x8_t af[2][C::TM], bf[2][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) af[0][i] = FGRPO_LDFRAG(smem + fr_a + i * 32 * C::ROWB + fr_c[0]);
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) bf[0][j] = FGRPO_LDFRAG(smem + fr_b + j * 32 * C::ROWB + fr_c[0]);
+  __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): enter the loop with these fragments in registers
+
+  int cur = 0;                 // stage of step kt
+  int nst = (NST - 1) % NST;   // stage that the loads issued during step kt go to (= stage of step kt-1)
+  for (int kt = 0; kt < nk_total; ++kt) {
+    const bool more = issued < nk_total;       // a step to issue during this one
+    const bool has_next = kt + 1 < nk_total;
+    const char* st = smem + cur * C::STAGE;
+    const int nx = (cur + 1 == NST) ? 0 : cur + 1;
+    const char* sn = smem + nx * C::STAGE;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int b = kk & 1;
+      // fragments of the next sub-step (or of the next K step's first sub-step) fly under these MFMAs
+      if (kk + 1 < KK) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) af[b ^ 1][i] = FGRPO_LDFRAG(st + fr_a + i * 32 * C::ROWB + fr_c[kk + 1]);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) bf[b ^ 1][j] = FGRPO_LDFRAG(st + fr_b + j * 32 * C::ROWB + fr_c[kk + 1]);
+      } else if (has_next) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) af[b ^ 1][i] = FGRPO_LDFRAG(sn + fr_a + i * 32 * C::ROWB + fr_c[0]);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) bf[b ^ 1][j] = FGRPO_LDFRAG(sn + fr_b + j * 32 * C::ROWB + fr_c[0]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) acc[i][j] = FGRPO_MFMA(af[b][i], bf[b][j], acc[i][j]);
+        if (kk * C::TM + i < LPT) {
+          if (more) issue_one(nst, kk * C::TM + i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    static_assert(KK % 2 == 0, "fragment buffer parity must return to 0 every K step");
+    if (more) ++issued;
+    // before the next step starts, step kt+2 must be complete (step kt+1 already is)
+    {
+      int allow = issued - (kt + 3);
+      wait_allow(allow < 0 ? 0 : allow);
+    }
+    wg_barrier();
+    cur = nx;
+    nst = (nst + 1 == NST) ? 0 : nst + 1;
+  }
+}
+
+template <class C>
+__device__ __forceinline__ void run_mainloop(const GemmOperands& g, int row0, int col0, char* smem,
+                                             f32x16_t (&acc)[C::TM][C::TN]) {
+  if constexpr (C::DMA && C::NSTAGE >= 4)
+    gemm_mainloop_la<C>(g, row0, col0, smem, acc);
+  else if constexpr (C::DMA)
+    gemm_mainloop_dma<C>(g, row0, col0, smem, acc);
+  else
+    gemm_mainloop<C>(g, row0, col0, smem, acc);
 }
 
 // Work-groups are handed to the 8 XCDs round-robin (block b runs on XCD b % 8)

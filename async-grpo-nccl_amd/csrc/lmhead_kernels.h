@@ -81,7 +81,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
     const int row0 = vt * C::BM;
     f32x16_t acc[C::TM][C::TN];
     zero_acc<C>(acc);
-    gemm_mainloop<C>(p.g, row0, col0, smem, acc);
+    run_mainloop<C>(p.g, row0, col0, smem, acc);
 
     const bool edge = row0 + C::BM > V;
     if (p.bias != nullptr || edge) {
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
 
   f32x16_t acc[C::TM][C::TN];
   zero_acc<C>(acc);
-  gemm_mainloop<C>(p.g, row0, col0, smem, acc);
+  run_mainloop<C>(p.g, row0, col0, smem, acc);
 
   if (p.bias != nullptr) {
 #pragma unroll
@@ -387,7 +387,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
 
   f32x16_t acc[C::TM][C::TN];
   zero_acc<C>(acc);
-  gemm_mainloop<C>(p.g, row0, col0, smem, acc);
+  run_mainloop<C>(p.g, row0, col0, smem, acc);
 
   const float alpha = p.alpha * (p.alpha_dev ? *p.alpha_dev : 1.f);
   const int mode = (p.c_in ? 1 : 0) | (p.c_out_bf16 ? 2 : 0);

@@ -7,7 +7,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(HERE), "csrc")
-LIB_PATH = os.path.join(CSRC, "libfgrpo.so")
+LIB_PATH = os.environ.get("FGRPO_LIB", os.path.join(CSRC, "libfgrpo.so"))
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-shared", "-fPIC",
