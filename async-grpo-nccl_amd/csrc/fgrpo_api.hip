@@ -52,7 +52,10 @@ typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg4;
 typedef TileCfg<256, 256, 32, 2, 2, 1, 5, true> Cfg5;
 typedef TileCfg<256, 256, 64, 2, 2, 1, 2, true> Cfg6;
 typedef TileCfg<256, 128, 32, 2, 2, 2, 3, true> Cfg7;
-constexpr int kNumCfg = 8;
+// id 8/9: as 6/5 with 8 wavefronts of 128x64 (two per SIMD)
+typedef TileCfg<256, 256, 64, 2, 4, 2, 2, true> Cfg8;
+typedef TileCfg<256, 256, 32, 2, 4, 2, 5, true> Cfg9;
+constexpr int kNumCfg = 10;
 
 struct CfgInfo {
   int bm, bn, bk, nt, lds, wgs_per_cu;
@@ -62,12 +65,12 @@ constexpr CfgInfo info_of(int wgs) {
   return CfgInfo{C::BM, C::BN, C::BK, C::NT, C::LDS_BYTES, wgs};
 }
 const CfgInfo kCfg[kNumCfg] = {info_of<Cfg0>(1), info_of<Cfg1>(1), info_of<Cfg2>(2), info_of<Cfg3>(1), info_of<Cfg4>(2),
-                                info_of<Cfg5>(1), info_of<Cfg6>(1), info_of<Cfg7>(2)};
+                                info_of<Cfg5>(1), info_of<Cfg6>(1), info_of<Cfg7>(2), info_of<Cfg8>(1), info_of<Cfg9>(1)};
 
 struct Tuning {
-  int fwd_variant = 6;
-  int ds_variant = 6;
-  int gemm_variant = 5;
+  int fwd_variant = 9;
+  int ds_variant = 8;
+  int gemm_variant = 8;
   int fwd_nsplit = 0;   // 0 = heuristic
   int fwd_group_t = 8;
   int ds_group_v = 8;
@@ -284,6 +287,8 @@ int launch_store(const StoreParams& p, hipStream_t st) {
     case 5: rc = fn<Cfg5>(__VA_ARGS__); break;            \
     case 6: rc = fn<Cfg6>(__VA_ARGS__); break;            \
     case 7: rc = fn<Cfg7>(__VA_ARGS__); break;            \
+    case 8: rc = fn<Cfg8>(__VA_ARGS__); break;            \
+    case 9: rc = fn<Cfg9>(__VA_ARGS__); break;            \
     default: rc = fn<Cfg4>(__VA_ARGS__); break;           \
   }
 

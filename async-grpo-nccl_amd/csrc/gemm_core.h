@@ -214,12 +214,15 @@ __device__ __forceinline__ void gemm_mainloop(const GemmOperands& g, int row0, i
 
 template <class C>
 __device__ __forceinline__ int lds_swizzle(int row) {
-  // Both choices were measured at the full 128 B/clk of the LDS for the MFMA
-  // fragment read pattern (lane l: row l%32, chunk l/32 + 2*kk).
+  // Chosen with SQ_LDS_BANK_CONFLICT on the real kernels (fragment read: lane l -> row l%32,
+  // chunk l/32 + 2*kk; the LDS serves 16 consecutive lanes per pass over 64 banks).
+#ifndef FGRPO_SWZ4
+#define FGRPO_SWZ4(row) (((row) >> 2) & 3)
+#endif
   if constexpr (C::CPR == 4)
-    return (row >> 1) & 3;                        // 64-byte rows
+    return FGRPO_SWZ4(row);                       // 64-byte rows
   else
-    return row & 7;                               // 128-byte rows
+    return (row + ((row >> 3) & 1)) & 7;          // 128-byte rows
 }
 
 __device__ __forceinline__ void wg_barrier() {
@@ -325,10 +328,17 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   int issued = 0;
   for (; issued < D && issued < nk_total; ++issued) issue(issued);
 
-  // With three or more LDS buffers the loads of a step are spread over the MFMAs of the step (one
-  // load after every TN MFMAs), so no wavefront ever sits on a full vector-memory queue; with two
-  // buffers they must go out right after the barrier to have a whole step to land.
-  constexpr bool kSpread = (C::NSTAGE >= 3) && (LPT <= (C::BK / 16) * C::TM);
+  // The loads of a step are interleaved with its MFMAs (a burst right after the barrier would keep
+  // every wavefront busy issuing addresses, about 40 cycles per load, before its first MFMA).
+  // With three or more LDS buffers they are spread over the whole step; with two buffers over the
+  // first half, so that the last one still has half a step to land.
+#ifndef FGRPO_SPREAD_DIV2
+#define FGRPO_SPREAD_DIV2 2
+#endif
+  constexpr int kGroups = (C::BK / 16) * C::TM;                                  // MFMA groups (TN MFMAs each) per step
+  constexpr int kSpreadG = (C::NSTAGE >= 3) ? kGroups : (kGroups / FGRPO_SPREAD_DIV2 > 0 ? kGroups / FGRPO_SPREAD_DIV2 : 1);
+  constexpr int kPer = (LPT + kSpreadG - 1) / kSpreadG;                          // loads after each group
+  constexpr bool kSpread = true;
   constexpr int KK = C::BK / 16;
 
   int cur = 0, nxt = D % C::NSTAGE;
@@ -369,8 +379,10 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
       for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
-        if (kSpread && kk * C::TM + i < LPT) {
-          if (more) issue_one(nxt, kk * C::TM + i);
+        if (kSpread && more) {
+#pragma unroll
+          for (int q = 0; q < kPer; ++q)
+            if ((kk * C::TM + i) * kPer + q < LPT) issue_one(nxt, (kk * C::TM + i) * kPer + q);
         }
         __builtin_amdgcn_sched_barrier(0);
       }

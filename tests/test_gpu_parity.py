@@ -132,7 +132,7 @@ def test_ragged_shapes(dev, T, H, V, dtype):
     check(want, got, o, g, f32=(dtype == "fp32"))
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
 def test_every_tile_variant(dev, variant):
     from fgrpo import _lib
     from fgrpo.synthetic import make_workload
@@ -141,7 +141,7 @@ def test_every_tile_variant(dev, variant):
     try:
         want, got, o, g, _, _ = run_case(w, dev, "north_star")
     finally:
-        _lib.set_tuning(fwd_variant=6, ds_variant=6, gemm_variant=5, small_variant=4)
+        _lib.set_tuning(fwd_variant=9, ds_variant=8, gemm_variant=8, small_variant=4)
     check(want, got, o, g, f32=False)
 
 
