@@ -77,6 +77,7 @@ struct Tuning {
   int gemm_group_m = 4;
   int panel_cols = 32768;  // default vocabulary panel width of the backward
   int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
+  int bwd_kmajor = 1;      // 1: the dW GEMM reads dLogits and hidden in place; 2: the dH GEMM reads W in place too
 } g_tune;
 
 int* tuning_slot(const char* key) {
@@ -90,6 +91,7 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "gemm_group_m")) return &g_tune.gemm_group_m;
   if (!strcmp(key, "panel_cols")) return &g_tune.panel_cols;
   if (!strcmp(key, "small_variant")) return &g_tune.small_variant;
+  if (!strcmp(key, "bwd_kmajor")) return &g_tune.bwd_kmajor;
   return nullptr;
 }
 
@@ -292,6 +294,30 @@ int launch_store(const StoreParams& p, hipStream_t st) {
     default: rc = fn<Cfg4>(__VA_ARGS__); break;           \
   }
 
+// Gradient GEMMs whose contraction index is the row index of an operand as it lies in memory.
+// akm/bkm: that operand is [K][M] (resp. [K][N]) with leading dimension lda (ldb); the other is [M][K] ([N][K]).
+int run_store_gemm_kmajor(StoreParams p, bool akm, bool bkm, hipStream_t st) {
+  const GemmOperands& g = p.g;
+  if (g.nseg != 1 || !g.seg[0].A || !g.seg[0].B) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): one segment expected");
+  if (g.M <= 0 || g.N <= 0 || g.seg[0].K <= 0 || g.seg[0].K % Cfg8::BK)
+    return fail(FGRPO_ERR_UNSUPPORTED, "gemm(k-major): M=%d N=%d K=%d", g.M, g.N, g.seg[0].K);
+  if (g.lda % 8 || g.ldb % 8 || !aligned16(g.seg[0].A) || !aligned16(g.seg[0].B))
+    return fail(FGRPO_ERR_ALIGN, "gemm(k-major): operands must be 16-byte aligned with ld %% 8 == 0");
+  p.tiles_m = (g.M + Cfg8::BM - 1) / Cfg8::BM;
+  p.tiles_n = (g.N + Cfg8::BN - 1) / Cfg8::BN;
+  // a K-major tile is read 256 columns wide without clamping: the rows must hold them
+  if (akm && (long long)p.tiles_m * Cfg8::BM > g.lda) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): lda < padded M");
+  if (bkm && (long long)p.tiles_n * Cfg8::BN > g.ldb) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): ldb < padded N");
+  if (256LL * g.lda * 2 >= (1LL << 32) || 256LL * g.ldb * 2 >= (1LL << 32))
+    return fail(FGRPO_ERR_UNSUPPORTED, "gemm(k-major): leading dimension too large");
+  p.group_m = g_tune.gemm_group_m > 0 ? g_tune.gemm_group_m : 1;
+  const int nb = p.tiles_m * p.tiles_n;
+  if (akm && bkm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, true, true>, p, nb, st);
+  if (akm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, true, false>, p, nb, st);
+  if (bkm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, false, true>, p, nb, st);
+  return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): no k-major operand");
+}
+
 int run_store_gemm(StoreParams p, int variant, hipStream_t st) {
   variant = pick_variant(variant, p.g.M, p.g.N);
   const CfgInfo& c = kCfg[variant];
@@ -312,6 +338,8 @@ struct BwdPlan {
   int panel, npanels;     // vocabulary rows per panel (multiple of 256)
   int tiles_t;
   bool copy_ops, f32;
+  bool kmajor;            // dW GEMM reads dLogits [token][vocab] and hidden in place: no [vocab][token] copy
+  bool kmajor_dh;         // dH GEMM reads W in place: no transposed weight copy
   bf16_t *w_hi, *w_lo, *h_hi, *h_lo;          // straight operands (staged only when copy_ops)
   bf16_t *wT_hi, *wT_lo, *hT_hi, *hT_lo;      // transposed copies [H x Vpad], [H x Tpad]
   bf16_t *tv_hi, *tv_lo, *vt_hi, *vt_lo;      // dS panels
@@ -348,18 +376,27 @@ void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long h
       pl.h_lo = cv.take<bf16_t>((size_t)T * pl.Hp);
     }
   }
+  // In-place (K-major) gradient GEMMs: bf16 operands used as they are, H a multiple of the tile width, and
+  // enough tiles to fill the device (small problems keep the small-tile path).
+  {
+    const long long th = (long long)((T + 255) / 256) * (H / 256);
+    const long long vh = (long long)(((V < pl.panel ? V : pl.panel) + 255) / 256) * (H / 256);
+    pl.kmajor = g_tune.bwd_kmajor && !pl.copy_ops && H % 256 == 0 && pl.bm % 64 == 0 && pl.bn % 64 == 0 &&
+                th >= num_cus() / 2 && vh >= num_cus() / 2;
+    pl.kmajor_dh = pl.kmajor && g_tune.bwd_kmajor >= 2;
+  }
   pl.wT_hi = pl.wT_lo = pl.hT_hi = pl.hT_lo = nullptr;
-  if (want_dh) {
+  if (want_dh && !pl.kmajor_dh) {
     pl.wT_hi = cv.take<bf16_t>((size_t)H * pl.Vpad);
     if (pl.f32) pl.wT_lo = cv.take<bf16_t>((size_t)H * pl.Vpad);
   }
-  if (want_dw) {
+  if (want_dw && !pl.kmajor) {
     pl.hT_hi = cv.take<bf16_t>((size_t)H * pl.Tpad);
     if (pl.f32) pl.hT_lo = cv.take<bf16_t>((size_t)H * pl.Tpad);
   }
   const size_t pe = (size_t)pl.Tpad * pl.panel;
   pl.tv_hi = cv.take<bf16_t>(pe);
-  pl.vt_hi = cv.take<bf16_t>(pe);
+  pl.vt_hi = pl.kmajor ? nullptr : cv.take<bf16_t>(pe);
   pl.tv_lo = pl.vt_lo = nullptr;
   if (pl.f32) {
     pl.tv_lo = cv.take<bf16_t>(pe);
@@ -478,11 +515,11 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
     HIP_TRY(hipGetLastError());
   }
   // contraction-major copies for the two gradient GEMMs
-  if (want_dh) {
+  if (want_dh && !pl.kmajor_dh) {
     rc = launch_convert(weight, f32, H, V, H, pl.Vpad, H, pl.wT_hi, pl.wT_lo, pl.Vpad, 1, st);
     if (rc) return rc;
   }
-  if (want_dw) {
+  if (want_dw && !pl.kmajor) {
     rc = launch_convert(hidden, f32, H, T, H, pl.Tpad, H, pl.hT_hi, pl.hT_lo, pl.Tpad, 1, st);
     if (rc) return rc;
   }
@@ -522,7 +559,12 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
       s.g.N = H;
       s.g.lda = pl.panel;
       s.g.ldb = pl.Vpad;
-      if (f32) {
+      if (pl.kmajor_dh) {  // B = W[v0 + k][h] read in place; vocabulary rows past V do not exist
+        s.g.nseg = 1;
+        s.g.seg[0] = GemmSeg{pl.tv_hi, (const bf16_t*)weight + (size_t)v0 * H, kv};
+        s.g.ldb = H;
+        s.g.kb_valid = rows;
+      } else if (f32) {
         s.g.nseg = 3;
         s.g.seg[0] = GemmSeg{pl.tv_hi, pl.wT_hi + v0, kv};
         s.g.seg[1] = GemmSeg{pl.tv_hi, pl.wT_lo + v0, kv};
@@ -546,7 +588,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
         else
           s.c_out_f32 = pl.dh_acc;
       }
-      rc = run_store_gemm(s, g_tune.gemm_variant, st);
+      rc = pl.kmajor_dh ? run_store_gemm_kmajor(s, false, true, st) : run_store_gemm(s, g_tune.gemm_variant, st);
       if (rc) return rc;
     }
     if (want_dw) {  // dW[v0 : v0+rows, H] = dS_vt[rows x kt] * hidden^T[H x kt]^T
@@ -556,7 +598,13 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
       s.g.N = H;
       s.g.lda = pl.Tpad;
       s.g.ldb = pl.Tpad;
-      if (f32) {
+      if (pl.kmajor) {  // A = dS[t][v] and B = hidden[t][h], both read in place with t as the contraction index
+        s.g.nseg = 1;
+        s.g.seg[0] = GemmSeg{pl.tv_hi, (const bf16_t*)hidden, kt};
+        s.g.lda = pl.panel;
+        s.g.ldb = H;
+        s.g.kb_valid = T;
+      } else if (f32) {
         s.g.nseg = 3;
         s.g.seg[0] = GemmSeg{pl.vt_hi, pl.hT_hi, kt};
         s.g.seg[1] = GemmSeg{pl.vt_hi, pl.hT_lo, kt};
@@ -571,14 +619,18 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
         s.c_out_f32 = (float*)dW_out + (size_t)v0 * H;
       else
         s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
-      rc = run_store_gemm(s, g_tune.gemm_variant, st);
+      rc = pl.kmajor ? run_store_gemm_kmajor(s, true, true, st) : run_store_gemm(s, g_tune.gemm_variant, st);
       if (rc) return rc;
     }
     if (dbias_out) {
       float* o32 = f32 ? (float*)dbias_out + v0 : nullptr;
       bf16_t* o16 = f32 ? nullptr : (bf16_t*)dbias_out + v0;
-      hipLaunchKernelGGL(panel_row_sum_kernel, dim3((rows + 3) / 4), dim3(256), 0, st, pl.vt_hi, pl.vt_lo,
-                         (long long)pl.Tpad, rows, T, o32, o16);
+      if (pl.kmajor)
+        hipLaunchKernelGGL(panel_col_sum_kernel, dim3((rows + 63) / 64), dim3(256), 0, st, pl.tv_hi, pl.tv_lo,
+                           (long long)pl.panel, T, rows, o32, o16);
+      else
+        hipLaunchKernelGGL(panel_row_sum_kernel, dim3((rows + 3) / 4), dim3(256), 0, st, pl.vt_hi, pl.vt_lo,
+                           (long long)pl.Tpad, rows, T, o32, o16);
       HIP_TRY(hipGetLastError());
     }
   }
@@ -755,6 +807,31 @@ int fgrpo_gemm_nt(const void* A, const void* B, int M, int N, int K, long long l
   int rc = run_store_gemm(s, variant, (hipStream_t)stream);
   g_tune.small_variant = keep;
   return rc;
+}
+
+int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long long lda, long long ldb, int a_kmajor,
+                      int b_kmajor, int k_valid, const float* c_in, float* c_out_f32, void* c_out_bf16, long long ldc,
+                      float alpha, void* stream) {
+  if (!A || !B || (!c_out_f32 == !c_out_bf16)) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: need A, B and exactly one output");
+  if (ldc < N) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: ldc < N");
+  if (!a_kmajor && !b_kmajor) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: neither operand is K-major");
+  if (k_valid < 0 || k_valid > K) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: k_valid=%d", k_valid);
+  StoreParams s;
+  memset(&s, 0, sizeof(s));
+  s.g.M = M;
+  s.g.N = N;
+  s.g.lda = lda;
+  s.g.ldb = ldb;
+  s.g.nseg = 1;
+  s.g.seg[0] = GemmSeg{(const bf16_t*)A, (const bf16_t*)B, K};
+  s.g.ka_valid = (a_kmajor && !b_kmajor) ? k_valid : 0;
+  s.g.kb_valid = b_kmajor ? k_valid : 0;
+  s.c_in = c_in;
+  s.c_out_f32 = c_out_f32;
+  s.c_out_bf16 = (bf16_t*)c_out_bf16;
+  s.ldc = ldc;
+  s.alpha = alpha;
+  return run_store_gemm_kmajor(s, a_kmajor != 0, b_kmajor != 0, (hipStream_t)stream);
 }
 
 }  // extern "C"

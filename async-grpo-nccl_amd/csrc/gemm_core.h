@@ -54,6 +54,9 @@ struct GemmOperands {
   int nseg;
   long long lda, ldb;  // elements
   int M, N;
+  // K-major operands only (gemm_mainloop_km): rows k >= ka_valid / kb_valid do not exist in memory
+  // and are read as row (valid - 1); the other operand is zero there.  0 = every row of K exists.
+  int ka_valid, kb_valid;
 };
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int NST_ = 2, bool DMA_ = false>
@@ -558,6 +561,211 @@ __device__ __forceinline__ void gemm_mainloop_la(const GemmOperands& g, int row0
     cur = nx;
     nst = (nst + 1 == NST) ? 0 : nst + 1;
   }
+}
+
+// ---------------------------------------------------------------------------
+// Main loop for operands stored "K-major" (the contraction index is the ROW
+// index: X[k][m], m contiguous), as dLogits [token][vocab], hidden [token][H] and
+// W [vocab][H] are when the contraction runs over tokens or vocabulary.  No
+// transposed copy is made: the tile goes to LDS as it lies in memory (two k rows
+// of 256 columns per wavefront-wide direct-to-LDS load) and the MFMA operand is
+// assembled by ds_read_b64_tr_b16, which hands lane i of every 16-lane group the
+// i-th column of a 4 (k) x 16 (m) block whose rows are addressed by lanes
+// 4e .. 4e+3.  Two such reads give the eight consecutive k values of a
+// 32x32x16 operand.  16-byte chunks of a row are XOR-swizzled with 4*(k%4) so
+// that the four rows one read touches fall into different banks.
+// Either operand may instead be K-contiguous (X[m][k]) and is then handled as in
+// gemm_mainloop_dma.  One segment, BM = BN = 256, BK = 64, two LDS buffers.
+// ---------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4_t;
+
+__device__ __forceinline__ bf16x8_t lds_read_tr_pair(const char* p0, const char* p1) {
+  const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p0));
+  const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p1));
+  typedef __attribute__((__vector_size__(8 * sizeof(short)))) short i16x8_t;
+  const i16x8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
+template <class C, bool AKM, bool BKM>
+__device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0, int col0, char* smem,
+                                                 f32x16_t (&acc)[C::TM][C::TN]) {
+  static_assert(C::DMA && C::NSTAGE == 2 && C::BM == 256 && C::BN == 256 && C::BK == 64, "K-major loop: 256x256x64, 2 buffers");
+  constexpr int LPT = C::PA + C::PB;
+  constexpr int KK = C::BK / 16;
+  constexpr int KROWB = 512;                    // bytes of one k row of a K-major tile (256 columns)
+  constexpr int REG = C::BM * C::ROWB;          // bytes of one operand region (32 KiB either way)
+  static_assert(C::ROWB == 128 && REG == C::BK * KROWB, "region size");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+
+  // ---- loader ------------------------------------------------------------------------------
+  uint32_t aoff[C::PA], boff[C::PB];
+  int akrow[C::PA], bkrow[C::PB];               // tile k row of each K-major load (tail clamping)
+  uint32_t acol = 0, bcol = 0;                  // byte offset of the fetched chunk inside its row
+  long long astep, bstep;                       // bytes to advance per K step
+  {
+    const int lrow = lane / C::CPR, lpc = lane % C::CPR;
+    const int amax = g.M - 1 - row0, bmax = g.N - 1 - col0;
+#pragma unroll
+    for (int i = 0; i < C::PA; ++i) {
+      if constexpr (AKM) {
+        const int kr = (i * C::NW + wave) * 2 + (lane >> 5);
+        akrow[i] = kr;
+        acol = (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
+        aoff[i] = (uint32_t)((long long)kr * g.lda * 2) + acol;
+      } else {
+        const int rt = (i * C::NW + wave) * C::RPI + lrow;
+        const int r = rt < amax ? rt : amax;
+        akrow[i] = 0;
+        aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < C::PB; ++i) {
+      if constexpr (BKM) {
+        const int kr = (i * C::NW + wave) * 2 + (lane >> 5);
+        bkrow[i] = kr;
+        bcol = (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
+        boff[i] = (uint32_t)((long long)kr * g.ldb * 2) + bcol;
+      } else {
+        const int rt = (i * C::NW + wave) * C::RPI + lrow;
+        const int r = rt < bmax ? rt : bmax;
+        bkrow[i] = 0;
+        boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+      }
+    }
+  }
+  const char* A0 = AKM ? (const char*)(g.seg[0].A + row0) : (const char*)(g.seg[0].A + (long long)row0 * g.lda);
+  const char* B0 = BKM ? (const char*)(g.seg[0].B + col0) : (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
+  astep = AKM ? (long long)C::BK * g.lda * 2 : (long long)C::BK * 2;
+  bstep = BKM ? (long long)C::BK * g.ldb * 2 : (long long)C::BK * 2;
+  const long long lda2 = g.lda * 2, ldb2 = g.ldb * 2;
+  const int ka_valid = (AKM && g.ka_valid > 0) ? g.ka_valid : 0x7fffffff;
+  const int kb_valid = (BKM && g.kb_valid > 0) ? g.kb_valid : 0x7fffffff;
+  const int dst_w = wave * 1024;                // both layouts: one load fills 1 KiB, loads i are NW KiB apart
+
+  const int nk_total = g.seg[0].K / C::BK;
+  const char* Ai = A0;
+  const char* Bi = B0;
+  int kissue = 0;                               // first k of the step being issued
+  auto issue_one = [&](int stage, int idx) {
+    char* base = smem + stage * C::STAGE;
+    if (idx < C::PA) {
+      const char* src;
+      if constexpr (AKM) {                       // rows past the end read the last valid row (no branch)
+        int kr = kissue + akrow[idx];
+        kr = kr < ka_valid ? kr : ka_valid - 1;
+        src = A0 + (long long)kr * lda2 + acol;
+      } else {
+        src = Ai + aoff[idx];
+      }
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(src), FGRPO_LDS_PTR(base + dst_w + idx * C::NW * 1024), 16, 0,
+                                       FGRPO_DMA_AUX);
+    } else {
+      const int ib = idx - C::PA;
+      const char* src;
+      if constexpr (BKM) {
+        int kr = kissue + bkrow[ib];
+        kr = kr < kb_valid ? kr : kb_valid - 1;
+        src = B0 + (long long)kr * ldb2 + bcol;
+      } else {
+        src = Bi + boff[ib];
+      }
+      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(src), FGRPO_LDS_PTR(base + REG + dst_w + ib * C::NW * 1024), 16,
+                                       0, FGRPO_DMA_AUX);
+    }
+    if (idx == LPT - 1) {
+      Ai += astep;
+      Bi += bstep;
+      kissue += C::BK;
+    }
+  };
+
+  // ---- fragment addressing -------------------------------------------------------------------
+  // K-contiguous operand: row (lane%32), chunk (2*kk + lane/32) ^ swizzle(row)
+  const int swn = lds_swizzle<C>(lane & 31);
+  int frn_c[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) frn_c[kk] = ((kk * 2 + (lane >> 5)) ^ swn) * 16;
+  const int frn_a = (wm * C::WTM + (lane & 31)) * C::ROWB;
+  const int frn_b = REG + (wn * C::WTN + (lane & 31)) * C::ROWB;
+  // K-major operand: lane l = 16*g + j supplies row k = 16*kk + 8*(g/2) + 4*r + j/4 and the 8 bytes at
+  // column (g%2)*16 + 4*(j%4) of the 32-column block; chunk index XOR 4*(k%4) = 4*(j/4)
+  const int j4 = (lane & 15) >> 2;
+  const int frk_row = (8 * (lane >> 5) + j4) * KROWB;                         // + (16*kk + 4*r) * KROWB
+  const int frk_sw = j4 << 2;
+  const int frk_cl = (((lane >> 4) & 1) * 16 + 4 * (lane & 3)) >> 3;          // chunk of the lane's column inside a block
+  const int frk_half = (lane & 1) * 8;
+  auto km_off = [&](int block_col0) {            // byte offset of this lane's 8 bytes inside a k row
+    return ((((block_col0 >> 3) + frk_cl) ^ frk_sw) << 4) + frk_half;
+  };
+  int fka[C::TM], fkb[C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) fka[i] = frk_row + km_off(wm * C::WTM + i * 32);
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) fkb[j] = REG + frk_row + km_off(wn * C::WTN + j * 32);
+
+  auto load_a = [&](const char* st, int i, int kk) -> bf16x8_t {
+    if constexpr (AKM)
+      return lds_read_tr_pair(st + fka[i] + (16 * kk) * KROWB, st + fka[i] + (16 * kk + 4) * KROWB);
+    else
+      return *(const bf16x8_t*)(st + frn_a + i * 32 * C::ROWB + frn_c[kk]);
+  };
+  auto load_b = [&](const char* st, int j, int kk) -> bf16x8_t {
+    if constexpr (BKM)
+      return lds_read_tr_pair(st + fkb[j] + (16 * kk) * KROWB, st + fkb[j] + (16 * kk + 4) * KROWB);
+    else
+      return *(const bf16x8_t*)(st + frn_b + j * 32 * C::ROWB + frn_c[kk]);
+  };
+
+  // ---- pipeline: two buffers, the loads of step kt+1 are spread over the first half of step kt ----
+  FGRPO_WAIT_VMCNT(0);
+  if (nk_total > 0) {
+#pragma unroll
+    for (int idx = 0; idx < LPT; ++idx) issue_one(0, idx);
+  }
+  constexpr int kGroups = KK * C::TM;
+  constexpr int kSpreadG = kGroups / 2;
+  constexpr int kPer = (LPT + kSpreadG - 1) / kSpreadG;
+  int cur = 0;
+  for (int kt = 0; kt < nk_total; ++kt) {
+    FGRPO_WAIT_VMCNT(0);
+    wg_barrier();
+    const bool more = kt + 1 < nk_total;
+    const char* st = smem + cur * C::STAGE;
+    const int nxt = cur ^ 1;
+    bf16x8_t af[2][C::TM], bf[2][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) af[0][i] = load_a(st, i, 0);
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) bf[0][j] = load_b(st, j, 0);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) af[(kk + 1) & 1][i] = load_a(st, i, kk + 1);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) bf[(kk + 1) & 1][j] = load_b(st, j, kk + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
+        if (more) {
+#pragma unroll
+          for (int q = 0; q < kPer; ++q)
+            if ((kk * C::TM + i) * kPer + q < LPT) issue_one(nxt, (kk * C::TM + i) * kPer + q);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    cur = nxt;
+  }
+  wg_barrier();
 }
 
 template <class C>

@@ -280,7 +280,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
   for (int j = 0; j < C::TN; ++j) {
     const int n = col0 + acc_col<C>(wn, j, lane);
     const bool tok_ok = n < T;
-    const float lse2 = tok_ok ? p.lse[n] * kLog2e : 0.f;
+    const float lse2 = tok_ok ? p.lse[n] * kLog2e : -kNegBig;  // padding columns: probability exactly 0
     const long long lab = tok_ok ? p.labels[n] : -100;
     const float c = (lab != -100) ? p.gtok[n] * go : 0.f;  // ignored tokens carry no gradient
     // target row relative to this lane's first row; out of range when not in this sub-tile
@@ -316,10 +316,12 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
           *(uint2*)(tv_lo + rr0) = pk;
         }
         // [vocab][token]: lanes hold consecutive tokens
+        if (p.vt_hi != nullptr) {   // absent when the consumer GEMM reads the [token][vocab] copy K-major
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          vt_hi[(long long)(rr0 + e) * p.ld_vt] = h[e];
-          if (SPLIT) vt_lo[(long long)(rr0 + e) * p.ld_vt] = l[e];
+          for (int e = 0; e < 4; ++e) {
+            vt_hi[(long long)(rr0 + e) * p.ld_vt] = h[e];
+            if (SPLIT) vt_lo[(long long)(rr0 + e) * p.ld_vt] = l[e];
+          }
         }
       }
     }
@@ -369,7 +371,7 @@ __device__ __forceinline__ void store_tile(const StoreParams& p, f32x16_t (&acc)
   }
 }
 
-template <class C>
+template <class C, bool AKM = false, bool BKM = false>
 __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StoreParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -387,7 +389,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
 
   f32x16_t acc[C::TM][C::TN];
   zero_acc<C>(acc);
-  run_mainloop<C>(p.g, row0, col0, smem, acc);
+  if constexpr (AKM || BKM)
+    gemm_mainloop_km<C, AKM, BKM>(p.g, row0, col0, smem, acc);
+  else
+    run_mainloop<C>(p.g, row0, col0, smem, acc);
 
   const float alpha = p.alpha * (p.alpha_dev ? *p.alpha_dev : 1.f);
   const int mode = (p.c_in ? 1 : 0) | (p.c_out_bf16 ? 2 : 0);
@@ -457,6 +462,29 @@ __global__ __launch_bounds__(256) void convert_pad_kernel(const ConvertParams p)
 __global__ void to_f32_kernel(const void* src, int src_is_f32, float* dst, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = src_is_f32 ? ((const float*)src)[i] : bf16_to_f32(((const bf16_t*)src)[i]);
+}
+
+// dbias from the [token][vocab] panel alone: out[v] = sum_t tv[t][v].  One block owns 64 columns; its four
+// row groups are combined in a fixed order, so the result does not depend on scheduling.
+__global__ void panel_col_sum_kernel(const bf16_t* tv_hi, const bf16_t* tv_lo, long long ld, int rows_t, int cols,
+                                     float* out_f32, bf16_t* out_bf16) {
+  __shared__ float red[4][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + tx;
+  float s = 0.f;
+  if (c < cols) {
+    for (int t = ty; t < rows_t; t += 4) {
+      s += bf16_to_f32(tv_hi[(long long)t * ld + c]);
+      if (tv_lo) s += bf16_to_f32(tv_lo[(long long)t * ld + c]);
+    }
+  }
+  red[ty][tx] = s;
+  __syncthreads();
+  if (ty == 0 && c < cols) {
+    const float r = (red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]);
+    if (out_f32) out_f32[c] = r;
+    if (out_bf16) out_bf16[c] = f32_to_bf16_rn(r);
+  }
 }
 
 // bias gradient: db[v] = sum_t dS[v][t] over one [vocab][token] panel

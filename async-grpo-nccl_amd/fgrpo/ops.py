@@ -376,6 +376,24 @@ def gemm_nt(A: torch.Tensor, B: torch.Tensor, out_dtype=torch.float32, c_in: Opt
     return out
 
 
+def gemm_kmajor(A: torch.Tensor, B: torch.Tensor, a_kmajor: bool, b_kmajor: bool, M: int, N: int, K: int,
+                k_valid: int = 0, out_dtype=torch.float32, c_in: Optional[torch.Tensor] = None,
+                alpha: float = 1.0) -> torch.Tensor:
+    """Test hook: C[m,n] = alpha * sum_k A(m,k) B(n,k) (+ c_in) with A given as [K', lda] when ``a_kmajor``
+    (else [M, K]) and B likewise; leading dimensions are the tensors' row strides."""
+    dev = _require_cuda(A, B)
+    lib = _lib.load()
+    assert A.stride(1) == 1 and B.stride(1) == 1
+    out = torch.empty((M, N), dtype=out_dtype, device=dev)
+    o32 = _ptr(out) if out_dtype == torch.float32 else None
+    o16 = _ptr(out) if out_dtype == torch.bfloat16 else None
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_gemm_kmajor(_ptr(A), _ptr(B), M, N, K, A.stride(0), B.stride(0), int(a_kmajor), int(b_kmajor),
+                                   int(k_valid), _ptr(c_in), o32, o16, N, float(alpha), _stream())
+    _lib.check(rc, "gemm_kmajor")
+    return out
+
+
 # --------------------------------------------------------------------------- autograd
 class _LMHeadLogprob(torch.autograd.Function):
     """(hidden, weight, bias, labels_shifted) -> (lp, entropy); entropy carries no gradient."""

@@ -159,6 +159,17 @@ int fgrpo_gemm_nt(const void* A, const void* B, int M, int N, int K, long long l
                   const float* c_in, float* c_out_f32, void* c_out_bf16, long long ldc, float alpha,
                   int variant, void* stream);
 
+/* Same contraction with operands stored contraction-major, as the gradient GEMMs
+ * of fgrpo_lmhead_bwd read dLogits [token][vocab], W [vocab][H] and hidden
+ * [token][H] in place: a_kmajor != 0 means A is [K x M] (lda >= M rounded up to
+ * 256), else [M x K]; likewise B.  k_valid > 0: rows k >= k_valid of the K-major
+ * operand (of B when both are K-major) are not read; the other operand must
+ * exist and hold zeros there.  K a multiple of 64.  No counterpart in the
+ * reference. */
+int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long long lda, long long ldb,
+                      int a_kmajor, int b_kmajor, int k_valid, const float* c_in, float* c_out_f32,
+                      void* c_out_bf16, long long ldc, float alpha, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

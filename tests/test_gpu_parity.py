@@ -154,6 +154,55 @@ def test_bias_and_temperature(dev):
         check(want, got, o, g, f32=(dtype == "fp32"))
 
 
+# ------------------------------------------------------------------ gradient GEMMs on operands read in place
+@pytest.mark.parametrize("layout,M,N,K,k_valid", [
+    ("b", 512, 256, 128, 0),
+    ("b", 1000, 768, 640, 577),       # contraction tail: rows 577.. of B do not exist
+    ("ab", 256, 256, 64, 0),
+    ("ab", 700, 512, 320, 300),
+    ("ab", 1024, 1536, 1024, 1000),
+    ("a", 512, 300, 192, 0),
+])
+def test_contraction_major_gemm_against_torch(dev, layout, M, N, K, k_valid):
+    """C = A B^T with A and/or B stored [K][M] / [K][N]; fp32 accumulation of bf16 products is exact up to
+    summation order, so the fp32 matmul of the same bf16 numbers is the reference."""
+    from fgrpo import ops
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    kr = k_valid if k_valid else K
+    a_km, b_km = "a" in layout, "b" in layout
+    Mp = (M + 255) // 256 * 256
+    A = torch.randn((K, Mp) if a_km else (M, K), generator=gen).bfloat16()
+    B = torch.randn((kr, N) if b_km else (N, K), generator=gen).bfloat16()
+    if k_valid:                        # the operand that exists past k_valid holds zeros there
+        if a_km:
+            A[k_valid:, :] = 0
+        else:
+            A[:, k_valid:] = 0
+    Am = (A[:kr, :M].float().t() if a_km else A[:, :kr].float())
+    Bm = (B.float() if b_km else B[:, :kr].float().t())
+    ref = Am @ Bm
+    out = ops.gemm_kmajor(A.to(dev), B.to(dev), a_km, b_km, M, N, K, k_valid)
+    torch.cuda.synchronize()
+    assert (out.cpu() - ref).abs().max().item() <= 1e-5 * ref.abs().max().item() * math.sqrt(K)
+
+
+@pytest.mark.parametrize("kmajor", [0, 1, 2])
+def test_backward_operand_layout_modes_agree(dev, kmajor):
+    """The backward with transposed copies (0), with dLogits/hidden read in place (1) and with W read in
+    place too (2): each against the oracle, with a bias so that the column-sum dbias path runs, at a shape
+    large enough for the in-place path to be chosen (tokens and vocabulary not multiples of the tile)."""
+    from fgrpo import _lib
+    from fgrpo.synthetic import make_workload
+    w = make_workload("cfg1", seed=6, overrides=dict(H=1024, V=8500, tokens=8100, len_lo=8, len_hi=400, h_scale=1.0))
+    bias = (torch.randn(w.V, generator=torch.Generator().manual_seed(10)) * 0.3).to(w.dtype)
+    _lib.set_tuning(bwd_kmajor=kmajor)
+    try:
+        want, got, o, g, _, _ = run_case(w, dev, "north_star", bias=bias)
+    finally:
+        _lib.set_tuning(bwd_kmajor=1)
+    check(want, got, o, g, f32=False)
+
+
 # ------------------------------------------------------------------ edge cases of the reference
 def test_all_masked_dummy_batch(dev):
     import grpo_loss as G
