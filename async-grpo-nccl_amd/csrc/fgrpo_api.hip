@@ -68,7 +68,7 @@ const CfgInfo kCfg[kNumCfg] = {info_of<Cfg0>(1), info_of<Cfg1>(1), info_of<Cfg2>
                                 info_of<Cfg5>(1), info_of<Cfg6>(1), info_of<Cfg7>(2), info_of<Cfg8>(1), info_of<Cfg9>(1)};
 
 struct Tuning {
-  int fwd_variant = 9;
+  int fwd_variant = 8;
   int ds_variant = 8;
   int gemm_variant = 8;
   int fwd_nsplit = 0;   // 0 = heuristic
@@ -138,11 +138,14 @@ int check_operands(const GemmOperands& g, int bk) {
     if (!g.seg[s].A || !g.seg[s].B) return fail(FGRPO_ERR_BAD_ARG, "gemm: null operand in segment %d", s);
     if (!aligned16(g.seg[s].A) || !aligned16(g.seg[s].B)) return fail(FGRPO_ERR_ALIGN, "gemm: operand of segment %d not 16-byte aligned", s);
     if (g.seg[s].K <= 0 || g.seg[s].K % bk) return fail(FGRPO_ERR_UNSUPPORTED, "gemm: K=%d of segment %d not a positive multiple of %d", g.seg[s].K, s, bk);
-    if (g.seg[s].K > g.lda || g.seg[s].K > g.ldb) return fail(FGRPO_ERR_BAD_ARG, "gemm: K=%d exceeds a leading dimension", g.seg[s].K);
+    if ((g.a_blk == 0 && g.seg[s].K > g.lda) || g.seg[s].K > g.ldb)
+      return fail(FGRPO_ERR_BAD_ARG, "gemm: K=%d exceeds a leading dimension", g.seg[s].K);
   }
   // a tile's rows must be addressable with 32-bit byte offsets
   if (256LL * g.lda * 2 >= (1LL << 32) || 256LL * g.ldb * 2 >= (1LL << 32))
     return fail(FGRPO_ERR_UNSUPPORTED, "gemm: leading dimension too large");
+  if (g.a_blk != 0 && (g.lda != 256 || g.nseg != 1 || g.a_blk % 8 || g.a_blk < 256LL * g.M))
+    return fail(FGRPO_ERR_BAD_ARG, "gemm: column-blocked A needs lda = 256, one segment and blocks of at least M rows");
   return 0;
 }
 
@@ -306,7 +309,9 @@ int run_store_gemm_kmajor(StoreParams p, bool akm, bool bkm, hipStream_t st) {
   p.tiles_m = (g.M + Cfg8::BM - 1) / Cfg8::BM;
   p.tiles_n = (g.N + Cfg8::BN - 1) / Cfg8::BN;
   // a K-major tile is read 256 columns wide without clamping: the rows must hold them
-  if (akm && (long long)p.tiles_m * Cfg8::BM > g.lda) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): lda < padded M");
+  if (g.a_blk != 0 && (g.lda != 256 || g.a_blk % 8 || g.a_blk < 256LL * (akm ? g.seg[0].K : g.M)))
+    return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): column-blocked A needs lda = 256 and blocks that hold every row");
+  if (akm && g.a_blk == 0 && (long long)p.tiles_m * Cfg8::BM > g.lda) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): lda < padded M");
   if (bkm && (long long)p.tiles_n * Cfg8::BN > g.ldb) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): ldb < padded N");
   if (256LL * g.lda * 2 >= (1LL << 32) || 256LL * g.ldb * 2 >= (1LL << 32))
     return fail(FGRPO_ERR_UNSUPPORTED, "gemm(k-major): leading dimension too large");
@@ -320,6 +325,7 @@ int run_store_gemm_kmajor(StoreParams p, bool akm, bool bkm, hipStream_t st) {
 
 int run_store_gemm(StoreParams p, int variant, hipStream_t st) {
   variant = pick_variant(variant, p.g.M, p.g.N);
+  if (p.g.a_blk != 0 && variant != 6 && variant != 7 && variant != 8) variant = 8;  // loops that know the layout
   const CfgInfo& c = kCfg[variant];
   int rc = check_operands(p.g, c.bk);
   if (rc) return rc;
@@ -381,7 +387,7 @@ void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long h
   {
     const long long th = (long long)((T + 255) / 256) * (H / 256);
     const long long vh = (long long)(((V < pl.panel ? V : pl.panel) + 255) / 256) * (H / 256);
-    pl.kmajor = g_tune.bwd_kmajor && !pl.copy_ops && H % 256 == 0 && pl.bm % 64 == 0 && pl.bn % 64 == 0 &&
+    pl.kmajor = g_tune.bwd_kmajor && !pl.copy_ops && H % 256 == 0 && pl.bm == 256 && pl.bn % 64 == 0 &&
                 th >= num_cus() / 2 && vh >= num_cus() / 2;
     pl.kmajor_dh = pl.kmajor && g_tune.bwd_kmajor >= 2;
   }
@@ -537,6 +543,10 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
   d.vt_lo = pl.vt_lo;
   d.ld_tv = pl.panel;
   d.ld_vt = pl.Tpad;
+  // in-place mode keeps the [token][vocab] panel as 256-column blocks: the dW GEMM then streams each block
+  // top to bottom, and the dH GEMM reads 128 KiB contiguous pieces
+  const long long tv_blk = pl.kmajor ? (long long)pl.Tpad * 256 : 0;
+  d.tv_blk = tv_blk;
 
   for (int pi = 0; pi < pl.npanels; ++pi) {
     const int v0 = pi * pl.panel;
@@ -557,7 +567,8 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
       memset(&s, 0, sizeof(s));
       s.g.M = T;
       s.g.N = H;
-      s.g.lda = pl.panel;
+      s.g.lda = tv_blk ? 256 : pl.panel;
+      s.g.a_blk = tv_blk;
       s.g.ldb = pl.Vpad;
       if (pl.kmajor_dh) {  // B = W[v0 + k][h] read in place; vocabulary rows past V do not exist
         s.g.nseg = 1;
@@ -601,7 +612,8 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
       if (pl.kmajor) {  // A = dS[t][v] and B = hidden[t][h], both read in place with t as the contraction index
         s.g.nseg = 1;
         s.g.seg[0] = GemmSeg{pl.tv_hi, (const bf16_t*)hidden, kt};
-        s.g.lda = pl.panel;
+        s.g.lda = 256;
+        s.g.a_blk = tv_blk;
         s.g.ldb = H;
         s.g.kb_valid = T;
       } else if (f32) {
@@ -627,7 +639,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
       bf16_t* o16 = f32 ? nullptr : (bf16_t*)dbias_out + v0;
       if (pl.kmajor)
         hipLaunchKernelGGL(panel_col_sum_kernel, dim3((rows + 63) / 64), dim3(256), 0, st, pl.tv_hi, pl.tv_lo,
-                           (long long)pl.panel, T, rows, o32, o16);
+                           (long long)pl.panel, tv_blk, T, rows, o32, o16);
       else
         hipLaunchKernelGGL(panel_row_sum_kernel, dim3((rows + 3) / 4), dim3(256), 0, st, pl.vt_hi, pl.vt_lo,
                            (long long)pl.Tpad, rows, T, o32, o16);
@@ -810,11 +822,11 @@ int fgrpo_gemm_nt(const void* A, const void* B, int M, int N, int K, long long l
 }
 
 int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long long lda, long long ldb, int a_kmajor,
-                      int b_kmajor, int k_valid, const float* c_in, float* c_out_f32, void* c_out_bf16, long long ldc,
-                      float alpha, void* stream) {
+                      int b_kmajor, long long a_blk, int k_valid, const float* c_in, float* c_out_f32,
+                      void* c_out_bf16, long long ldc, float alpha, void* stream) {
   if (!A || !B || (!c_out_f32 == !c_out_bf16)) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: need A, B and exactly one output");
   if (ldc < N) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: ldc < N");
-  if (!a_kmajor && !b_kmajor) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: neither operand is K-major");
+  if (!a_kmajor && !b_kmajor && !a_blk) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: plain layouts go through gemm_nt");
   if (k_valid < 0 || k_valid > K) return fail(FGRPO_ERR_BAD_ARG, "gemm_kmajor: k_valid=%d", k_valid);
   StoreParams s;
   memset(&s, 0, sizeof(s));
@@ -824,6 +836,7 @@ int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long lo
   s.g.ldb = ldb;
   s.g.nseg = 1;
   s.g.seg[0] = GemmSeg{(const bf16_t*)A, (const bf16_t*)B, K};
+  s.g.a_blk = a_blk;
   s.g.ka_valid = (a_kmajor && !b_kmajor) ? k_valid : 0;
   s.g.kb_valid = b_kmajor ? k_valid : 0;
   s.c_in = c_in;
@@ -831,6 +844,13 @@ int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long lo
   s.c_out_bf16 = (bf16_t*)c_out_bf16;
   s.ldc = ldc;
   s.alpha = alpha;
+  if (!a_kmajor && !b_kmajor) {  // K-contiguous operands, A column-blocked
+    const int keep = g_tune.small_variant;
+    g_tune.small_variant = -1;
+    const int rc = run_store_gemm(s, 8, (hipStream_t)stream);
+    g_tune.small_variant = keep;
+    return rc;
+  }
   return run_store_gemm_kmajor(s, a_kmajor != 0, b_kmajor != 0, (hipStream_t)stream);
 }
 

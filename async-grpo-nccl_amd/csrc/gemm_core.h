@@ -22,6 +22,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
+#include <utility>
 
 #ifdef FGRPO_EXP_NO_MFMA  // experiment: keep the data movement, drop the arithmetic
 #define FGRPO_MFMA(a, b, c) (c)
@@ -57,6 +59,12 @@ struct GemmOperands {
   // K-major operands only (gemm_mainloop_km): rows k >= ka_valid / kb_valid do not exist in memory
   // and are read as row (valid - 1); the other operand is zero there.  0 = every row of K exists.
   int ka_valid, kb_valid;
+  // Column-blocked A (direct-to-LDS two/three-buffer loops and gemm_mainloop_km only): when a_blk != 0 the
+  // logical matrix X[r][c] (r = row as stored, c = contiguous index) is kept as 256-column blocks,
+  // X[r][c] at A + (c / 256) * a_blk + r * 256 + (c % 256) elements (lda must be 256).  A tile that walks
+  // down the rows of one block (K-major use) then reads one sequential stream, and a tile that walks along
+  // the columns (K-contiguous use) reads 128 KiB contiguous pieces.
+  long long a_blk;
 };
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int NST_ = 2, bool DMA_ = false>
@@ -234,6 +242,135 @@ __device__ __forceinline__ void wg_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// The fragment reads of the two-buffer direct-to-LDS loops are written as inline assembly: for an LDS access it can see, the
+// compiler waits (vmcnt) for every direct-to-LDS load in flight, which would serialise the prefetch of the
+// next K step behind each fragment read.  The price: the compiler does not count these reads either, so
+// the loop waits for them itself (s_waitcnt lgkmcnt(n); LDS operations return in order).
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t lds_addr(const char* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+template <int OFF0, int OFF1>
+__device__ __forceinline__ bf16x8_t lds_read_tr_pair(uint32_t addr) {
+  static_assert(OFF0 >= 0 && OFF1 < 65536, "DS offset field");
+  u32x2_t lo, hi;
+  asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+               : "=&v"(lo), "=&v"(hi)
+               : "v"(addr), "i"(OFF0), "i"(OFF1));
+  const u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+template <int OFF>
+__device__ __forceinline__ bf16x8_t lds_read_b128_asm(uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "DS offset field");
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
+// ---------------------------------------------------------------------------
+// Two-buffer schedule shared by the direct-to-LDS loops ("barrier one sub-step early").
+// The barrier of step kt sits before its LAST 16-wide sub-step: by then every
+// wavefront has its last fragments of buffer `cur` in registers and the loads of
+// step kt+1 have landed, so (a) the first fragments of step kt+1 are fetched right
+// after the barrier and arrive under the MFMAs of the last sub-step (no LDS
+// latency is exposed), and (b) buffer `cur` is free from that point: the loads of
+// step kt+2 start into it at once, spread one by one over the MFMA groups of the
+// next EB_PHASES sub-steps, which leaves them the rest of the step to land.
+//   issue_one(stage, idx): load idx (0 .. LPT-1) of the next K step into `stage`;
+//                          idx == LPT-1 also advances the source cursor.
+//   load_a/load_b(stage_ptr, block, kk): one MFMA operand from LDS.
+// On entry the loads of step 0 have been issued into buffer 0 (if nk_total > 0).
+// ---------------------------------------------------------------------------
+#ifndef FGRPO_EB_PHASES
+#define FGRPO_EB_PHASES 2
+#endif
+// compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N-1>{})
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+//   load_a/load_b(stage_ptr, I, KK): one MFMA operand from LDS (I, KK are std::integral_constant)
+//   wait_frags(newer): called before the MFMAs of a sub-step; `newer` = 1 if the fragments of the following
+//                      sub-step were requested after the ones about to be used, else 0.  A no-op when the
+//                      fragment reads are ordinary loads (the compiler counts them itself).
+template <class C, int LPT, class IssueOne, class LoadA, class LoadB, class WaitFrags>
+__device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem, f32x16_t (&acc)[C::TM][C::TN],
+                                                       IssueOne&& issue_one, LoadA&& load_a, LoadB&& load_b,
+                                                       WaitFrags&& wait_frags) {
+  constexpr int KK = C::BK / 16;
+  static_assert(KK % 2 == 0 && KK >= FGRPO_EB_PHASES + 1, "sub-steps per K step");
+  constexpr int NSLOT = FGRPO_EB_PHASES * C::TM;      // MFMA groups over which one step's loads are spread
+  FGRPO_WAIT_VMCNT(0);
+  wg_barrier();                                       // step 0 is in buffer 0
+  int steps_issued = nk_total > 0 ? 1 : 0;
+  bool active = steps_issued < nk_total;              // a step is being loaded
+  int tgt = 1;                                        // ... into this buffer
+  if (active) {
+    ++steps_issued;
+    static_for<LPT>([&](auto q) {
+      if constexpr (decltype(q)::value * NSLOT / LPT < C::TM) issue_one(1, decltype(q)::value);  // phase 0's share
+    });
+  }
+  bf16x8_t af[2][C::TM], bf[2][C::TN];
+  static_for<C::TM>([&](auto i) { af[0][decltype(i)::value] = load_a(smem, i, std::integral_constant<int, 0>{}); });
+  static_for<C::TN>([&](auto j) { bf[0][decltype(j)::value] = load_b(smem, j, std::integral_constant<int, 0>{}); });
+  int cur = 0;
+  for (int kt = 0; kt < nk_total; ++kt) {
+    const char* st = smem + cur * C::STAGE;
+    const char* sn = smem + (cur ^ 1) * C::STAGE;
+    const bool next = kt + 1 < nk_total;
+    static_for<KK>([&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value;
+      int newer = 0;
+      if constexpr (kk + 1 < KK) {
+        static_for<C::TM>([&](auto i) {
+          af[(kk + 1) & 1][decltype(i)::value] = load_a(st, i, std::integral_constant<int, kk + 1>{});
+        });
+        static_for<C::TN>([&](auto j) {
+          bf[(kk + 1) & 1][decltype(j)::value] = load_b(st, j, std::integral_constant<int, kk + 1>{});
+        });
+        newer = 1;
+      } else if (next) {
+        FGRPO_WAIT_VMCNT_LGKM0(0);                    // my loads of step kt+1 landed; my reads of `cur` returned
+        wg_barrier();
+        static_for<C::TM>([&](auto i) { af[0][decltype(i)::value] = load_a(sn, i, std::integral_constant<int, 0>{}); });
+        static_for<C::TN>([&](auto j) { bf[0][decltype(j)::value] = load_b(sn, j, std::integral_constant<int, 0>{}); });
+        newer = 1;
+        active = steps_issued < nk_total;             // loads of step kt+2 go into the buffer just freed
+        tgt = cur;
+        if (active) ++steps_issued;
+      }
+      // phase of the load spreading this sub-step belongs to: 0 = last sub-step, then 1, 2 .. from the top
+      constexpr int phase = (kk == KK - 1) ? 0 : kk + 1;
+      const bool loads_here = active && phase < FGRPO_EB_PHASES && (phase > 0 || next);
+      wait_frags(newer);
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<C::TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
+        if constexpr (phase < FGRPO_EB_PHASES) {
+          if (loads_here) {
+            static_for<LPT>([&](auto q) {
+              if constexpr (decltype(q)::value * NSLOT / LPT == phase * C::TM + i) issue_one(tgt, decltype(q)::value);
+            });
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+    cur ^= 1;
+  }
+  wg_barrier();                                       // LDS may be reused by the caller
+}
+
 template <class C>
 __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row0, int col0, char* smem,
                                                   f32x16_t (&acc)[C::TM][C::TN]) {
@@ -278,6 +415,25 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   int iseg = 0, ileft = g.seg[0].K / C::BK;
   const char* Ai = (const char*)(g.seg[0].A + (long long)row0 * g.lda);
   const char* Bi = (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
+  // after the last load of a K step: next K slice, next 256-column block of a blocked A, next segment
+  constexpr int kStepsPerBlk = 256 / C::BK;
+  const long long a_jump = g.a_blk ? g.a_blk * 2 - 512 : 0;     // bytes added when a block of A is exhausted
+  int ablk_left = kStepsPerBlk;
+  auto advance = [&]() {
+    Ai += C::BK * 2;
+    Bi += C::BK * 2;
+    if (--ablk_left == 0) {
+      Ai += a_jump;
+      ablk_left = kStepsPerBlk;
+    }
+    if (--ileft == 0 && iseg + 1 < g.nseg) {
+      ++iseg;
+      ileft = g.seg[iseg].K / C::BK;
+      Ai = (const char*)(g.seg[iseg].A + (long long)row0 * g.lda);
+      Bi = (const char*)(g.seg[iseg].B + (long long)col0 * g.ldb);
+      ablk_left = kStepsPerBlk;
+    }
+  };
   auto issue = [&](int stage) {
 #ifdef FGRPO_EXP_NO_GLOBAL  // experiment: no global traffic at all
     return;
@@ -291,14 +447,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
     for (int i = 0; i < C::PB; ++i)
       __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[i]),
                                        FGRPO_LDS_PTR(base + dst_b + i * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
-    Ai += C::BK * 2;
-    Bi += C::BK * 2;
-    if (--ileft == 0 && iseg + 1 < g.nseg) {
-      ++iseg;
-      ileft = g.seg[iseg].K / C::BK;
-      Ai = (const char*)(g.seg[iseg].A + (long long)row0 * g.lda);
-      Bi = (const char*)(g.seg[iseg].B + (long long)col0 * g.ldb);
-    }
+    advance();
   };
 
   // One load of the current issue step (idx < PA: operand A, else B); the last one advances the cursor.
@@ -314,22 +463,40 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
       __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[idx - C::PA]),
                                        FGRPO_LDS_PTR(base + dst_b + (idx - C::PA) * C::NW * C::RPI * C::ROWB), 16, 0,
                                        FGRPO_DMA_AUX);
-    if (idx == LPT - 1) {
-      Ai += C::BK * 2;
-      Bi += C::BK * 2;
-      if (--ileft == 0 && iseg + 1 < g.nseg) {
-        ++iseg;
-        ileft = g.seg[iseg].K / C::BK;
-        Ai = (const char*)(g.seg[iseg].A + (long long)row0 * g.lda);
-        Bi = (const char*)(g.seg[iseg].B + (long long)col0 * g.ldb);
-      }
-    }
+    if (idx == LPT - 1) advance();
   };
 
   // loads issued before this call (by the caller's epilogue) must not be mistaken for ours
   FGRPO_WAIT_VMCNT(0);
   int issued = 0;
   for (; issued < D && issued < nk_total; ++issued) issue(issued);
+
+#ifndef FGRPO_EARLY_BARRIER
+#define FGRPO_EARLY_BARRIER 1
+#endif
+  if constexpr (C::NSTAGE == 2 && FGRPO_EARLY_BARRIER && (C::BK / 16) % 2 == 0) {
+    early_barrier_pipeline<C, LPT>(
+        nk_total, smem, acc, issue_one,
+        [&](const char* st, auto i, auto kk) {
+#ifdef FGRPO_EXP_NO_LDSREAD
+          return FGRPO_LDFRAG(st);
+#endif
+          return lds_read_b128_asm<decltype(i)::value * 32 * C::ROWB>(lds_addr(st) + fr_a + fr_c[decltype(kk)::value]);
+        },
+        [&](const char* st, auto j, auto kk) {
+#ifdef FGRPO_EXP_NO_LDSREAD
+          return FGRPO_LDFRAG(st);
+#endif
+          return lds_read_b128_asm<decltype(j)::value * 32 * C::ROWB>(lds_addr(st) + fr_b + fr_c[decltype(kk)::value]);
+        },
+        [](int newer) {
+          if (newer)
+            __builtin_amdgcn_s_waitcnt(0xC07F | ((C::TM + C::TN) << 8));   // lgkmcnt(TM + TN): the newer reads may fly
+          else
+            __builtin_amdgcn_s_waitcnt(0xC07F);                            // lgkmcnt(0)
+        });
+    return;
+  }
 
   // The loads of a step are interleaved with its MFMAs (a burst right after the barrier would keep
   // every wavefront busy issuing addresses, about 40 cycles per load, before its first MFMA).
@@ -577,16 +744,6 @@ __device__ __forceinline__ void gemm_mainloop_la(const GemmOperands& g, int row0
 // Either operand may instead be K-contiguous (X[m][k]) and is then handled as in
 // gemm_mainloop_dma.  One segment, BM = BN = 256, BK = 64, two LDS buffers.
 // ---------------------------------------------------------------------------
-typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4_t;
-
-__device__ __forceinline__ bf16x8_t lds_read_tr_pair(const char* p0, const char* p1) {
-  const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p0));
-  const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p1));
-  typedef __attribute__((__vector_size__(8 * sizeof(short)))) short i16x8_t;
-  const i16x8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  return __builtin_bit_cast(bf16x8_t, v);
-}
-
 template <class C, bool AKM, bool BKM>
 __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0, int col0, char* smem,
                                                  f32x16_t (&acc)[C::TM][C::TN]) {
@@ -638,7 +795,9 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
       }
     }
   }
-  const char* A0 = AKM ? (const char*)(g.seg[0].A + row0) : (const char*)(g.seg[0].A + (long long)row0 * g.lda);
+  // K-major A kept in 256-column blocks: tile column block row0/256 is one [K][256] matrix of its own
+  const char* A0 = AKM ? (const char*)(g.seg[0].A + (g.a_blk ? (long long)(row0 >> 8) * g.a_blk : (long long)row0))
+                       : (const char*)(g.seg[0].A + (long long)row0 * g.lda);
   const char* B0 = BKM ? (const char*)(g.seg[0].B + col0) : (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
   astep = AKM ? (long long)C::BK * g.lda * 2 : (long long)C::BK * 2;
   bstep = BKM ? (long long)C::BK * g.ldb * 2 : (long long)C::BK * 2;
@@ -651,7 +810,12 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   const char* Ai = A0;
   const char* Bi = B0;
   int kissue = 0;                               // first k of the step being issued
+  const long long a_jump = (!AKM && g.a_blk) ? g.a_blk * 2 - 512 : 0;
+  int ablk_left = 256 / C::BK;
   auto issue_one = [&](int stage, int idx) {
+#ifdef FGRPO_EXP_NO_GLOBAL
+    return;
+#endif
     char* base = smem + stage * C::STAGE;
     if (idx < C::PA) {
       const char* src;
@@ -681,6 +845,12 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
       Ai += astep;
       Bi += bstep;
       kissue += C::BK;
+      if constexpr (!AKM) {                      // K-contiguous A kept in 256-column blocks
+        if (--ablk_left == 0) {
+          Ai += a_jump;
+          ablk_left = 256 / C::BK;
+        }
+      }
     }
   };
 
@@ -708,64 +878,43 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
 #pragma unroll
   for (int j = 0; j < C::TN; ++j) fkb[j] = REG + frk_row + km_off(wn * C::WTN + j * 32);
 
-  auto load_a = [&](const char* st, int i, int kk) -> bf16x8_t {
+  auto load_a = [&](const char* st, auto ic, auto kc) -> bf16x8_t {
+    constexpr int i = decltype(ic)::value, kk = decltype(kc)::value;
+#ifdef FGRPO_EXP_NO_LDSREAD
+    return FGRPO_LDFRAG(st);
+#endif
     if constexpr (AKM)
-      return lds_read_tr_pair(st + fka[i] + (16 * kk) * KROWB, st + fka[i] + (16 * kk + 4) * KROWB);
+      return lds_read_tr_pair<(16 * kk) * KROWB, (16 * kk + 4) * KROWB>(lds_addr(st) + fka[i]);
     else
-      return *(const bf16x8_t*)(st + frn_a + i * 32 * C::ROWB + frn_c[kk]);
+      return lds_read_b128_asm<i * 32 * C::ROWB>(lds_addr(st) + frn_a + frn_c[kk]);
   };
-  auto load_b = [&](const char* st, int j, int kk) -> bf16x8_t {
+  auto load_b = [&](const char* st, auto jc, auto kc) -> bf16x8_t {
+    constexpr int j = decltype(jc)::value, kk = decltype(kc)::value;
+#ifdef FGRPO_EXP_NO_LDSREAD
+    return FGRPO_LDFRAG(st);
+#endif
     if constexpr (BKM)
-      return lds_read_tr_pair(st + fkb[j] + (16 * kk) * KROWB, st + fkb[j] + (16 * kk + 4) * KROWB);
+      return lds_read_tr_pair<(16 * kk) * KROWB, (16 * kk + 4) * KROWB>(lds_addr(st) + fkb[j]);
     else
-      return *(const bf16x8_t*)(st + frn_b + j * 32 * C::ROWB + frn_c[kk]);
+      return lds_read_b128_asm<j * 32 * C::ROWB>(lds_addr(st) + frn_b + frn_c[kk]);
+  };
+  // LDS instructions per sub-step's worth of fragments (what may stay outstanding behind the ones in use)
+  constexpr int kReadsPerSub = C::TM * (AKM ? 2 : 1) + C::TN * (BKM ? 2 : 1);
+  static_assert(kReadsPerSub <= 15, "lgkmcnt field");
+  auto wait_frags = [](int newer) {
+    if (newer)
+      __builtin_amdgcn_s_waitcnt(0xC07F | (kReadsPerSub << 8));   // vmcnt, expcnt untouched; lgkmcnt(kReadsPerSub)
+    else
+      __builtin_amdgcn_s_waitcnt(0xC07F);                         // lgkmcnt(0)
   };
 
-  // ---- pipeline: two buffers, the loads of step kt+1 are spread over the first half of step kt ----
+  // ---- pipeline: two buffers, barrier one sub-step early ----
   FGRPO_WAIT_VMCNT(0);
   if (nk_total > 0) {
 #pragma unroll
     for (int idx = 0; idx < LPT; ++idx) issue_one(0, idx);
   }
-  constexpr int kGroups = KK * C::TM;
-  constexpr int kSpreadG = kGroups / 2;
-  constexpr int kPer = (LPT + kSpreadG - 1) / kSpreadG;
-  int cur = 0;
-  for (int kt = 0; kt < nk_total; ++kt) {
-    FGRPO_WAIT_VMCNT(0);
-    wg_barrier();
-    const bool more = kt + 1 < nk_total;
-    const char* st = smem + cur * C::STAGE;
-    const int nxt = cur ^ 1;
-    bf16x8_t af[2][C::TM], bf[2][C::TN];
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i) af[0][i] = load_a(st, i, 0);
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j) bf[0][j] = load_b(st, j, 0);
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      if (kk + 1 < KK) {
-#pragma unroll
-        for (int i = 0; i < C::TM; ++i) af[(kk + 1) & 1][i] = load_a(st, i, kk + 1);
-#pragma unroll
-        for (int j = 0; j < C::TN; ++j) bf[(kk + 1) & 1][j] = load_b(st, j, kk + 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < C::TM; ++i) {
-#pragma unroll
-        for (int j = 0; j < C::TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
-        if (more) {
-#pragma unroll
-          for (int q = 0; q < kPer; ++q)
-            if ((kk * C::TM + i) * kPer + q < LPT) issue_one(nxt, (kk * C::TM + i) * kPer + q);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    cur = nxt;
-  }
-  wg_barrier();
+  early_barrier_pipeline<C, LPT>(nk_total, smem, acc, issue_one, load_a, load_b, wait_frags);
 }
 
 template <class C>

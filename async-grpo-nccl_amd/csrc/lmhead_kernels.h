@@ -6,6 +6,7 @@
 // the lane and need one cross-lane step (lanes l and l^32) at the very end.
 #pragma once
 #include "gemm_core.h"
+#include <type_traits>
 
 namespace fgrpo {
 
@@ -14,12 +15,14 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rn(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+// fp32 -> bf16, round to nearest even, through the hardware conversion (v_cvt_pk_bf16_f32)
+typedef __bf16 hwbf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, hwbf16x2_t));
 }
+__device__ __forceinline__ uint16_t f32_to_bf16_rn(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
 
 // (m1,s1,x1) (+) (m2,s2,x2) for sums of exp(v - m) and exp(v - m) * v.
@@ -83,6 +86,8 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
     zero_acc<C>(acc);
     run_mainloop<C>(p.g, row0, col0, smem, acc);
 
+    // Statistics are kept in units of the raw product (before the temperature): inv_temp > 0 commutes with
+    // the maximum, enters the exponent through one fused multiply-add, and scales m and sum(e*x) once at the end.
     const bool edge = row0 + C::BM > V;
     if (p.bias != nullptr || edge) {
 #pragma unroll
@@ -92,20 +97,11 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
           const int v = row0 + acc_row<C>(wm, i, r, lane);
           const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
 #pragma unroll
-          for (int j = 0; j < C::TN; ++j) {
-            const float x = (acc[i][j][r] + b) * p.inv_temp;
-            acc[i][j][r] = (v < V) ? x : kNegBig;
-          }
+          for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
         }
-    } else {
-#pragma unroll
-      for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[i][j][r] *= p.inv_temp;
     }
 
+    const float xs = p.inv_temp * kLog2e;
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
       float mt = kNegBig;
@@ -114,17 +110,17 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
 #pragma unroll
         for (int r = 0; r < 16; ++r) mt = fmaxf(mt, acc[i][j][r]);
       const float mn = fmaxf(m_run[j], mt);
-      const float alpha = fast_exp2((m_run[j] - mn) * kLog2e);
+      const float alpha = fast_exp2((m_run[j] - mn) * xs);
       // a slot that has seen only masked rows keeps (m, s, sx) = (kNegBig, 0, 0):
-      // x*log2e - mb would otherwise be the rounding residue of two 1e30-sized terms
-      const float mb = (mn > 0.5f * kNegBig) ? mn * kLog2e : 0.f;
+      // x*xs - mb would otherwise be the rounding residue of two huge terms
+      const float mb = (mn > 0.5f * kNegBig) ? mn * xs : 0.f;
       float s = s_run[j] * alpha, sx = sx_run[j] * alpha;
 #pragma unroll
       for (int i = 0; i < C::TM; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float x = acc[i][j][r];
-          const float e = fast_exp2(__builtin_fmaf(x, kLog2e, -mb));
+          const float e = fast_exp2(__builtin_fmaf(x, xs, -mb));
           s += e;
           sx = __builtin_fmaf(e, x, sx);
         }
@@ -144,11 +140,17 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
             xv = h ? acc[i][j][r] : xv;
             hit = hit || h;
           }
-        if (hit) p.xt[col0 + acc_col<C>(wn, j, lane)] = xv;
+        if (hit) p.xt[col0 + acc_col<C>(wn, j, lane)] = xv * p.inv_temp;
       }
     }
   }
 
+  // back to logit units (a masked-only slot keeps a huge negative maximum and zero sums)
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) {
+    m_run[j] *= p.inv_temp;
+    sx_run[j] *= p.inv_temp;
+  }
   // lanes l and l^32 hold the same tokens (different vocabulary rows)
 #pragma unroll
   for (int j = 0; j < C::TN; ++j) {
@@ -232,6 +234,8 @@ struct DsParams {
   bf16_t* tv_hi;             // [tiles_t*BN][ld_tv]
   bf16_t* tv_lo;             // low half for the fp32 path, or null
   long long ld_tv;
+  long long tv_blk;          // != 0: [token][vocab] panel kept as 256-column blocks, block b at + b * tv_blk
+                             //       with row length 256 (needs BM == 256); 0: plain rows of ld_tv
   bf16_t* vt_hi;             // [tiles_v*BM][ld_vt]
   bf16_t* vt_lo;
   long long ld_vt;
@@ -261,21 +265,21 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
   zero_acc<C>(acc);
   run_mainloop<C>(p.g, row0, col0, smem, acc);
 
-  if (p.bias != nullptr) {
+  // vocabulary rows past V get a logit that exponentiates to exactly 0; the bias joins the raw product
+  if (p.bias != nullptr || row0 + C::BM > V) {
 #pragma unroll
     for (int i = 0; i < C::TM; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int v = row0 + acc_row<C>(wm, i, r, lane);
-        const float b = (v < V) ? p.bias[v] : 0.f;
+        const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j) acc[i][j][r] += b;
+        for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
       }
   }
-  // rows of this lane inside the wavefront sub-tile that are real vocabulary entries
-  const int vrem = V - (row0 + wm * C::WTM + 4 * (lane >> 5));  // rr < vrem  <=>  v < V
   const float go = (p.gout ? *p.gout : 1.f) * p.inv_temp;
   const float xs = p.inv_temp * kLog2e;
+  const int lane_row0 = wm * C::WTM + 4 * (lane >> 5);   // first row of this lane inside the tile
 #pragma unroll
   for (int j = 0; j < C::TN; ++j) {
     const int n = col0 + acc_col<C>(wn, j, lane);
@@ -283,48 +287,64 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
     const float lse2 = tok_ok ? p.lse[n] * kLog2e : -kNegBig;  // padding columns: probability exactly 0
     const long long lab = tok_ok ? p.labels[n] : -100;
     const float c = (lab != -100) ? p.gtok[n] * go : 0.f;  // ignored tokens carry no gradient
+    const float nc = -c;
     // target row relative to this lane's first row; out of range when not in this sub-tile
-    const int yrel = (lab >= 0 && lab < V) ? (int)(lab - row0) - wm * C::WTM - 4 * (lane >> 5) : -1;
-    bf16_t* tv_hi = p.tv_hi + (long long)n * p.ld_tv + prow0 + wm * C::WTM + 4 * (lane >> 5);
-    bf16_t* tv_lo = SPLIT ? p.tv_lo + (long long)n * p.ld_tv + prow0 + wm * C::WTM + 4 * (lane >> 5) : nullptr;
-    bf16_t* vt_hi = p.vt_hi + (long long)(prow0 + wm * C::WTM + 4 * (lane >> 5)) * p.ld_vt + n;
-    bf16_t* vt_lo = SPLIT ? p.vt_lo + (long long)(prow0 + wm * C::WTM + 4 * (lane >> 5)) * p.ld_vt + n : nullptr;
+    const int yrel = (lab >= 0 && lab < V) ? (int)(lab - row0) - lane_row0 : -1;
+    const long long tv_off = p.tv_blk ? (long long)tv * p.tv_blk + (long long)n * 256 + lane_row0
+                                      : (long long)n * p.ld_tv + prow0 + lane_row0;
+    bf16_t* tv_hi = p.tv_hi + tv_off;
+    bf16_t* tv_lo = SPLIT ? p.tv_lo + tv_off : nullptr;
+    bf16_t* vt_hi = p.vt_hi ? p.vt_hi + (long long)(prow0 + lane_row0) * p.ld_vt + n : nullptr;
+    bf16_t* vt_lo = (SPLIT && p.vt_lo) ? p.vt_lo + (long long)(prow0 + lane_row0) * p.ld_vt + n : nullptr;
+    // Few wavefronts hold a target row at all (64 tokens x WTM of V rows): the common case runs without
+    // the per-element comparison.
+    const bool any_y = __builtin_amdgcn_ballot_w64(yrel >= 0 && yrel < C::WTM) != 0;
+    auto emit = [&](auto with_y) {
 #pragma unroll
-    for (int i = 0; i < C::TM; ++i) {
+      for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        uint16_t h[4], l[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int rr = i * 32 + 8 * q + e;  // row relative to the lane's first row
-          float pr = fast_exp2(__builtin_fmaf(acc[i][j][q * 4 + e], xs, -lse2));
-          pr = (rr < vrem) ? pr : 0.f;
-          float ds = -c * pr;
-          ds = (rr == yrel) ? ds + c : ds;
-          h[e] = f32_to_bf16_rn(ds);
-          if (SPLIT) l[e] = f32_to_bf16_rn(ds - bf16_to_f32(h[e]));
-        }
-        const int rr0 = i * 32 + 8 * q;
-        // [token][vocab]: four consecutive vocabulary entries = one 8-byte store
-        uint2 pk;
-        pk.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
-        pk.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
-        *(uint2*)(tv_hi + rr0) = pk;
-        if (SPLIT) {
-          pk.x = (uint32_t)l[0] | ((uint32_t)l[1] << 16);
-          pk.y = (uint32_t)l[2] | ((uint32_t)l[3] << 16);
-          *(uint2*)(tv_lo + rr0) = pk;
-        }
-        // [vocab][token]: lanes hold consecutive tokens
-        if (p.vt_hi != nullptr) {   // absent when the consumer GEMM reads the [token][vocab] copy K-major
+        for (int q = 0; q < 4; ++q) {
+          const int rr0 = i * 32 + 8 * q;  // row relative to the lane's first row
+          float ds[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            vt_hi[(long long)(rr0 + e) * p.ld_vt] = h[e];
-            if (SPLIT) vt_lo[(long long)(rr0 + e) * p.ld_vt] = l[e];
+            const float pr = fast_exp2(__builtin_fmaf(acc[i][j][q * 4 + e], xs, -lse2));
+            if constexpr (decltype(with_y)::value)
+              ds[e] = __builtin_fmaf(nc, pr, (rr0 + e == yrel) ? c : 0.f);
+            else
+              ds[e] = nc * pr;
+          }
+          // [token][vocab]: four consecutive vocabulary entries = one 8-byte store
+          uint2 pk;
+          pk.x = pack_bf16x2(ds[0], ds[1]);
+          pk.y = pack_bf16x2(ds[2], ds[3]);
+          *(uint2*)(tv_hi + rr0) = pk;
+          uint2 pl;
+          if (SPLIT) {
+            pl.x = pack_bf16x2(ds[0] - __uint_as_float(pk.x << 16), ds[1] - __uint_as_float(pk.x & 0xffff0000u));
+            pl.y = pack_bf16x2(ds[2] - __uint_as_float(pk.y << 16), ds[3] - __uint_as_float(pk.y & 0xffff0000u));
+            *(uint2*)(tv_lo + rr0) = pl;
+          }
+          // [vocab][token] (only when the consumer GEMM wants that copy): lanes hold consecutive tokens
+          if (vt_hi != nullptr) {
+            vt_hi[(long long)(rr0 + 0) * p.ld_vt] = (uint16_t)(pk.x & 0xffffu);
+            vt_hi[(long long)(rr0 + 1) * p.ld_vt] = (uint16_t)(pk.x >> 16);
+            vt_hi[(long long)(rr0 + 2) * p.ld_vt] = (uint16_t)(pk.y & 0xffffu);
+            vt_hi[(long long)(rr0 + 3) * p.ld_vt] = (uint16_t)(pk.y >> 16);
+            if (SPLIT && vt_lo != nullptr) {
+              vt_lo[(long long)(rr0 + 0) * p.ld_vt] = (uint16_t)(pl.x & 0xffffu);
+              vt_lo[(long long)(rr0 + 1) * p.ld_vt] = (uint16_t)(pl.x >> 16);
+              vt_lo[(long long)(rr0 + 2) * p.ld_vt] = (uint16_t)(pl.y & 0xffffu);
+              vt_lo[(long long)(rr0 + 3) * p.ld_vt] = (uint16_t)(pl.y >> 16);
+            }
           }
         }
       }
-    }
+    };
+    if (any_y)
+      emit(std::true_type{});
+    else
+      emit(std::false_type{});
   }
 }
 
@@ -466,16 +486,19 @@ __global__ void to_f32_kernel(const void* src, int src_is_f32, float* dst, int n
 
 // dbias from the [token][vocab] panel alone: out[v] = sum_t tv[t][v].  One block owns 64 columns; its four
 // row groups are combined in a fixed order, so the result does not depend on scheduling.
-__global__ void panel_col_sum_kernel(const bf16_t* tv_hi, const bf16_t* tv_lo, long long ld, int rows_t, int cols,
-                                     float* out_f32, bf16_t* out_bf16) {
+__global__ void panel_col_sum_kernel(const bf16_t* tv_hi, const bf16_t* tv_lo, long long ld, long long blk, int rows_t,
+                                     int cols, float* out_f32, bf16_t* out_bf16) {
   __shared__ float red[4][64];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int c = blockIdx.x * 64 + tx;
   float s = 0.f;
   if (c < cols) {
+    // blk != 0: 256-column blocks of row length 256 (block b at + b * blk)
+    const long long base = blk ? (long long)(c >> 8) * blk + (c & 255) : (long long)c;
+    const long long step = blk ? 256 : ld;
     for (int t = ty; t < rows_t; t += 4) {
-      s += bf16_to_f32(tv_hi[(long long)t * ld + c]);
-      if (tv_lo) s += bf16_to_f32(tv_lo[(long long)t * ld + c]);
+      s += bf16_to_f32(tv_hi[base + (long long)t * step]);
+      if (tv_lo) s += bf16_to_f32(tv_lo[base + (long long)t * step]);
     }
   }
   red[ty][tx] = s;

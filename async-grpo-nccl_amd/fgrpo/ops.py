@@ -73,6 +73,16 @@ def shift_labels(labels: torch.Tensor) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- raw ops
+# Optional timing hook: when a list is installed, every forward launch appends a pair of events recorded on
+# the launch stream right before and right after the library call (nothing is synchronised here).
+_fwd_event_sink = None
+
+
+def set_fwd_event_sink(sink) -> None:
+    global _fwd_event_sink
+    _fwd_event_sink = sink
+
+
 def lmhead_logprob_fwd(hidden: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
                        labels_shifted: torch.Tensor, temperature: float = 1.0,
                        want_entropy: bool = True, want_lse: bool = True):
@@ -104,9 +114,16 @@ def lmhead_logprob_fwd(hidden: torch.Tensor, weight: torch.Tensor, bias: Optiona
     nbytes = lib.fgrpo_logprob_fwd_workspace(T, H, V, code)
     ws = _ws(nbytes, dev)
     with torch.cuda.device(dev):
+        sink = _fwd_event_sink
+        if sink is not None:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
         rc = lib.fgrpo_logprob_fwd(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted),
                                    1.0 / float(temperature), T, H, V, code,
                                    _ptr(lp), _ptr(ent), _ptr(lse), _ptr(ws), ws.numel(), _stream())
+        if sink is not None:
+            e1.record()
+            sink.append((e0, e1))
     _lib.check(rc, "logprob_fwd")
     return lp, ent, lse
 
@@ -378,18 +395,20 @@ def gemm_nt(A: torch.Tensor, B: torch.Tensor, out_dtype=torch.float32, c_in: Opt
 
 def gemm_kmajor(A: torch.Tensor, B: torch.Tensor, a_kmajor: bool, b_kmajor: bool, M: int, N: int, K: int,
                 k_valid: int = 0, out_dtype=torch.float32, c_in: Optional[torch.Tensor] = None,
-                alpha: float = 1.0) -> torch.Tensor:
+                alpha: float = 1.0, a_blk: int = 0) -> torch.Tensor:
     """Test hook: C[m,n] = alpha * sum_k A(m,k) B(n,k) (+ c_in) with A given as [K', lda] when ``a_kmajor``
-    (else [M, K]) and B likewise; leading dimensions are the tensors' row strides."""
+    (else [M, K]) and B likewise; leading dimensions are the tensors' row strides.  ``a_blk`` != 0: A is a
+    buffer of 256-column blocks, ``a_blk`` elements apart, each with rows of 256."""
     dev = _require_cuda(A, B)
     lib = _lib.load()
-    assert A.stride(1) == 1 and B.stride(1) == 1
+    assert A.stride(-1) == 1 and B.stride(1) == 1
     out = torch.empty((M, N), dtype=out_dtype, device=dev)
     o32 = _ptr(out) if out_dtype == torch.float32 else None
     o16 = _ptr(out) if out_dtype == torch.bfloat16 else None
+    lda = 256 if a_blk else A.stride(0)
     with torch.cuda.device(dev):
-        rc = lib.fgrpo_gemm_kmajor(_ptr(A), _ptr(B), M, N, K, A.stride(0), B.stride(0), int(a_kmajor), int(b_kmajor),
-                                   int(k_valid), _ptr(c_in), o32, o16, N, float(alpha), _stream())
+        rc = lib.fgrpo_gemm_kmajor(_ptr(A), _ptr(B), M, N, K, lda, B.stride(0), int(a_kmajor), int(b_kmajor),
+                                   int(a_blk), int(k_valid), _ptr(c_in), o32, o16, N, float(alpha), _stream())
     _lib.check(rc, "gemm_kmajor")
     return out
 

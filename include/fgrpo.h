@@ -159,16 +159,17 @@ int fgrpo_gemm_nt(const void* A, const void* B, int M, int N, int K, long long l
                   const float* c_in, float* c_out_f32, void* c_out_bf16, long long ldc, float alpha,
                   int variant, void* stream);
 
-/* Same contraction with operands stored contraction-major, as the gradient GEMMs
- * of fgrpo_lmhead_bwd read dLogits [token][vocab], W [vocab][H] and hidden
- * [token][H] in place: a_kmajor != 0 means A is [K x M] (lda >= M rounded up to
- * 256), else [M x K]; likewise B.  k_valid > 0: rows k >= k_valid of the K-major
- * operand (of B when both are K-major) are not read; the other operand must
- * exist and hold zeros there.  K a multiple of 64.  No counterpart in the
- * reference. */
+/* Same contraction with the operand layouts the gradient GEMMs of fgrpo_lmhead_bwd
+ * use to read dLogits, W and hidden in place.  a_kmajor != 0: A is stored [K x M]
+ * (contraction index = row), else [M x K]; likewise B.  a_blk != 0: A is kept as
+ * 256-column blocks, stored element (r, c) at A + (c/256)*a_blk + r*256 + c%256
+ * (lda must be 256; r, c are the row and the contiguous index as stored).
+ * k_valid > 0: rows k >= k_valid of the K-major operand (of B when both are
+ * K-major) are not read; the other operand must exist and hold zeros there.
+ * K a multiple of 64.  No counterpart in the reference. */
 int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long long lda, long long ldb,
-                      int a_kmajor, int b_kmajor, int k_valid, const float* c_in, float* c_out_f32,
-                      void* c_out_bf16, long long ldc, float alpha, void* stream);
+                      int a_kmajor, int b_kmajor, long long a_blk, int k_valid, const float* c_in,
+                      float* c_out_f32, void* c_out_bf16, long long ldc, float alpha, void* stream);
 
 #ifdef __cplusplus
 }
