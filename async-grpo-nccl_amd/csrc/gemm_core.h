@@ -25,11 +25,10 @@
 #include <type_traits>
 #include <utility>
 
-#ifdef FGRPO_EXP_NO_MFMA  // experiment: keep the data movement, drop the arithmetic
-#define FGRPO_MFMA(a, b, c) (c)
-#else
+// Every fragment read must stay consumed by an MFMA: the two-buffer loops issue their LDS reads as inline
+// assembly, and a read whose result is dead lets the register allocator reuse its destination while the
+// data is still in flight (a build that dropped the MFMAs corrupted load addresses that way).
 #define FGRPO_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
-#endif
 
 #define FGRPO_EXP_FRAG_BASE(st) (st)
 #ifdef FGRPO_EXP_NO_LDSREAD  // experiment: MFMA operands never come from LDS
@@ -338,8 +337,15 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
         });
         newer = 1;
       } else if (next) {
+#if defined(FGRPO_EXP_NO_BARRIER)                     // timing experiments only (results are wrong)
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+#elif defined(FGRPO_EXP_NO_VMWAIT)
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        wg_barrier();
+#else
         FGRPO_WAIT_VMCNT_LGKM0(0);                    // my loads of step kt+1 landed; my reads of `cur` returned
         wg_barrier();
+#endif
         static_for<C::TM>([&](auto i) { af[0][decltype(i)::value] = load_a(sn, i, std::integral_constant<int, 0>{}); });
         static_for<C::TN>([&](auto j) { bf[0][decltype(j)::value] = load_b(sn, j, std::integral_constant<int, 0>{}); });
         newer = 1;
