@@ -20,9 +20,11 @@ for p in (os.path.join(ROOT, "async-grpo-nccl_amd"), ROOT):
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 
-# HBM bytes per launch of the forward kernel at cfg1 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (scaled by a copy kernel of known size); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg1": None}
+# Bytes per launch of the forward kernel that leave the L2s, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 1 GiB
+# device copy of --copy-probe: FETCH_SIZE reads 524317.75 KiB for 2^20 KiB (factor 2.0000), WRITE_SIZE reads
+# 1048576 KiB (factor 1.0).  cfg1: 16421681 KiB x 2.0 + 2034 KiB x 1.0.  None for workloads not measured.
+MEASURED_TRAFFIC_BYTES = {"cfg1": 16421681 * 1024 * (1048576 / 524317.75) + 2034 * 1024}
 
 
 def cpu_baseline(name: str, cfg_chunk, seed: int):
