@@ -232,7 +232,10 @@ __device__ __forceinline__ int lds_swizzle(int row) {
   if constexpr (C::CPR == 4)
     return FGRPO_SWZ4(row);                       // 64-byte rows
   else
-    return (row + ((row >> 3) & 1)) & 7;          // 128-byte rows
+#ifndef FGRPO_SWZ8
+#define FGRPO_SWZ8(row) (((row) + (((row) >> 3) & 1)) & 7)
+#endif
+    return FGRPO_SWZ8(row);                       // 128-byte rows
 }
 
 __device__ __forceinline__ void wg_barrier() {
@@ -295,17 +298,46 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-//   load_a/load_b(stage_ptr, I, KK): one MFMA operand from LDS (I, KK are std::integral_constant)
-//   wait_frags(newer): called before the MFMAs of a sub-step; `newer` = 1 if the fragments of the following
-//                      sub-step were requested after the ones about to be used, else 0.  A no-op when the
-//                      fragment reads are ordinary loads (the compiler counts them itself).
-template <class C, int LPT, class IssueOne, class LoadA, class LoadB, class WaitFrags>
+//   load_a/load_b(stage_ptr, I, KK): one MFMA operand from LDS (I, KK are std::integral_constant), issued as
+//   RA / RB inline-assembly LDS instructions that the compiler does not count: this function places every
+//   s_waitcnt lgkmcnt(n) itself (LDS operations return in order).
+// The fragments of the following sub-step are requested between the MFMA row groups of the current one, in the
+// order a0, b0 .. b(TN-1), a1 .. a(TM-1) (row group 0 needs a0 and every b), so that the LDS sees a steady
+// trickle of reads next to the direct-to-LDS stream instead of a burst per sub-step.
+#ifndef FGRPO_EB_FINE
+#define FGRPO_EB_FINE 1
+#endif
+#ifndef FGRPO_EB_STAGGER
+#define FGRPO_EB_STAGGER 0
+#endif
+template <int N>
+__device__ __forceinline__ void wait_lgkm() {
+  static_assert(N >= 0, "wait count");
+  __builtin_amdgcn_s_waitcnt(0xC07F | ((N > 15 ? 15 : N) << 8));   // vmcnt / expcnt untouched
+}
+
+template <class C, int LPT, int RA, int RB, class IssueOne, class LoadA, class LoadB>
 __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem, f32x16_t (&acc)[C::TM][C::TN],
-                                                       IssueOne&& issue_one, LoadA&& load_a, LoadB&& load_b,
-                                                       WaitFrags&& wait_frags) {
+                                                       IssueOne&& issue_one, LoadA&& load_a, LoadB&& load_b) {
   constexpr int KK = C::BK / 16;
+  constexpr int TM = C::TM, TN = C::TN, NR = TM + TN;
   static_assert(KK % 2 == 0 && KK >= FGRPO_EB_PHASES + 1, "sub-steps per K step");
-  constexpr int NSLOT = FGRPO_EB_PHASES * C::TM;      // MFMA groups over which one step's loads are spread
+  constexpr int NSLOT = FGRPO_EB_PHASES * TM;         // MFMA groups over which one step's loads are spread
+  // fragment order and bookkeeping (all compile time)
+  struct Ord {
+    static constexpr int cum(int i) { return FGRPO_EB_FINE ? (i * NR + TM - 1) / TM : (i > 0 ? NR : 0); }  // entries requested before row group i ends.. starts
+    static constexpr int instrs(int n) {              // LDS instructions of the first n entries
+      int c = 0;
+      for (int e = 0; e < n; ++e) c += (e == 0 || e > TN) ? RA : RB;
+      return c;
+    }
+    static constexpr int need(int i) { return i == 0 ? TN : TN + i; }   // last entry row group i waits for
+    // instructions that may still be outstanding when row group i starts
+    static constexpr int allowed(int i, bool issuing) {
+      return instrs(NR) - instrs(need(i) + 1) + (issuing ? instrs(cum(i)) : 0);
+    }
+  };
+  const int team = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) & 1;   // wavefronts w and w+4 share a SIMD
   FGRPO_WAIT_VMCNT(0);
   wg_barrier();                                       // step 0 is in buffer 0
   int steps_issued = nk_total > 0 ? 1 : 0;
@@ -314,12 +346,21 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
   if (active) {
     ++steps_issued;
     static_for<LPT>([&](auto q) {
-      if constexpr (decltype(q)::value * NSLOT / LPT < C::TM) issue_one(1, decltype(q)::value);  // phase 0's share
+      if constexpr (decltype(q)::value * NSLOT / LPT < TM) issue_one(1, decltype(q)::value);  // phase 0's share
     });
   }
-  bf16x8_t af[2][C::TM], bf[2][C::TN];
-  static_for<C::TM>([&](auto i) { af[0][decltype(i)::value] = load_a(smem, i, std::integral_constant<int, 0>{}); });
-  static_for<C::TN>([&](auto j) { bf[0][decltype(j)::value] = load_b(smem, j, std::integral_constant<int, 0>{}); });
+  bf16x8_t af[2][TM], bf[2][TN];
+  // entry e of the request order, for sub-step KN of the buffer at `base`, into register buffer BUF
+  auto request = [&](const char* base, auto ec, auto knc, auto bufc) {
+    constexpr int e = decltype(ec)::value, buf = decltype(bufc)::value;
+    if constexpr (e == 0)
+      af[buf][0] = load_a(base, std::integral_constant<int, 0>{}, knc);
+    else if constexpr (e <= TN)
+      bf[buf][e - 1] = load_b(base, std::integral_constant<int, e - 1>{}, knc);
+    else
+      af[buf][e - TN] = load_a(base, std::integral_constant<int, e - TN>{}, knc);
+  };
+  static_for<NR>([&](auto e) { request(smem, e, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
   int cur = 0;
   for (int kt = 0; kt < nk_total; ++kt) {
     const char* st = smem + cur * C::STAGE;
@@ -327,46 +368,63 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
     const bool next = kt + 1 < nk_total;
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value;
-      int newer = 0;
-      if constexpr (kk + 1 < KK) {
-        static_for<C::TM>([&](auto i) {
-          af[(kk + 1) & 1][decltype(i)::value] = load_a(st, i, std::integral_constant<int, kk + 1>{});
-        });
-        static_for<C::TN>([&](auto j) {
-          bf[(kk + 1) & 1][decltype(j)::value] = load_b(st, j, std::integral_constant<int, kk + 1>{});
-        });
-        newer = 1;
-      } else if (next) {
-#if defined(FGRPO_EXP_NO_BARRIER)                     // timing experiments only (results are wrong)
-        __builtin_amdgcn_s_waitcnt(0xC07F);
-#elif defined(FGRPO_EXP_NO_VMWAIT)
-        __builtin_amdgcn_s_waitcnt(0xC07F);
-        wg_barrier();
-#else
-        FGRPO_WAIT_VMCNT_LGKM0(0);                    // my loads of step kt+1 landed; my reads of `cur` returned
-        wg_barrier();
-#endif
-        static_for<C::TM>([&](auto i) { af[0][decltype(i)::value] = load_a(sn, i, std::integral_constant<int, 0>{}); });
-        static_for<C::TN>([&](auto j) { bf[0][decltype(j)::value] = load_b(sn, j, std::integral_constant<int, 0>{}); });
-        newer = 1;
-        active = steps_issued < nk_total;             // loads of step kt+2 go into the buffer just freed
-        tgt = cur;
-        if (active) ++steps_issued;
+      constexpr bool last = (kk == KK - 1);
+      constexpr int kn = last ? 0 : kk + 1, nbuf = (kk + 1) & 1;
+      const char* src = last ? sn : st;
+      const bool issuing = !last || next;
+      if constexpr (last) {
+        if (next) {
+          FGRPO_WAIT_VMCNT_LGKM0(0);                  // my loads of step kt+1 landed; my reads of `cur` returned
+          wg_barrier();
+          active = steps_issued < nk_total;           // loads of step kt+2 go into the buffer just freed
+          tgt = cur;
+          if (active) ++steps_issued;
+        }
       }
       // phase of the load spreading this sub-step belongs to: 0 = last sub-step, then 1, 2 .. from the top
-      constexpr int phase = (kk == KK - 1) ? 0 : kk + 1;
+      constexpr int phase = last ? 0 : kk + 1;
       const bool loads_here = active && phase < FGRPO_EB_PHASES && (phase > 0 || next);
-      wait_frags(newer);
+      if constexpr (!FGRPO_EB_FINE) {                 // burst: every fragment of the next sub-step up front
+        if (issuing) static_for<NR>([&](auto e) { request(src, e, std::integral_constant<int, kn>{}, std::integral_constant<int, nbuf>{}); });
+        if (issuing) wait_lgkm<Ord::instrs(NR)>(); else wait_lgkm<0>();
+      }
       __builtin_amdgcn_sched_barrier(0);
-      static_for<C::TM>([&](auto ic) {
+      static_for<TM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
+        if constexpr (FGRPO_EB_FINE) {
+          if constexpr (!last) {
+            wait_lgkm<Ord::allowed(i, true)>();
+          } else {
+            if (next) wait_lgkm<Ord::allowed(i, true)>(); else wait_lgkm<Ord::allowed(i, false)>();
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
-        if constexpr (phase < FGRPO_EB_PHASES) {
-          if (loads_here) {
-            static_for<LPT>([&](auto q) {
-              if constexpr (decltype(q)::value * NSLOT / LPT == phase * C::TM + i) issue_one(tgt, decltype(q)::value);
+        for (int j = 0; j < TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
+        if constexpr (FGRPO_EB_FINE) {
+          if (issuing) {
+            static_for<Ord::cum(i + 1) - Ord::cum(i)>([&](auto d) {
+              request(src, std::integral_constant<int, Ord::cum(i) + decltype(d)::value>{}, std::integral_constant<int, kn>{},
+                      std::integral_constant<int, nbuf>{});
             });
+          }
+        }
+        if constexpr (phase < FGRPO_EB_PHASES) {
+          if constexpr (FGRPO_EB_STAGGER && C::NW == 8 && TM % 2 == 0 && LPT % (2 * FGRPO_EB_PHASES) == 0) {
+            // The two wavefronts of a SIMD (w and w+4) issue their loads under different MFMA row groups,
+            // so that while one sits in the vector-memory issue queue the other still feeds the matrix pipe.
+            constexpr int HALF = TM / 2, PER_PHASE = LPT / FGRPO_EB_PHASES, PER_GROUP = PER_PHASE / HALF;
+            if (loads_here && (i / HALF) == team) {
+              static_for<PER_GROUP>([&](auto d) {
+                issue_one(tgt, std::integral_constant<int, phase * PER_PHASE + (i % HALF) * PER_GROUP + decltype(d)::value>{});
+              });
+            }
+          } else {
+            if (loads_here) {
+              static_for<LPT>([&](auto q) {
+                if constexpr (decltype(q)::value * NSLOT / LPT == phase * TM + i) issue_one(tgt, decltype(q)::value);
+              });
+            }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -466,6 +524,9 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
       __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Ai + aoff[idx]),
                                        FGRPO_LDS_PTR(base + dst_a + idx * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
     else
+#ifdef FGRPO_EXP_SKIP_B_ODD   // timing experiment (wrong results): 3/4 of the load volume
+      if (!(ileft & 1))
+#endif
       __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[idx - C::PA]),
                                        FGRPO_LDS_PTR(base + dst_b + (idx - C::PA) * C::NW * C::RPI * C::ROWB), 16, 0,
                                        FGRPO_DMA_AUX);
@@ -481,7 +542,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
 #define FGRPO_EARLY_BARRIER 1
 #endif
   if constexpr (C::NSTAGE == 2 && FGRPO_EARLY_BARRIER && (C::BK / 16) % 2 == 0) {
-    early_barrier_pipeline<C, LPT>(
+    early_barrier_pipeline<C, LPT, 1, 1>(
         nk_total, smem, acc, issue_one,
         [&](const char* st, auto i, auto kk) {
 #ifdef FGRPO_EXP_NO_LDSREAD
@@ -494,12 +555,6 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
           return FGRPO_LDFRAG(st);
 #endif
           return lds_read_b128_asm<decltype(j)::value * 32 * C::ROWB>(lds_addr(st) + fr_b + fr_c[decltype(kk)::value]);
-        },
-        [](int newer) {
-          if (newer)
-            __builtin_amdgcn_s_waitcnt(0xC07F | ((C::TM + C::TN) << 8));   // lgkmcnt(TM + TN): the newer reads may fly
-          else
-            __builtin_amdgcn_s_waitcnt(0xC07F);                            // lgkmcnt(0)
         });
     return;
   }
@@ -904,23 +959,13 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
     else
       return lds_read_b128_asm<j * 32 * C::ROWB>(lds_addr(st) + frn_b + frn_c[kk]);
   };
-  // LDS instructions per sub-step's worth of fragments (what may stay outstanding behind the ones in use)
-  constexpr int kReadsPerSub = C::TM * (AKM ? 2 : 1) + C::TN * (BKM ? 2 : 1);
-  static_assert(kReadsPerSub <= 15, "lgkmcnt field");
-  auto wait_frags = [](int newer) {
-    if (newer)
-      __builtin_amdgcn_s_waitcnt(0xC07F | (kReadsPerSub << 8));   // vmcnt, expcnt untouched; lgkmcnt(kReadsPerSub)
-    else
-      __builtin_amdgcn_s_waitcnt(0xC07F);                         // lgkmcnt(0)
-  };
-
   // ---- pipeline: two buffers, barrier one sub-step early ----
   FGRPO_WAIT_VMCNT(0);
   if (nk_total > 0) {
 #pragma unroll
     for (int idx = 0; idx < LPT; ++idx) issue_one(0, idx);
   }
-  early_barrier_pipeline<C, LPT>(nk_total, smem, acc, issue_one, load_a, load_b, wait_frags);
+  early_barrier_pipeline<C, LPT, AKM ? 2 : 1, BKM ? 2 : 1>(nk_total, smem, acc, issue_one, load_a, load_b);
 }
 
 template <class C>

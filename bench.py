@@ -128,12 +128,16 @@ def main():
     # (the bracket also holds the per-token combine kernel, some tens of microseconds).
     fwd_events = []
     ops.set_fwd_event_sink(fwd_events)
+    step_events = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    step_events[0].record()
+    for i in range(args.steps):
         step()
+        step_events[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ops.set_fwd_event_sink(None)
+    per_step = sorted(step_events[i].elapsed_time(step_events[i + 1]) for i in range(args.steps))
     ms = dt / args.steps * 1e3
     tok_s = T / (ms / 1e3)
     k_ms = sum(a.elapsed_time(b) for a, b in fwd_events) / max(1, len(fwd_events))
@@ -163,6 +167,7 @@ def main():
                      "kernel": "lmhead_fwd_kernel (+ per-token combine)", "kernel_ms": k_ms,
                      "kernel_launches_timed": len(fwd_events),
                      "algorithmic_flops_per_launch": flops_launch},
+        "ms_per_step_median": per_step[len(per_step) // 2], "ms_per_step_min": per_step[0],
         "path_mfma_frac": alg_flops_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "path_algorithmic_tflops": alg_flops_step / (ms * 1e-3) / 1e12,
     }
