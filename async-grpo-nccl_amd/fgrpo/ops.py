@@ -466,6 +466,36 @@ class _FusedGRPOLoss(torch.autograd.Function):
         return (dH, dW, db) + (None,) * 13
 
 
+class _GRPOLossFromLogprobs(torch.autograd.Function):
+    """The dual-clip objective on per-token logprobs that some other autograd graph produced
+    (the materialised-logits path of a caller-supplied ``per_token_fn``)."""
+
+    @staticmethod
+    def forward(ctx, lp, labels_shifted, old_lp, adv, ref_lp, cu_seqlens, clip_low, clip_high, clip_ratio_c, kl_beta,
+                loss_agg_mode, denom_override):
+        loss, g, lr, c1, l1, l2, scal = grpo_loss_fwd(lp.detach(), old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
+                                                      clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
+                                                      denom_override)
+        ctx.save_for_backward(g)
+        ctx.lp_dtype = lp.dtype
+        ctx.mark_non_differentiable(lr, c1, l1, l2)
+        return loss, lr, c1, l1, l2
+
+    @staticmethod
+    def backward(ctx, g_loss, *_unused):
+        (g,) = ctx.saved_tensors
+        return ((g * g_loss).to(ctx.lp_dtype),) + (None,) * 11
+
+
+def grpo_loss_from_logprobs(lp, labels_shifted, old_lp, adv, ref_lp=None, cu_seqlens=None, clip_low=0.2,
+                            clip_high=0.4, clip_ratio_c=1e32, kl_beta=0.0, loss_agg_mode="token_mean",
+                            denom_override=0.0):
+    """(loss, log_ratio, clip1, unclipped, clipped); the gradient flows into ``lp``."""
+    return _GRPOLossFromLogprobs.apply(lp.reshape(-1), labels_shifted, old_lp, adv, ref_lp, cu_seqlens, float(clip_low),
+                                       float(clip_high), float(clip_ratio_c), float(kl_beta), loss_agg_mode,
+                                       float(denom_override))
+
+
 def lmhead_logprob(hidden, weight, bias, labels_shifted, temperature=1.0, panel_hint=0) -> Tuple[torch.Tensor, torch.Tensor]:
     return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint))
 

@@ -19,7 +19,7 @@ Differences a caller can observe, all documented where they occur:
 per-token logprobs are returned in fp32 (the reference returns the logits'
 dtype on its un-chunked path); entropy is computed from fp32 logits (the
 reference rounds logits to bf16 first, grpo_loss.py:245/:310); a foreign
-``per_token_fn`` is rejected because it needs the logits this path never forms.
+``per_token_fn`` (a function of logits) takes the chunked materialised-logits route, as in the reference.
 Extensions reachable through the ``**unused_kwargs`` hole of the reference
 signature: ``ref_logprobs``/``kl_beta`` (k3 KL penalty), ``loss_agg_mode``
 (``"token_mean"`` = reference, ``"sample_mean"``), ``cu_seqlens``,
@@ -134,11 +134,41 @@ COMPUTE_ENTROPY_FN = entropy_from_logits
 _OWN_PER_TOKEN_FNS = (logprobs_from_logits, logprobs_from_logits_flash_attn)
 
 
-def _check_per_token_fn(per_token_fn) -> None:
-    if per_token_fn is not None and per_token_fn not in _OWN_PER_TOKEN_FNS:
-        raise NotImplementedError(
-            "fused LM-head path: a custom per_token_fn needs materialised [tokens x vocab] logits, "
-            "which this implementation never forms; pass logprobs_from_logits (the default)")
+def _is_own_per_token_fn(per_token_fn) -> bool:
+    return per_token_fn is None or per_token_fn in _OWN_PER_TOKEN_FNS
+
+
+def _materialised_log_probs_and_entropy(w, b, hidden_states, shifted_labels, temperature, per_token_fn, chunk):
+    """A caller-supplied ``per_token_fn`` is a function of logits, so for it (and only for it) the logits of one
+    chunk of positions at a time are formed, exactly as the reference does (grpo_loss.py:227-249, 286-313):
+    ``per_token_fn(logits, shifted_labels, vocab_size=V)`` may return the logprobs or ``(logprobs, logits_flat)``;
+    entropy comes from the row kernel on the valid rows.  Gradients reach hidden/weight through torch's own
+    autograd of the projection."""
+    ops._require_cuda(hidden_states, w, shifted_labels)
+    B, L = shifted_labels.shape
+    V = w.shape[0]
+    hs = hidden_states.to(w.dtype)
+    step = int(chunk) if (chunk is not None and chunk > 0) else L
+    lps, ents = [], []
+    for start in range(0, max(L, 1), max(step, 1)):
+        end = min(start + step, L)
+        logits = torch.matmul(hs[:, start:end, :], w.t())
+        if b is not None:
+            logits = logits + b
+        logits = logits / temperature
+        lab = shifted_labels[:, start:end]
+        out = per_token_fn(logits, lab, vocab_size=V)
+        if isinstance(out, tuple):
+            lp_c, logits_flat = out[0], out[1]
+        else:
+            lp_c, logits_flat = out, logits.reshape(-1, logits.shape[-1])
+        lps.append(lp_c.reshape(B, end - start))
+        ent_c = torch.zeros(B * (end - start), device=logits.device, dtype=torch.float32)
+        valid = lab.reshape(-1) != -100
+        if bool(valid.any()):
+            ent_c[valid] = COMPUTE_ENTROPY_FN(logits_flat[valid].detach().bfloat16()).to(ent_c.dtype)
+        ents.append(ent_c.reshape(B, end - start))
+    return torch.cat(lps, dim=1).reshape(-1), torch.cat(ents, dim=1).reshape(-1)
 
 
 def _prep(lm_head_weights, lm_head_bias, hidden_states):
@@ -172,9 +202,11 @@ def fused_log_probs_and_entropy_fn(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """(per-token logprob [B*L] fp32, entropy [B*L] fp32); labels are shifted by
     one inside, masked positions give 0 (reference: grpo_loss.py:211-250)."""
-    _check_per_token_fn(per_token_fn)
-    shifted = ops.shift_labels(labels).reshape(-1)
     w, b, hs = _prep(lm_head_weights, lm_head_bias, hidden_states)
+    if not _is_own_per_token_fn(per_token_fn):
+        return _materialised_log_probs_and_entropy(w, b, hidden_states, ops.shift_labels(labels), temperature,
+                                                   per_token_fn, None)
+    shifted = ops.shift_labels(labels).reshape(-1)
     lp, ent = ops.lmhead_logprob(hs, w, b, shifted, temperature)
     return lp, ent
 
@@ -208,7 +240,6 @@ def grpo_loss_and_entropy_ce_fn(
     grpo_loss.py:256-348).  ``loss_chunksize`` only bounds the transient of the
     backward (a dLogits panel of about ``loss_chunksize * V`` elements); the
     result does not depend on it."""
-    _check_per_token_fn(per_token_fn)
     if advantages is None:
         raise ValueError("grpo_loss_and_entropy_ce_fn: advantages are required")
     ref_logprobs = unused_kwargs.get("ref_logprobs", None)
@@ -222,6 +253,14 @@ def grpo_loss_and_entropy_ce_fn(
     V = w.shape[0]
     hint = int(loss_chunksize) * int(V) if (loss_chunksize is not None and loss_chunksize > 0) else 0
     denom = float(num_samples_total) if (num_samples_total and loss_agg_mode == "sample_mean") else 0.0
+    if not _is_own_per_token_fn(per_token_fn):
+        lp, ent = _materialised_log_probs_and_entropy(w, b, hidden_states, ops.shift_labels(labels), temperature,
+                                                      per_token_fn, loss_chunksize)
+        loss, lr, c1, l1, l2 = ops.grpo_loss_from_logprobs(
+            lp, shifted, None if old_logprobs is None else old_logprobs.reshape(-1), advantages.reshape(-1),
+            None if ref_logprobs is None else ref_logprobs.reshape(-1), cu_seqlens, clip_low, clip_high,
+            clip_ratio_c, kl_beta, loss_agg_mode, denom)
+        return loss, ent, lr, c1, l1, l2
     loss, ent, lr, c1, l1, l2, _lp = ops.fused_grpo_loss(
         hs, w, b, shifted,
         None if old_logprobs is None else old_logprobs.reshape(-1),

@@ -8,6 +8,7 @@ from types import SimpleNamespace
 import numpy as np
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import grpo_oracle as O
 
@@ -225,3 +226,47 @@ def test_trainer_harness_scaling_and_dummy(dev):
     ratio = (g1.float().norm() / g2.float().norm()).item()
     assert abs(ratio - 0.25) < 0.02
     assert tr.compute_gradients([{"dummy": True}], 0) == {"loss": 0.0, "pg_clip": 0, "kl_div": 0.0, "entropy": 0.0}
+
+
+@pytest.mark.parametrize("returns_tuple", [False, True])
+def test_foreign_per_token_fn_takes_the_materialised_route(dev, returns_tuple):
+    """per_token_fn(logits, shifted_labels, vocab_size=V) supplied by the caller (reference: grpo_loss.py:232-239,
+    :296-303, either a tensor or (logprobs, logits_flat)): same loss, diagnostics and gradients as the fused route
+    and as the oracle, with and without chunking."""
+    import grpo_loss as G
+    from fgrpo.synthetic import make_workload
+    w = make_workload("cfg1", seed=8, overrides=dict(H=128, V=3000, tokens=700, len_lo=8, len_hi=120, h_scale=1.0))
+    p = w.params
+    calls = []
+
+    def my_fn(logits, labels, vocab_size=None):
+        calls.append(tuple(logits.shape))
+        assert vocab_size == w.V
+        lp = torch.log_softmax(logits.float(), -1).gather(-1, labels.clamp(min=0).unsqueeze(-1)).squeeze(-1)
+        lp = lp * (labels != -100)
+        return (lp, logits.reshape(-1, logits.shape[-1])) if returns_tuple else lp
+
+    T = w.T
+    adv = torch.randn(T, generator=torch.Generator().manual_seed(3)).to(dev)
+    with torch.no_grad():
+        lp0, _ = G.fused_log_probs_and_entropy_fn(w.weight.to(dev), None, w.hidden.to(dev), w.labels.to(dev))
+    old = lp0 + w.noise_old.to(dev)
+    outs = []
+    for fn, chunk in ((G.logprobs_from_logits, None), (my_fn, None), (my_fn, 256)):
+        hs = w.hidden.to(dev).clone().requires_grad_(True)
+        W = w.weight.to(dev).clone().requires_grad_(True)
+        out = G.grpo_loss_and_entropy_ce_fn(W, None, hs, w.labels.to(dev), 1.0, old, adv, p["clip_low"], p["clip_high"],
+                                            p["clip_ratio_c"], per_token_fn=fn, loss_chunksize=chunk)
+        out[0].backward()
+        outs.append((out, hs.grad, W.grad))
+    assert calls[0] == (1, T, w.V) and len(calls) == 1 + (T + 255) // 256
+    ref = outs[0]
+    for out, dh, dw in outs[1:]:
+        # logits are rounded to bf16 on the materialised route (as in the reference): logprob errors ~1e-2
+        assert abs(out[0].item() - ref[0][0].item()) <= 5e-4
+        assert (out[2] - ref[0][2]).abs().max().item() <= 2e-2
+        assert (out[1] - ref[0][1]).abs().max().item() <= 5e-2
+        assert F.cosine_similarity(dh.float().flatten(), ref[1].float().flatten(), dim=0).item() >= 0.999
+        assert F.cosine_similarity(dw.float().flatten(), ref[2].float().flatten(), dim=0).item() >= 0.999
+    lp_m, ent_m = G.fused_log_probs_and_entropy_fn(w.weight.to(dev), None, w.hidden.to(dev), w.labels.to(dev), per_token_fn=my_fn)
+    assert (lp_m - lp0).abs().max().item() <= 2e-2

@@ -32,9 +32,10 @@ def test_product_path_refuses_cpu_tensors():
         G.logprobs_from_logits(torch.randn(4, 9), torch.zeros(4, dtype=torch.long))
 
 
-def test_foreign_per_token_fn_is_rejected():
+def test_foreign_per_token_fn_needs_the_gpu_too():
+    """A caller-supplied per_token_fn takes the materialised-logits route; that route has no CPU version either."""
     import grpo_loss as G
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="GPU"):
         G.fused_log_probs_and_entropy_fn(torch.randn(4, 4), None, torch.randn(1, 2, 4), torch.zeros(1, 2, dtype=torch.long),
                                          per_token_fn=lambda *a, **k: None)
 
