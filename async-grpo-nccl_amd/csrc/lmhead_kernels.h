@@ -299,7 +299,14 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
     // Few wavefronts hold a target row at all (64 tokens x WTM of V rows): the common case runs without
     // the per-element comparison.
     const bool any_y = __builtin_amdgcn_ballot_w64(yrel >= 0 && yrel < C::WTM) != 0;
-    auto emit = [&](auto with_y) {
+    // Column-blocked panel: a lane's 8 bytes (4 vocabulary entries of one token) would be a 64-line scatter per
+    // store instruction.  The wavefront instead parks 32 tokens x WTM entries in a private LDS patch and writes
+    // them out as 16-byte pieces, 16 lanes per token row: every store instruction fills whole 128-byte lines.
+    constexpr int EROW = C::WTM * 2 + 16;               // patch row: one token's WTM entries + 16 bytes of padding
+    constexpr int PPT = C::WTM * 2 / 16, TPP = 64 / PPT;  // 16-byte pieces per token, tokens per store instruction
+    char* patch = smem + wave * (32 * EROW);
+    static_assert(C::NW * 32 * EROW <= C::LDS_BYTES && 64 % PPT == 0 && 32 % TPP == 0, "epilogue patch");
+    auto emit = [&](auto with_y, auto via_lds) {
 #pragma unroll
       for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
@@ -318,6 +325,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
           uint2 pk;
           pk.x = pack_bf16x2(ds[0], ds[1]);
           pk.y = pack_bf16x2(ds[2], ds[3]);
+          if constexpr (decltype(via_lds)::value) {
+            *(uint2*)(patch + (lane & 31) * EROW + (rr0 + 4 * (lane >> 5)) * 2) = pk;
+            continue;
+          }
           *(uint2*)(tv_hi + rr0) = pk;
           uint2 pl;
           if (SPLIT) {
@@ -340,11 +351,28 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
           }
         }
       }
+      if constexpr (decltype(via_lds)::value) {
+        bf16_t* out = p.tv_hi + (long long)tv * p.tv_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
+#pragma unroll
+        for (int r = 0; r < 32 / TPP; ++r) {
+          const int tok = r * TPP + lane / PPT, piece = lane % PPT;
+          const u32x4_t v = *(const u32x4_t*)(patch + tok * EROW + piece * 16);
+          *(u32x4_t*)(out + (long long)tok * 256 + piece * 8) = v;
+        }
+      }
     };
-    if (any_y)
-      emit(std::true_type{});
-    else
-      emit(std::false_type{});
+    const bool through_lds = !SPLIT && p.tv_blk != 0;
+    if (through_lds) {
+      if (any_y)
+        emit(std::true_type{}, std::true_type{});
+      else
+        emit(std::false_type{}, std::true_type{});
+    } else {
+      if (any_y)
+        emit(std::true_type{}, std::false_type{});
+      else
+        emit(std::false_type{}, std::false_type{});
+    }
   }
 }
 
