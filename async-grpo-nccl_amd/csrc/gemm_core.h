@@ -56,7 +56,7 @@ struct GemmOperands {
   long long lda, ldb;  // elements
   int M, N;
   // K-major operands only (gemm_mainloop_km): rows k >= ka_valid / kb_valid do not exist in memory
-  // and are read as row (valid - 1); the other operand is zero there.  0 = every row of K exists.
+  // and read as zero (buffer bounds).  0 = every row of K exists.
   int ka_valid, kb_valid;
   // Column-blocked A (direct-to-LDS two/three-buffer loops and gemm_mainloop_km only): when a_blk != 0 the
   // logical matrix X[r][c] (r = row as stored, c = contiguous index) is kept as 256-column blocks,
@@ -216,6 +216,11 @@ __device__ __forceinline__ void gemm_mainloop(const GemmOperands& g, int row0, i
 #endif
 #define FGRPO_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define FGRPO_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// Raw buffer descriptor over [base, base + bytes): offsets past `bytes` read as zero.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
 
 // s_waitcnt that waits only for the vector-memory counter to drop to n (n < 64).
 #define FGRPO_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
@@ -443,7 +448,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   static_assert(D >= 1 && D <= 4 && LPT * (D - 1) < 64, "pipeline depth");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront-uniform: LDS targets stay scalar
   const int wm = wave / C::WN, wn = wave % C::WN;
 
   // loader: instruction i of this wavefront covers tile rows (i*NW + wave)*RPI ..
@@ -475,45 +480,41 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   int nk_total = 0;
   for (int s = 0; s < g.nseg; ++s) nk_total += g.seg[s].K / C::BK;
 
-  // issue cursor over (segment, k)
+  // Issue cursor over (segment, k).  The loads are buffer loads: a 128-bit descriptor per operand (base = first
+  // row of the tile in the current segment / column block), the lane's constant byte offset in a VGPR and the
+  // running K offset in an SGPR, so that issuing a load costs two scalar instructions and no vector arithmetic.
   int iseg = 0, ileft = g.seg[0].K / C::BK;
-  const char* Ai = (const char*)(g.seg[0].A + (long long)row0 * g.lda);
-  const char* Bi = (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
+  const char* Abase = (const char*)(g.seg[0].A + (long long)row0 * g.lda);
+  const char* Bbase = (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
+  __amdgpu_buffer_rsrc_t rsa = make_rsrc(Abase, 0xffffffffu);
+  __amdgpu_buffer_rsrc_t rsb = make_rsrc(Bbase, 0xffffffffu);
+  uint32_t ka = 0, kb = 0;                            // byte offset of the K slice being issued
   // after the last load of a K step: next K slice, next 256-column block of a blocked A, next segment
   constexpr int kStepsPerBlk = 256 / C::BK;
-  const long long a_jump = g.a_blk ? g.a_blk * 2 - 512 : 0;     // bytes added when a block of A is exhausted
+  const long long a_blk_bytes = g.a_blk * 2;
   int ablk_left = kStepsPerBlk;
   auto advance = [&]() {
-    Ai += C::BK * 2;
-    Bi += C::BK * 2;
+    ka += C::BK * 2;
+    kb += C::BK * 2;
     if (--ablk_left == 0) {
-      Ai += a_jump;
       ablk_left = kStepsPerBlk;
+      if (a_blk_bytes != 0) {                          // next column block of A: re-base the descriptor
+        Abase += a_blk_bytes;
+        rsa = make_rsrc(Abase, 0xffffffffu);
+        ka = 0;
+      }
     }
     if (--ileft == 0 && iseg + 1 < g.nseg) {
       ++iseg;
       ileft = g.seg[iseg].K / C::BK;
-      Ai = (const char*)(g.seg[iseg].A + (long long)row0 * g.lda);
-      Bi = (const char*)(g.seg[iseg].B + (long long)col0 * g.ldb);
+      Abase = (const char*)(g.seg[iseg].A + (long long)row0 * g.lda);
+      Bbase = (const char*)(g.seg[iseg].B + (long long)col0 * g.ldb);
+      rsa = make_rsrc(Abase, 0xffffffffu);
+      rsb = make_rsrc(Bbase, 0xffffffffu);
+      ka = kb = 0;
       ablk_left = kStepsPerBlk;
     }
   };
-  auto issue = [&](int stage) {
-#ifdef FGRPO_EXP_NO_GLOBAL  // experiment: no global traffic at all
-    return;
-#endif
-    char* base = smem + stage * C::STAGE;
-#pragma unroll
-    for (int i = 0; i < C::PA; ++i)
-      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Ai + aoff[i]),
-                                       FGRPO_LDS_PTR(base + dst_a + i * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
-#pragma unroll
-    for (int i = 0; i < C::PB; ++i)
-      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[i]),
-                                       FGRPO_LDS_PTR(base + dst_b + i * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
-    advance();
-  };
-
   // One load of the current issue step (idx < PA: operand A, else B); the last one advances the cursor.
   auto issue_one = [&](int stage, int idx) {
 #ifdef FGRPO_EXP_NO_GLOBAL
@@ -521,16 +522,16 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
 #endif
     char* base = smem + stage * C::STAGE;
     if (idx < C::PA)
-      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Ai + aoff[idx]),
-                                       FGRPO_LDS_PTR(base + dst_a + idx * C::NW * C::RPI * C::ROWB), 16, 0, FGRPO_DMA_AUX);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsa, FGRPO_LDS_PTR(base + dst_a + idx * C::NW * C::RPI * C::ROWB), 16,
+                                               (int)aoff[idx], (int)ka, 0, FGRPO_DMA_AUX);
     else
-#ifdef FGRPO_EXP_SKIP_B_ODD   // timing experiment (wrong results): 3/4 of the load volume
-      if (!(ileft & 1))
-#endif
-      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[idx - C::PA]),
-                                       FGRPO_LDS_PTR(base + dst_b + (idx - C::PA) * C::NW * C::RPI * C::ROWB), 16, 0,
-                                       FGRPO_DMA_AUX);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsb, FGRPO_LDS_PTR(base + dst_b + (idx - C::PA) * C::NW * C::RPI * C::ROWB),
+                                               16, (int)boff[idx - C::PA], (int)kb, 0, FGRPO_DMA_AUX);
     if (idx == LPT - 1) advance();
+  };
+  auto issue = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) issue_one(stage, i);
   };
 
   // loads issued before this call (by the caller's epilogue) must not be mistaken for ours
@@ -816,14 +817,11 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   static_assert(C::ROWB == 128 && REG == C::BK * KROWB, "region size");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront-uniform
   const int wm = wave / C::WN, wn = wave % C::WN;
 
   // ---- loader ------------------------------------------------------------------------------
-  uint32_t aoff[C::PA], boff[C::PB];
-  int akrow[C::PA], bkrow[C::PB];               // tile k row of each K-major load (tail clamping)
-  uint32_t acol = 0, bcol = 0;                  // byte offset of the fetched chunk inside its row
-  long long astep, bstep;                       // bytes to advance per K step
+  uint32_t aoff[C::PA], boff[C::PB];            // per-lane byte offset of each load inside the step's slice
   {
     const int lrow = lane / C::CPR, lpc = lane % C::CPR;
     const int amax = g.M - 1 - row0, bmax = g.N - 1 - col0;
@@ -831,13 +829,10 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
     for (int i = 0; i < C::PA; ++i) {
       if constexpr (AKM) {
         const int kr = (i * C::NW + wave) * 2 + (lane >> 5);
-        akrow[i] = kr;
-        acol = (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
-        aoff[i] = (uint32_t)((long long)kr * g.lda * 2) + acol;
+        aoff[i] = (uint32_t)((long long)kr * g.lda * 2) + (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
       } else {
         const int rt = (i * C::NW + wave) * C::RPI + lrow;
         const int r = rt < amax ? rt : amax;
-        akrow[i] = 0;
         aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
       }
     }
@@ -845,72 +840,72 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
     for (int i = 0; i < C::PB; ++i) {
       if constexpr (BKM) {
         const int kr = (i * C::NW + wave) * 2 + (lane >> 5);
-        bkrow[i] = kr;
-        bcol = (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
-        boff[i] = (uint32_t)((long long)kr * g.ldb * 2) + bcol;
+        boff[i] = (uint32_t)((long long)kr * g.ldb * 2) + (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
       } else {
         const int rt = (i * C::NW + wave) * C::RPI + lrow;
         const int r = rt < bmax ? rt : bmax;
-        bkrow[i] = 0;
         boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
       }
     }
   }
+  // Buffer loads: the lane's constant byte offset travels in a VGPR, everything that moves is scalar.
+  //  * K-contiguous operand: descriptor on the tile's first row, K offset in an SGPR (re-based per 256-column
+  //    block when A is column-blocked);
+  //  * K-major operand: descriptor re-based on the first k row of every step, with num_records = the bytes of
+  //    the k rows that exist from there on, so rows past the end of the contraction read as zero.
   // K-major A kept in 256-column blocks: tile column block row0/256 is one [K][256] matrix of its own
-  const char* A0 = AKM ? (const char*)(g.seg[0].A + (g.a_blk ? (long long)(row0 >> 8) * g.a_blk : (long long)row0))
+  const char* Ap = AKM ? (const char*)(g.seg[0].A + (g.a_blk ? (long long)(row0 >> 8) * g.a_blk : (long long)row0))
                        : (const char*)(g.seg[0].A + (long long)row0 * g.lda);
-  const char* B0 = BKM ? (const char*)(g.seg[0].B + col0) : (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
-  astep = AKM ? (long long)C::BK * g.lda * 2 : (long long)C::BK * 2;
-  bstep = BKM ? (long long)C::BK * g.ldb * 2 : (long long)C::BK * 2;
+  const char* Bp = BKM ? (const char*)(g.seg[0].B + col0) : (const char*)(g.seg[0].B + (long long)col0 * g.ldb);
   const long long lda2 = g.lda * 2, ldb2 = g.ldb * 2;
-  const int ka_valid = (AKM && g.ka_valid > 0) ? g.ka_valid : 0x7fffffff;
-  const int kb_valid = (BKM && g.kb_valid > 0) ? g.kb_valid : 0x7fffffff;
+  long long a_rem = (AKM && g.ka_valid > 0) ? g.ka_valid : (1LL << 40);   // k rows of A that exist from Ap on
+  long long b_rem = (BKM && g.kb_valid > 0) ? g.kb_valid : (1LL << 40);
+  auto bytes_of = [](long long rows, long long ld2) -> uint32_t {
+    if (rows <= 0) return 0u;
+    const long long bts = rows * ld2;
+    return (rows > (1LL << 31) || bts > 0xffffffffLL) ? 0xffffffffu : (uint32_t)bts;
+  };
+  __amdgpu_buffer_rsrc_t rsa = make_rsrc(Ap, AKM ? bytes_of(a_rem, lda2) : 0xffffffffu);
+  __amdgpu_buffer_rsrc_t rsb = make_rsrc(Bp, BKM ? bytes_of(b_rem, ldb2) : 0xffffffffu);
+  uint32_t ka = 0, kb = 0;                      // running K byte offset of a K-contiguous operand
   const int dst_w = wave * 1024;                // both layouts: one load fills 1 KiB, loads i are NW KiB apart
 
   const int nk_total = g.seg[0].K / C::BK;
-  const char* Ai = A0;
-  const char* Bi = B0;
-  int kissue = 0;                               // first k of the step being issued
-  const long long a_jump = (!AKM && g.a_blk) ? g.a_blk * 2 - 512 : 0;
+  const long long a_blk_bytes = (!AKM) ? g.a_blk * 2 : 0;
   int ablk_left = 256 / C::BK;
   auto issue_one = [&](int stage, int idx) {
 #ifdef FGRPO_EXP_NO_GLOBAL
     return;
 #endif
     char* base = smem + stage * C::STAGE;
-    if (idx < C::PA) {
-      const char* src;
-      if constexpr (AKM) {                       // rows past the end read the last valid row (no branch)
-        int kr = kissue + akrow[idx];
-        kr = kr < ka_valid ? kr : ka_valid - 1;
-        src = A0 + (long long)kr * lda2 + acol;
+    if (idx < C::PA)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsa, FGRPO_LDS_PTR(base + dst_w + idx * C::NW * 1024), 16, (int)aoff[idx],
+                                               (int)ka, 0, FGRPO_DMA_AUX);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsb, FGRPO_LDS_PTR(base + REG + dst_w + (idx - C::PA) * C::NW * 1024), 16,
+                                               (int)boff[idx - C::PA], (int)kb, 0, FGRPO_DMA_AUX);
+    if (idx == LPT - 1) {                        // next K step
+      if constexpr (AKM) {
+        Ap += (long long)C::BK * lda2;
+        a_rem -= C::BK;
+        rsa = make_rsrc(Ap, bytes_of(a_rem, lda2));
       } else {
-        src = Ai + aoff[idx];
-      }
-      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(src), FGRPO_LDS_PTR(base + dst_w + idx * C::NW * 1024), 16, 0,
-                                       FGRPO_DMA_AUX);
-    } else {
-      const int ib = idx - C::PA;
-      const char* src;
-      if constexpr (BKM) {
-        int kr = kissue + bkrow[ib];
-        kr = kr < kb_valid ? kr : kb_valid - 1;
-        src = B0 + (long long)kr * ldb2 + bcol;
-      } else {
-        src = Bi + boff[ib];
-      }
-      __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(src), FGRPO_LDS_PTR(base + REG + dst_w + ib * C::NW * 1024), 16,
-                                       0, FGRPO_DMA_AUX);
-    }
-    if (idx == LPT - 1) {
-      Ai += astep;
-      Bi += bstep;
-      kissue += C::BK;
-      if constexpr (!AKM) {                      // K-contiguous A kept in 256-column blocks
+        ka += C::BK * 2;
         if (--ablk_left == 0) {
-          Ai += a_jump;
           ablk_left = 256 / C::BK;
+          if (a_blk_bytes != 0) {                // K-contiguous A kept in 256-column blocks: next block
+            Ap += a_blk_bytes;
+            rsa = make_rsrc(Ap, 0xffffffffu);
+            ka = 0;
+          }
         }
+      }
+      if constexpr (BKM) {
+        Bp += (long long)C::BK * ldb2;
+        b_rem -= C::BK;
+        rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2));
+      } else {
+        kb += C::BK * 2;
       }
     }
   };
