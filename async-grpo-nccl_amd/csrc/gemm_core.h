@@ -367,28 +367,31 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
   };
   static_for<NR>([&](auto e) { request(smem, e, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
   int cur = 0;
-  for (int kt = 0; kt < nk_total; ++kt) {
+  // One K step.  STEADY: at least two more steps follow, so a next step exists and a further one is always
+  // there to be loaded; the body then carries no conditionals at all.
+  auto step = [&](int kt, auto steady_c) {
+    constexpr bool STEADY = decltype(steady_c)::value;
     const char* st = smem + cur * C::STAGE;
     const char* sn = smem + (cur ^ 1) * C::STAGE;
-    const bool next = kt + 1 < nk_total;
+    const bool next = STEADY || kt + 1 < nk_total;
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value;
       constexpr bool last = (kk == KK - 1);
       constexpr int kn = last ? 0 : kk + 1, nbuf = (kk + 1) & 1;
       const char* src = last ? sn : st;
-      const bool issuing = !last || next;
+      const bool issuing = STEADY || !last || next;
       if constexpr (last) {
         if (next) {
           FGRPO_WAIT_VMCNT_LGKM0(0);                  // my loads of step kt+1 landed; my reads of `cur` returned
           wg_barrier();
-          active = steps_issued < nk_total;           // loads of step kt+2 go into the buffer just freed
+          active = STEADY || steps_issued < nk_total; // loads of step kt+2 go into the buffer just freed
           tgt = cur;
           if (active) ++steps_issued;
         }
       }
       // phase of the load spreading this sub-step belongs to: 0 = last sub-step, then 1, 2 .. from the top
       constexpr int phase = last ? 0 : kk + 1;
-      const bool loads_here = active && phase < FGRPO_EB_PHASES && (phase > 0 || next);
+      const bool loads_here = STEADY || (active && phase < FGRPO_EB_PHASES && (phase > 0 || next));
       if constexpr (!FGRPO_EB_FINE) {                 // burst: every fragment of the next sub-step up front
         if (issuing) static_for<NR>([&](auto e) { request(src, e, std::integral_constant<int, kn>{}, std::integral_constant<int, nbuf>{}); });
         if (issuing) wait_lgkm<Ord::instrs(NR)>(); else wait_lgkm<0>();
@@ -436,7 +439,10 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
       });
     });
     cur ^= 1;
-  }
+  };
+  int kt = 0;
+  for (; kt + 2 < nk_total; ++kt) step(kt, std::true_type{});
+  for (; kt < nk_total; ++kt) step(kt, std::false_type{});
   wg_barrier();                                       // LDS may be reused by the caller
 }
 
