@@ -22,9 +22,10 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 
 # Bytes per launch of the forward kernel that leave the L2s, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 1 GiB
-# device copy of --copy-probe: FETCH_SIZE reads 524317.75 KiB for 2^20 KiB (factor 2.0000), WRITE_SIZE reads
-# 1048576 KiB (factor 1.0).  cfg1: 16421681 KiB x 2.0 + 2034 KiB x 1.0.  None for workloads not measured.
-MEASURED_TRAFFIC_BYTES = {"cfg1": 16421681 * 1024 * (1048576 / 524317.75) + 2034 * 1024}
+# device copy of --copy-probe: FETCH_SIZE reads 524317.4 KiB for 2^20 KiB (factor 2.0000), WRITE_SIZE reads
+# 1048576 KiB (factor 1.0).  cfg1, launches of the timed steps: 10995346 KiB x 2.0 + 3046 KiB x 1.0.
+# None for workloads not measured.
+MEASURED_TRAFFIC_BYTES = {"cfg1": 10995346 * 1024 * (1048576 / 524317.4) + 3046 * 1024}
 
 
 def cpu_baseline(name: str, cfg_chunk, seed: int):
