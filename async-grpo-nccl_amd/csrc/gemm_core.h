@@ -30,12 +30,7 @@
 // data is still in flight (a build that dropped the MFMAs corrupted load addresses that way).
 #define FGRPO_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
 
-#define FGRPO_EXP_FRAG_BASE(st) (st)
-#ifdef FGRPO_EXP_NO_LDSREAD  // experiment: MFMA operands never come from LDS
-#define FGRPO_LDFRAG(ptr) (__builtin_bit_cast(bf16x8_t, u32x4_t{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, (uint32_t)threadIdx.x}))
-#else
 #define FGRPO_LDFRAG(ptr) (*(const bf16x8_t*)(ptr))
-#endif
 
 namespace fgrpo {
 
@@ -211,9 +206,7 @@ __device__ __forceinline__ void gemm_mainloop(const GemmOperands& g, int row0, i
 // steps of loads in flight; completion is tracked with explicit vmcnt waits and
 // one s_barrier per K step.
 // ---------------------------------------------------------------------------
-#ifndef FGRPO_DMA_AUX
 #define FGRPO_DMA_AUX 0   // cache-policy bits of the direct-to-LDS loads
-#endif
 #define FGRPO_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define FGRPO_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
@@ -231,16 +224,10 @@ template <class C>
 __device__ __forceinline__ int lds_swizzle(int row) {
   // Chosen with SQ_LDS_BANK_CONFLICT on the real kernels (fragment read: lane l -> row l%32,
   // chunk l/32 + 2*kk; the LDS serves 16 consecutive lanes per pass over 64 banks).
-#ifndef FGRPO_SWZ4
-#define FGRPO_SWZ4(row) (((row) >> 2) & 3)
-#endif
   if constexpr (C::CPR == 4)
-    return FGRPO_SWZ4(row);                       // 64-byte rows
+    return (row >> 2) & 3;                       // 64-byte rows
   else
-#ifndef FGRPO_SWZ8
-#define FGRPO_SWZ8(row) (((row) + (((row) >> 3) & 1)) & 7)
-#endif
-    return FGRPO_SWZ8(row);                       // 128-byte rows
+    return (row + ((row >> 3) & 1)) & 7;                       // 128-byte rows
 }
 
 __device__ __forceinline__ void wg_barrier() {
@@ -290,9 +277,7 @@ __device__ __forceinline__ bf16x8_t lds_read_b128_asm(uint32_t addr) {
 //   load_a/load_b(stage_ptr, block, kk): one MFMA operand from LDS.
 // On entry the loads of step 0 have been issued into buffer 0 (if nk_total > 0).
 // ---------------------------------------------------------------------------
-#ifndef FGRPO_EB_PHASES
-#define FGRPO_EB_PHASES 2
-#endif
+constexpr int kLoadPhases = 2;   // sub-steps over which one K step's loads are issued (1 and 3 measured slower)
 // compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N-1>{})
 template <class F, int... Is>
 __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
@@ -309,12 +294,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 // The fragments of the following sub-step are requested between the MFMA row groups of the current one, in the
 // order a0, b0 .. b(TN-1), a1 .. a(TM-1) (row group 0 needs a0 and every b), so that the LDS sees a steady
 // trickle of reads next to the direct-to-LDS stream instead of a burst per sub-step.
-#ifndef FGRPO_EB_FINE
-#define FGRPO_EB_FINE 1
-#endif
-#ifndef FGRPO_EB_STAGGER
-#define FGRPO_EB_STAGGER 0
-#endif
+constexpr bool kTrickleReads = true;   // false: all fragments of a sub-step requested in one burst (measured equal or slower)
 template <int N>
 __device__ __forceinline__ void wait_lgkm() {
   static_assert(N >= 0, "wait count");
@@ -326,11 +306,11 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
                                                        IssueOne&& issue_one, LoadA&& load_a, LoadB&& load_b) {
   constexpr int KK = C::BK / 16;
   constexpr int TM = C::TM, TN = C::TN, NR = TM + TN;
-  static_assert(KK % 2 == 0 && KK >= FGRPO_EB_PHASES + 1, "sub-steps per K step");
-  constexpr int NSLOT = FGRPO_EB_PHASES * TM;         // MFMA groups over which one step's loads are spread
+  static_assert(KK % 2 == 0 && KK >= kLoadPhases + 1, "sub-steps per K step");
+  constexpr int NSLOT = kLoadPhases * TM;         // MFMA groups over which one step's loads are spread
   // fragment order and bookkeeping (all compile time)
   struct Ord {
-    static constexpr int cum(int i) { return FGRPO_EB_FINE ? (i * NR + TM - 1) / TM : (i > 0 ? NR : 0); }  // entries requested before row group i ends.. starts
+    static constexpr int cum(int i) { return kTrickleReads ? (i * NR + TM - 1) / TM : (i > 0 ? NR : 0); }  // entries requested before row group i ends.. starts
     static constexpr int instrs(int n) {              // LDS instructions of the first n entries
       int c = 0;
       for (int e = 0; e < n; ++e) c += (e == 0 || e > TN) ? RA : RB;
@@ -342,7 +322,6 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
       return instrs(NR) - instrs(need(i) + 1) + (issuing ? instrs(cum(i)) : 0);
     }
   };
-  const int team = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) & 1;   // wavefronts w and w+4 share a SIMD
   FGRPO_WAIT_VMCNT(0);
   wg_barrier();                                       // step 0 is in buffer 0
   int steps_issued = nk_total > 0 ? 1 : 0;
@@ -391,15 +370,15 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
       }
       // phase of the load spreading this sub-step belongs to: 0 = last sub-step, then 1, 2 .. from the top
       constexpr int phase = last ? 0 : kk + 1;
-      const bool loads_here = STEADY || (active && phase < FGRPO_EB_PHASES && (phase > 0 || next));
-      if constexpr (!FGRPO_EB_FINE) {                 // burst: every fragment of the next sub-step up front
+      const bool loads_here = STEADY || (active && phase < kLoadPhases && (phase > 0 || next));
+      if constexpr (!kTrickleReads) {                 // burst: every fragment of the next sub-step up front
         if (issuing) static_for<NR>([&](auto e) { request(src, e, std::integral_constant<int, kn>{}, std::integral_constant<int, nbuf>{}); });
         if (issuing) wait_lgkm<Ord::instrs(NR)>(); else wait_lgkm<0>();
       }
       __builtin_amdgcn_sched_barrier(0);
       static_for<TM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        if constexpr (FGRPO_EB_FINE) {
+        if constexpr (kTrickleReads) {
           if constexpr (!last) {
             wait_lgkm<Ord::allowed(i, true)>();
           } else {
@@ -409,7 +388,7 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
-        if constexpr (FGRPO_EB_FINE) {
+        if constexpr (kTrickleReads) {
           if (issuing) {
             static_for<Ord::cum(i + 1) - Ord::cum(i)>([&](auto d) {
               request(src, std::integral_constant<int, Ord::cum(i) + decltype(d)::value>{}, std::integral_constant<int, kn>{},
@@ -417,22 +396,11 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
             });
           }
         }
-        if constexpr (phase < FGRPO_EB_PHASES) {
-          if constexpr (FGRPO_EB_STAGGER && C::NW == 8 && TM % 2 == 0 && LPT % (2 * FGRPO_EB_PHASES) == 0) {
-            // The two wavefronts of a SIMD (w and w+4) issue their loads under different MFMA row groups,
-            // so that while one sits in the vector-memory issue queue the other still feeds the matrix pipe.
-            constexpr int HALF = TM / 2, PER_PHASE = LPT / FGRPO_EB_PHASES, PER_GROUP = PER_PHASE / HALF;
-            if (loads_here && (i / HALF) == team) {
-              static_for<PER_GROUP>([&](auto d) {
-                issue_one(tgt, std::integral_constant<int, phase * PER_PHASE + (i % HALF) * PER_GROUP + decltype(d)::value>{});
-              });
-            }
-          } else {
-            if (loads_here) {
-              static_for<LPT>([&](auto q) {
-                if constexpr (decltype(q)::value * NSLOT / LPT == phase * TM + i) issue_one(tgt, decltype(q)::value);
-              });
-            }
+        if constexpr (phase < kLoadPhases) {
+          if (loads_here) {
+            static_for<LPT>([&](auto q) {
+              if constexpr (decltype(q)::value * NSLOT / LPT == phase * TM + i) issue_one(tgt, decltype(q)::value);
+            });
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -523,9 +491,6 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   };
   // One load of the current issue step (idx < PA: operand A, else B); the last one advances the cursor.
   auto issue_one = [&](int stage, int idx) {
-#ifdef FGRPO_EXP_NO_GLOBAL
-    return;
-#endif
     char* base = smem + stage * C::STAGE;
     if (idx < C::PA)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsa, FGRPO_LDS_PTR(base + dst_a + idx * C::NW * C::RPI * C::ROWB), 16,
@@ -545,22 +510,13 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   int issued = 0;
   for (; issued < D && issued < nk_total; ++issued) issue(issued);
 
-#ifndef FGRPO_EARLY_BARRIER
-#define FGRPO_EARLY_BARRIER 1
-#endif
-  if constexpr (C::NSTAGE == 2 && FGRPO_EARLY_BARRIER && (C::BK / 16) % 2 == 0) {
+  if constexpr (C::NSTAGE == 2 && (C::BK / 16) % 2 == 0) {
     early_barrier_pipeline<C, LPT, 1, 1>(
         nk_total, smem, acc, issue_one,
         [&](const char* st, auto i, auto kk) {
-#ifdef FGRPO_EXP_NO_LDSREAD
-          return FGRPO_LDFRAG(st);
-#endif
           return lds_read_b128_asm<decltype(i)::value * 32 * C::ROWB>(lds_addr(st) + fr_a + fr_c[decltype(kk)::value]);
         },
         [&](const char* st, auto j, auto kk) {
-#ifdef FGRPO_EXP_NO_LDSREAD
-          return FGRPO_LDFRAG(st);
-#endif
           return lds_read_b128_asm<decltype(j)::value * 32 * C::ROWB>(lds_addr(st) + fr_b + fr_c[decltype(kk)::value]);
         });
     return;
@@ -570,11 +526,8 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   // every wavefront busy issuing addresses, about 40 cycles per load, before its first MFMA).
   // With three or more LDS buffers they are spread over the whole step; with two buffers over the
   // first half, so that the last one still has half a step to land.
-#ifndef FGRPO_SPREAD_DIV2
-#define FGRPO_SPREAD_DIV2 2
-#endif
   constexpr int kGroups = (C::BK / 16) * C::TM;                                  // MFMA groups (TN MFMAs each) per step
-  constexpr int kSpreadG = (C::NSTAGE >= 3) ? kGroups : (kGroups / FGRPO_SPREAD_DIV2 > 0 ? kGroups / FGRPO_SPREAD_DIV2 : 1);
+  constexpr int kSpreadG = (C::NSTAGE >= 3) ? kGroups : (kGroups / 2 > 0 ? kGroups / 2 : 1);
   constexpr int kPer = (LPT + kSpreadG - 1) / kSpreadG;                          // loads after each group
   constexpr bool kSpread = true;
   constexpr int KK = C::BK / 16;
@@ -694,7 +647,6 @@ __device__ __forceinline__ void gemm_mainloop_la(const GemmOperands& g, int row0
   const char* Ai = segA[0];
   const char* Bi = segB[0];
   auto issue_one = [&](int stage, int idx) {
-#ifndef FGRPO_EXP_NO_GLOBAL
     char* base = smem + stage * C::STAGE;
     if (idx < C::PA)
       __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Ai + aoff[idx]),
@@ -703,7 +655,6 @@ __device__ __forceinline__ void gemm_mainloop_la(const GemmOperands& g, int row0
       __builtin_amdgcn_global_load_lds(FGRPO_GLOBAL_PTR(Bi + boff[idx - C::PA]),
                                        FGRPO_LDS_PTR(base + dst_b + (idx - C::PA) * C::NW * C::RPI * C::ROWB), 16, 0,
                                        FGRPO_DMA_AUX);
-#endif
     if (idx == LPT - 1) {
       Ai += C::BK * 2;
       Bi += C::BK * 2;
@@ -880,9 +831,6 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   const long long a_blk_bytes = (!AKM) ? g.a_blk * 2 : 0;
   int ablk_left = 256 / C::BK;
   auto issue_one = [&](int stage, int idx) {
-#ifdef FGRPO_EXP_NO_GLOBAL
-    return;
-#endif
     char* base = smem + stage * C::STAGE;
     if (idx < C::PA)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsa, FGRPO_LDS_PTR(base + dst_w + idx * C::NW * 1024), 16, (int)aoff[idx],
@@ -942,9 +890,6 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
 
   auto load_a = [&](const char* st, auto ic, auto kc) -> bf16x8_t {
     constexpr int i = decltype(ic)::value, kk = decltype(kc)::value;
-#ifdef FGRPO_EXP_NO_LDSREAD
-    return FGRPO_LDFRAG(st);
-#endif
     if constexpr (AKM)
       return lds_read_tr_pair<(16 * kk) * KROWB, (16 * kk + 4) * KROWB>(lds_addr(st) + fka[i]);
     else
@@ -952,9 +897,6 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   };
   auto load_b = [&](const char* st, auto jc, auto kc) -> bf16x8_t {
     constexpr int j = decltype(jc)::value, kk = decltype(kc)::value;
-#ifdef FGRPO_EXP_NO_LDSREAD
-    return FGRPO_LDFRAG(st);
-#endif
     if constexpr (BKM)
       return lds_read_tr_pair<(16 * kk) * KROWB, (16 * kk + 4) * KROWB>(lds_addr(st) + fkb[j]);
     else
