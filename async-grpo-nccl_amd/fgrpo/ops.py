@@ -414,14 +414,59 @@ def gemm_kmajor(A: torch.Tensor, B: torch.Tensor, a_kmajor: bool, b_kmajor: bool
 
 
 # --------------------------------------------------------------------------- autograd
+# Rows whose shifted label is -100 take no part in the objective: their logprob and entropy are 0 by definition and
+# they receive no gradient.  With ``compact`` the projection runs on the other rows only (one host sync to learn how
+# many there are), which pays off when prompts make up a sizeable part of the packed batch.
+COMPACT_MIN_TOKENS = 2048
+COMPACT_MAX_VALID_FRACTION = 0.9
+
+
+def _valid_rows(labels_shifted: torch.Tensor, compact: bool):
+    T = labels_shifted.numel()
+    if not compact or T < COMPACT_MIN_TOKENS:
+        return None
+    mask = labels_shifted.reshape(-1) != -100
+    n = int(mask.sum())
+    if n == 0 or n > COMPACT_MAX_VALID_FRACTION * T:
+        return None
+    return mask.nonzero(as_tuple=False).squeeze(1)
+
+
+def _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx):
+    """Forward on the rows ``idx`` (or on all rows when idx is None); outputs scattered back into [T] vectors."""
+    if idx is None:
+        lp, ent, lse = lmhead_logprob_fwd(hidden, weight, bias, labels_shifted, temperature)
+        return lp, ent, lse, hidden, labels_shifted
+    T = hidden.shape[0]
+    h_c = hidden.index_select(0, idx)
+    y_c = labels_shifted.reshape(-1).index_select(0, idx)
+    lp_c, ent_c, lse_c = lmhead_logprob_fwd(h_c, weight, bias, y_c, temperature)
+    lp = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, lp_c)
+    ent = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, ent_c)
+    return lp, ent, lse_c, h_c, y_c
+
+
+def _bwd_rows(h_used, weight, bias, y_used, lse, g_full, gout, temperature, need, panel_hint, idx, hidden_shape):
+    g_used = g_full if idx is None else g_full.reshape(-1).index_select(0, idx)
+    dH, dW, db = lmhead_bwd(h_used, weight, bias, y_used, lse, g_used, gout, temperature, need[0], need[1], need[2],
+                            panel_hint)
+    if idx is not None and dH is not None:
+        dH = torch.zeros(hidden_shape, dtype=dH.dtype, device=dH.device).index_copy_(0, idx, dH)
+    return dH, dW, db
+
+
 class _LMHeadLogprob(torch.autograd.Function):
     """(hidden, weight, bias, labels_shifted) -> (lp, entropy); entropy carries no gradient."""
 
     @staticmethod
-    def forward(ctx, hidden, weight, bias, labels_shifted, temperature, panel_hint):
-        lp, ent, lse = lmhead_logprob_fwd(hidden, weight, bias, labels_shifted, temperature)
-        ctx.save_for_backward(hidden, weight, bias if bias is not None else hidden.new_empty(0), labels_shifted, lse)
+    def forward(ctx, hidden, weight, bias, labels_shifted, temperature, panel_hint, compact):
+        idx = _valid_rows(labels_shifted, compact)
+        lp, ent, lse, h_used, y_used = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx)
+        ctx.save_for_backward(h_used, weight, bias if bias is not None else hidden.new_empty(0), y_used, lse,
+                              idx if idx is not None else hidden.new_empty(0))
         ctx.has_bias = bias is not None
+        ctx.compacted = idx is not None
+        ctx.hidden_shape = tuple(hidden.shape)
         ctx.temperature = temperature
         ctx.panel_hint = panel_hint
         ctx.mark_non_differentiable(ent)
@@ -429,12 +474,12 @@ class _LMHeadLogprob(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_lp, _g_ent):
-        hidden, weight, bias, labels_shifted, lse = ctx.saved_tensors
+        h_used, weight, bias, y_used, lse, idx = ctx.saved_tensors
         bias = bias if ctx.has_bias else None
-        dH, dW, db = lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g_lp, None, ctx.temperature,
-                                ctx.needs_input_grad[0], ctx.needs_input_grad[1],
-                                ctx.has_bias and ctx.needs_input_grad[2], ctx.panel_hint)
-        return dH, dW, db, None, None, None
+        need = (ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.has_bias and ctx.needs_input_grad[2])
+        dH, dW, db = _bwd_rows(h_used, weight, bias, y_used, lse, g_lp, None, ctx.temperature, need, ctx.panel_hint,
+                               idx if ctx.compacted else None, ctx.hidden_shape)
+        return dH, dW, db, None, None, None, None
 
 
 class _FusedGRPOLoss(torch.autograd.Function):
@@ -443,14 +488,17 @@ class _FusedGRPOLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens, temperature,
-                clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode, denom_override, panel_hint):
-        lp, ent, lse = lmhead_logprob_fwd(hidden, weight, bias, labels_shifted, temperature)
+                clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode, denom_override, panel_hint, compact):
+        idx = _valid_rows(labels_shifted, compact)
+        lp, ent, lse, h_used, y_used = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx)
         loss, g, lr, c1, l1, l2, scal = grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
                                                       clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
                                                       denom_override)
-        ctx.save_for_backward(hidden, weight, bias if bias is not None else hidden.new_empty(0), labels_shifted,
-                              lse, g)
+        ctx.save_for_backward(h_used, weight, bias if bias is not None else hidden.new_empty(0), y_used, lse, g,
+                              idx if idx is not None else hidden.new_empty(0))
         ctx.has_bias = bias is not None
+        ctx.compacted = idx is not None
+        ctx.hidden_shape = tuple(hidden.shape)
         ctx.temperature = temperature
         ctx.panel_hint = panel_hint
         ctx.mark_non_differentiable(ent, lr, c1, l1, l2, lp)
@@ -458,12 +506,12 @@ class _FusedGRPOLoss(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
-        hidden, weight, bias, labels_shifted, lse, g = ctx.saved_tensors
+        h_used, weight, bias, y_used, lse, g, idx = ctx.saved_tensors
         bias = bias if ctx.has_bias else None
-        dH, dW, db = lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, g_loss, ctx.temperature,
-                                ctx.needs_input_grad[0], ctx.needs_input_grad[1],
-                                ctx.has_bias and ctx.needs_input_grad[2], ctx.panel_hint)
-        return (dH, dW, db) + (None,) * 13
+        need = (ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.has_bias and ctx.needs_input_grad[2])
+        dH, dW, db = _bwd_rows(h_used, weight, bias, y_used, lse, g, g_loss, ctx.temperature, need, ctx.panel_hint,
+                               idx if ctx.compacted else None, ctx.hidden_shape)
+        return (dH, dW, db) + (None,) * 14
 
 
 class _GRPOLossFromLogprobs(torch.autograd.Function):
@@ -496,14 +544,15 @@ def grpo_loss_from_logprobs(lp, labels_shifted, old_lp, adv, ref_lp=None, cu_seq
                                        float(denom_override))
 
 
-def lmhead_logprob(hidden, weight, bias, labels_shifted, temperature=1.0, panel_hint=0) -> Tuple[torch.Tensor, torch.Tensor]:
-    return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint))
+def lmhead_logprob(hidden, weight, bias, labels_shifted, temperature=1.0, panel_hint=0,
+                   compact=False) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint), bool(compact))
 
 
 def fused_grpo_loss(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp=None, cu_seqlens=None,
                     temperature=1.0, clip_low=0.2, clip_high=0.4, clip_ratio_c=1e32, kl_beta=0.0,
-                    loss_agg_mode="token_mean", denom_override=0.0, panel_hint=0):
+                    loss_agg_mode="token_mean", denom_override=0.0, panel_hint=0, compact=False):
     """(loss, entropy, log_ratio, clip1, unclipped, clipped, lp); only loss carries a gradient."""
     return _FusedGRPOLoss.apply(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens,
                                 float(temperature), float(clip_low), float(clip_high), float(clip_ratio_c),
-                                float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint))
+                                float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint), bool(compact))

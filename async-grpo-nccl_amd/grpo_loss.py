@@ -23,7 +23,9 @@ reference rounds logits to bf16 first, grpo_loss.py:245/:310); a foreign
 Extensions reachable through the ``**unused_kwargs`` hole of the reference
 signature: ``ref_logprobs``/``kl_beta`` (k3 KL penalty), ``loss_agg_mode``
 (``"token_mean"`` = reference, ``"sample_mean"``), ``cu_seqlens``,
-``num_samples_total``.
+``num_samples_total``, ``compact_masked_tokens`` (project only the rows whose
+shifted label is not -100: same results, one host sync, worth it when prompts
+are a sizeable part of the packed batch).
 """
 from __future__ import annotations
 
@@ -207,7 +209,8 @@ def fused_log_probs_and_entropy_fn(
         return _materialised_log_probs_and_entropy(w, b, hidden_states, ops.shift_labels(labels), temperature,
                                                    per_token_fn, None)
     shifted = ops.shift_labels(labels).reshape(-1)
-    lp, ent = ops.lmhead_logprob(hs, w, b, shifted, temperature)
+    lp, ent = ops.lmhead_logprob(hs, w, b, shifted, temperature,
+                                 compact=bool(unused_kwargs.get("compact_masked_tokens", False)))
     return lp, ent
 
 
@@ -247,6 +250,7 @@ def grpo_loss_and_entropy_ce_fn(
     loss_agg_mode = unused_kwargs.get("loss_agg_mode", "token_mean")
     cu_seqlens = unused_kwargs.get("cu_seqlens", None)
     num_samples_total = unused_kwargs.get("num_samples_total", None)
+    compact = bool(unused_kwargs.get("compact_masked_tokens", False))
 
     shifted = ops.shift_labels(labels).reshape(-1)
     w, b, hs = _prep(lm_head_weights, lm_head_bias, hidden_states)
@@ -267,7 +271,7 @@ def grpo_loss_and_entropy_ce_fn(
         advantages.reshape(-1),
         None if ref_logprobs is None else ref_logprobs.reshape(-1),
         cu_seqlens, temperature, clip_low, clip_high, clip_ratio_c, kl_beta,
-        loss_agg_mode, denom, hint)
+        loss_agg_mode, denom, hint, compact)
     return loss, ent, lr, c1, l1, l2
 
 
@@ -314,7 +318,8 @@ def make_grpo_forward(model, temperature: float = 1.0, mode: str = 'training', u
         output_hidden_states = output_hidden_states if output_hidden_states is not None else cfg.output_hidden_states
         return_dict = return_dict if return_dict is not None else cfg.use_return_dict
         # objective extensions travel in kwargs but are not for the transformer body
-        extra = {k: kwargs.pop(k) for k in ("ref_logprobs", "kl_beta", "loss_agg_mode", "cu_seqlens", "num_samples_total")
+        extra = {k: kwargs.pop(k) for k in ("ref_logprobs", "kl_beta", "loss_agg_mode", "cu_seqlens", "num_samples_total",
+                                            "compact_masked_tokens")
                  if k in kwargs}
         body_out = model.model(
             input_ids=input_ids,
@@ -365,6 +370,7 @@ def make_grpo_forward(model, temperature: float = 1.0, mode: str = 'training', u
                 hidden_states=hidden_states,
                 labels=labels,
                 temperature=temperature,
+                **{k: v for k, v in extra.items() if k == "compact_masked_tokens"},
             )
             return LogProbsOutput(loss=out[0], entropy=out[1])
         else:
@@ -399,6 +405,11 @@ def compute_dual_clip_grpo_loss(
     advantages = minibatch["advantages"]
     labels = minibatch["labels"]
 
+    # Shapes alone (no sync) tell when prompts are a sizeable part of the batch: output_indices lists exactly the
+    # positions whose shifted label is valid (sample_processing_utils.py:29-67).  The LM head then skips the rest.
+    extra = {}
+    if 0 < int(output_indices.numel()) < ops.COMPACT_MAX_VALID_FRACTION * int(labels.numel()):
+        extra["compact_masked_tokens"] = True
     grpo_output = policy_model(
         input_ids=batch_ids,
         attention_mask=minibatch.get("attention_mask", None),
@@ -411,6 +422,7 @@ def compute_dual_clip_grpo_loss(
         clip_high=clip_high,
         clip_ratio_c=clip_ratio_c,
         compute_entropy=compute_entropy,
+        **extra,
     )
 
     old_entropy = minibatch.get("reference_output_entropies", None)

@@ -224,6 +224,47 @@ def test_backward_operand_layout_modes_agree(dev, kmajor):
     check(want, got, o, g, f32=False)
 
 
+def test_compaction_of_masked_tokens_changes_nothing(dev):
+    """Packed batch with prompts (40% of the positions carry label -100): projecting only the valid rows gives the
+    same loss, logprobs, entropy and gradients as projecting every row, and both match the oracle."""
+    import grpo_loss as G
+    from fgrpo.synthetic import make_workload
+    w = make_workload("cfg1", seed=9, overrides=dict(H=256, V=5000, tokens=3000, len_lo=8, len_hi=300, h_scale=1.0))
+    p = w.params
+    labels = w.labels.clone()
+    drop = torch.rand(labels.shape, generator=torch.Generator().manual_seed(4)) < 0.4
+    labels[drop] = -100
+    T = w.T
+    adv = torch.randn(T, generator=torch.Generator().manual_seed(5))
+    hs_c, W_c = oracle_inputs(w)
+    lp0, _ = O.fused_log_probs_and_entropy(W_c, None, hs_c, labels, 1.0)
+    old = lp0 + w.noise_old.cpu()
+    hs_o = hs_c.clone().requires_grad_(True)
+    W_o = W_c.clone().requires_grad_(True)
+    want = O.grpo_loss_and_entropy(W_o, None, hs_o, labels, 1.0, old, adv, p["clip_low"], p["clip_high"], p["clip_ratio_c"])
+    want[0].backward()
+    res = []
+    for compact in (False, True):
+        hs = w.hidden.to(dev).clone().requires_grad_(True)
+        W = w.weight.to(dev).clone().requires_grad_(True)
+        out = G.grpo_loss_and_entropy_ce_fn(W, None, hs, labels.to(dev), 1.0, old.to(dev), adv.to(dev), p["clip_low"],
+                                            p["clip_high"], p["clip_ratio_c"], compact_masked_tokens=compact)
+        out[0].backward()
+        check(want, out, (hs_o, W_o, None), (hs, W, None), f32=False)
+        res.append((out, hs.grad, W.grad))
+    (a, dha, dwa), (b, dhb, dwb) = res
+    assert torch.equal(a[2], b[2]) and torch.equal(a[1], b[1])          # per-token results do not depend on the other rows
+    assert abs(a[0].item() - b[0].item()) <= 1e-6 * abs(a[0].item()) + 1e-9
+    assert torch.equal(dha, dhb)
+    assert cos(dwa, dwb) >= 0.99999
+    masked = ops_shift(labels) == -100
+    assert (dhb[0][masked[0].to(dev)] == 0).all()
+
+
+def ops_shift(labels):
+    return O.shift_labels(labels)
+
+
 # ------------------------------------------------------------------ edge cases of the reference
 def test_all_masked_dummy_batch(dev):
     import grpo_loss as G
