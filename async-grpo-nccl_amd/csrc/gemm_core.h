@@ -1,15 +1,17 @@
-// bf16 "NT" GEMM main loop for gfx950 (CDNA4): D[m,n] = sum_k A[m,k] * B[n,k].
+// bf16 GEMM main loops for gfx950 (CDNA4): D[m,n] = sum_k A[m,k] * B[n,k] on v_mfma_f32_32x32x16_bf16
+// (lane l supplies row l % 32 and the eight k values 8*(l/32) .. 8*(l/32)+7 of each operand).
 //
-// Both operands are row-major with the contraction index contiguous, which is
-// the layout v_mfma_f32_32x32x16_bf16 wants from a 16-byte LDS read: lane l
-// supplies row (l % 32) and the eight k values 8*(l/32) .. 8*(l/32)+7.
-//
-// Work-group tile BM x BN, K step BK, WM x WN wavefronts (64 lanes each), every
-// wavefront owning a (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA blocks kept
-// in fp32 accumulators.  Global -> register -> LDS staging with NSTAGE LDS
-// buffers: the loads of K step kt+1 are in flight while step kt is multiplied.
-// LDS rows are padded by 16 bytes so that the 16-byte fragment reads of 8 or 16
-// consecutive rows fall into distinct bank groups.
+// Work-group tile BM x BN, K step BK, WM x WN wavefronts (64 lanes each), every wavefront owning a
+// (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA blocks kept in fp32 accumulators.  Four loops, chosen by the
+// tile configuration (run_mainloop) or by the caller:
+//   gemm_mainloop      global -> registers -> LDS, padded LDS rows, two buffers (small tiles, fp32 split path);
+//   gemm_mainloop_dma  global -> LDS directly (buffer_load ... lds), swizzled LDS rows; with two buffers it runs
+//                      the early-barrier schedule below (the default for large problems), with three a plain
+//                      prefetch loop;
+//   gemm_mainloop_la   direct-to-LDS with four or more BK=32 buffers and one K step of fragment look-ahead;
+//   gemm_mainloop_km   operands whose contraction index is the ROW index as stored (read through
+//                      ds_read_b64_tr_b16), early-barrier schedule.
+// Operands are K-contiguous (X[m][k]) unless a loop says otherwise.
 //
 // A contraction may be the sum of up to three (A_s, B_s, K_s) segments sharing
 // the leading dimensions; the fp32 path uses that for the bf16 hi/lo split

@@ -1,6 +1,6 @@
-// LM-head kernels built on the NT GEMM main loop: vocabulary statistics
+// LM-head kernels built on the GEMM main loops: vocabulary statistics
 // (forward), dLogits panels (backward recompute) and plain GEMM with a store
-// epilogue (dHidden, dW).  In the two LM-head kernels the MFMA "M" index is the
+// epilogue (dHidden with K-contiguous operands, dW with contraction-major ones).  In the two LM-head kernels the MFMA "M" index is the
 // vocabulary and "N" is the token, so one lane owns a single token per 32x32
 // block and 16 vocabulary entries of it: the soft-max statistics reduce inside
 // the lane and need one cross-lane step (lanes l and l^32) at the very end.
@@ -215,11 +215,13 @@ __global__ void lmhead_fwd_combine_kernel(const CombineParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// Backward recompute: dLogits for one vocabulary panel, written as bf16 in
-// both [token][vocab] and [vocab][token] order (the contraction index of the
-// GEMM that consumes each copy is its contiguous index).
+// Backward recompute: dLogits for one vocabulary panel, written as bf16
+//   * in-place mode (tv_blk != 0, vt_hi == null): once, as 256-column blocks [v/256][token][256], which both
+//     gradient GEMMs read (dHidden K-contiguous, dW contraction-major);
+//   * otherwise: in [token][vocab] and in [vocab][token] order (the contraction index of the GEMM that consumes
+//     each copy is its contiguous index).
 //   dS[t, v] = c_t * (1[v == y_t] - exp(x_tv - lse_t)),  c_t = g_t * gout / temperature
-// Every element of both padded panel buffers is written (zeros outside T x V).
+// Every element of the padded panel buffers is written (zeros outside T x V).
 // ---------------------------------------------------------------------------
 struct DsParams {
   GemmOperands g;            // A = W [V x K] (M = V), B = hidden [T x K] (N = T)
