@@ -416,9 +416,17 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
   wg_barrier();                                       // LDS may be reused by the caller
 }
 
+// MODE 0: the whole contraction.  MODE 2: only issue the loads of K step 0 into buffer 0 and return (the caller
+// does something else, e.g. the epilogue of the previous tile, while they fly); MODE 1: the contraction, given that
+// a MODE 2 call for the same tile has been made since the last MODE 0/1 call returned.  Modes 1 and 2 exist for
+// the two-buffer schedule only (kSplitPrologue).
 template <class C>
+constexpr bool kSplitPrologue = C::DMA && C::NSTAGE == 2 && (C::BK / 16) % 2 == 0;
+
+template <class C, int MODE = 0>
 __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row0, int col0, char* smem,
                                                   f32x16_t (&acc)[C::TM][C::TN]) {
+  static_assert(MODE == 0 || kSplitPrologue<C>, "split prologue needs the two-buffer schedule");
   constexpr int D = C::NSTAGE - 1;              // K steps of loads in flight
   constexpr int LPT = C::PA + C::PB;            // loads per thread per K step
   static_assert(D >= 1 && D <= 4 && LPT * (D - 1) < 64, "pipeline depth");
@@ -507,10 +515,18 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
     for (int i = 0; i < LPT; ++i) issue_one(stage, i);
   };
 
-  // loads issued before this call (by the caller's epilogue) must not be mistaken for ours
-  FGRPO_WAIT_VMCNT(0);
   int issued = 0;
-  for (; issued < D && issued < nk_total; ++issued) issue(issued);
+  if constexpr (MODE == 1) {                    // step 0 is already on its way into buffer 0
+    if (nk_total > 0) {
+      advance();
+      issued = 1;
+    }
+  } else {
+    // loads issued before this call (by the caller's epilogue) must not be mistaken for ours
+    FGRPO_WAIT_VMCNT(0);
+    for (; issued < D && issued < nk_total; ++issued) issue(issued);
+    if constexpr (MODE == 2) return;
+  }
 
   if constexpr (C::NSTAGE == 2 && (C::BK / 16) % 2 == 0) {
     early_barrier_pipeline<C, LPT, 1, 1>(

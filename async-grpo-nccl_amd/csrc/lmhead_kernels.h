@@ -80,11 +80,24 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
     y[j] = (lab >= 0 && lab < V) ? (int)lab : -1;
   }
 
+  // With the two-buffer direct-to-LDS loop the first K slice of the NEXT vocabulary tile is requested before this
+  // tile's statistics are folded in, so its latency hides under that arithmetic.
+  if constexpr (kSplitPrologue<C>) {
+    if (vt_begin < vt_end) {
+      f32x16_t none[C::TM][C::TN];
+      gemm_mainloop_dma<C, 2>(p.g, vt_begin * C::BM, col0, smem, none);
+    }
+  }
   for (int vt = vt_begin; vt < vt_end; ++vt) {
     const int row0 = vt * C::BM;
     f32x16_t acc[C::TM][C::TN];
     zero_acc<C>(acc);
-    run_mainloop<C>(p.g, row0, col0, smem, acc);
+    if constexpr (kSplitPrologue<C>) {
+      gemm_mainloop_dma<C, 1>(p.g, row0, col0, smem, acc);
+      if (vt + 1 < vt_end) gemm_mainloop_dma<C, 2>(p.g, row0 + C::BM, col0, smem, acc);
+    } else {
+      run_mainloop<C>(p.g, row0, col0, smem, acc);
+    }
 
     // Statistics are kept in units of the raw product (before the temperature): inv_temp > 0 commutes with
     // the maximum, enters the exponent through one fused multiply-add, and scales m and sum(e*x) once at the end.
