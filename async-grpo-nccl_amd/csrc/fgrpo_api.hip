@@ -73,7 +73,6 @@ struct Tuning {
   int gemm_variant = 8;
   int fwd_nsplit = 0;   // 0 = heuristic
   int fwd_group_t = 8;
-  int ds_group_v = 8;
   int gemm_group_m = 4;
   int panel_cols = 32768;  // default vocabulary panel width of the backward
   int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
@@ -87,7 +86,6 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "gemm_variant")) return &g_tune.gemm_variant;
   if (!strcmp(key, "fwd_nsplit")) return &g_tune.fwd_nsplit;
   if (!strcmp(key, "fwd_group_t")) return &g_tune.fwd_group_t;
-  if (!strcmp(key, "ds_group_v")) return &g_tune.ds_group_v;
   if (!strcmp(key, "gemm_group_m")) return &g_tune.gemm_group_m;
   if (!strcmp(key, "panel_cols")) return &g_tune.panel_cols;
   if (!strcmp(key, "small_variant")) return &g_tune.small_variant;
@@ -280,11 +278,11 @@ int launch_fwd(const FwdParams& p, hipStream_t st) {
 }
 template <class C>
 int launch_ds(const DsParams& p, hipStream_t st) {
-  return launch_tile_kernel<C>(lmhead_ds_kernel<C, false>, p, p.tiles_t * p.tiles_v, st);
+  return launch_tile_kernel<C>(lmhead_ds_kernel<C, false>, p, p.tiles_t * p.nsplit, st);
 }
 // fp32 inputs: dS is written as bf16 hi + lo halves; only the small tile carries that epilogue
 int launch_ds_split(const DsParams& p, hipStream_t st) {
-  return launch_tile_kernel<Cfg4>(lmhead_ds_kernel<Cfg4, true>, p, p.tiles_t * p.tiles_v, st);
+  return launch_tile_kernel<Cfg4>(lmhead_ds_kernel<Cfg4, true>, p, p.tiles_t * p.nsplit, st);
 }
 template <class C>
 int launch_store(const StoreParams& p, hipStream_t st) {
@@ -544,7 +542,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
   d.gout = gout_dev;
   d.inv_temp = inv_temp;
   d.tiles_t = pl.tiles_t;
-  d.group_v = g_tune.ds_group_v > 0 ? g_tune.ds_group_v : 1;
+  d.group_t = g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1;
   d.tv_hi = pl.tv_hi;
   d.tv_lo = pl.tv_lo;
   d.vt_hi = pl.vt_hi;
@@ -561,6 +559,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
     const int rows = (V - v0) < pl.panel ? (V - v0) : pl.panel;
     d.v0 = v0;
     d.tiles_v = (rows + pl.bm - 1) / pl.bm;
+    d.nsplit = choose_nsplit(pl.tiles_t, d.tiles_v, num_cus() * kCfg[pl.variant].wgs_per_cu);
     const int kv = d.tiles_v * pl.bm;        // written panel width
     const int kt = pl.tiles_t * pl.bn;       // written token extent
     if (f32) {

@@ -245,7 +245,8 @@ struct DsParams {
   const float* gout;         // device scalar (upstream gradient) or null
   float inv_temp;
   int v0;                    // first vocabulary row of the panel (multiple of BM)
-  int tiles_v, tiles_t, group_v;
+  int tiles_v, tiles_t;      // tiles of the panel / of the tokens
+  int nsplit, group_t;       // work-group = (token tile, 1/nsplit of the panel's vocabulary tiles); raster group
   bf16_t* tv_hi;             // [tiles_t*BN][ld_tv]
   bf16_t* tv_lo;             // low half for the fp32 path, or null
   long long ld_tv;
@@ -263,131 +264,174 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
   const int wm = wave / C::WN, wn = wave % C::WN;
   const int V = p.g.M, T = p.g.N;
 
-  // grouped raster: group_v vocabulary tiles share the token sweep
+  // work-group -> (token tile, share of the panel's vocabulary tiles), rastered like the forward kernel: the
+  // per-token inputs are read once and the next tile's first K slice is requested under this tile's epilogue
   const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int per_group = p.group_v * p.tiles_t;
+  const int per_group = p.group_t * p.nsplit;
   const int grp = lid / per_group;
-  const int first_v = grp * p.group_v;
-  const int gsz = (p.tiles_v - first_v) < p.group_v ? (p.tiles_v - first_v) : p.group_v;
+  const int first_t = grp * p.group_t;
+  const int gsz = (p.tiles_t - first_t) < p.group_t ? (p.tiles_t - first_t) : p.group_t;
   const int w = lid - grp * per_group;
-  const int tv = first_v + w % gsz;
-  const int tt = w / gsz;
-  const int prow0 = tv * C::BM;        // row inside the panel
-  const int row0 = p.v0 + prow0;       // vocabulary row
+  const int tt = first_t + w % gsz;
+  const int split = w / gsz;
+  const int vt_begin = (int)((long long)split * p.tiles_v / p.nsplit);
+  const int vt_end = (int)((long long)(split + 1) * p.tiles_v / p.nsplit);
   const int col0 = tt * C::BN;
 
-  f32x16_t acc[C::TM][C::TN];
-  zero_acc<C>(acc);
-  run_mainloop<C>(p.g, row0, col0, smem, acc);
-
-  // vocabulary rows past V get a logit that exponentiates to exactly 0; the bias joins the raw product
-  if (p.bias != nullptr || row0 + C::BM > V) {
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int v = row0 + acc_row<C>(wm, i, r, lane);
-        const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
-#pragma unroll
-        for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
-      }
-  }
   const float go = (p.gout ? *p.gout : 1.f) * p.inv_temp;
   const float xs = p.inv_temp * kLog2e;
   const int lane_row0 = wm * C::WTM + 4 * (lane >> 5);   // first row of this lane inside the tile
+  float lse2[C::TN], cj[C::TN];
+  int ylab[C::TN];
 #pragma unroll
   for (int j = 0; j < C::TN; ++j) {
     const int n = col0 + acc_col<C>(wn, j, lane);
     const bool tok_ok = n < T;
-    const float lse2 = tok_ok ? p.lse[n] * kLog2e : -kNegBig;  // padding columns: probability exactly 0
+    lse2[j] = tok_ok ? p.lse[n] * kLog2e : -kNegBig;          // padding columns: probability exactly 0
     const long long lab = tok_ok ? p.labels[n] : -100;
-    const float c = (lab != -100) ? p.gtok[n] * go : 0.f;  // ignored tokens carry no gradient
-    const float nc = -c;
-    // target row relative to this lane's first row; out of range when not in this sub-tile
-    const int yrel = (lab >= 0 && lab < V) ? (int)(lab - row0) - lane_row0 : -1;
-    const long long tv_off = p.tv_blk ? (long long)tv * p.tv_blk + (long long)n * 256 + lane_row0
-                                      : (long long)n * p.ld_tv + prow0 + lane_row0;
-    bf16_t* tv_hi = p.tv_hi + tv_off;
-    bf16_t* tv_lo = SPLIT ? p.tv_lo + tv_off : nullptr;
-    bf16_t* vt_hi = p.vt_hi ? p.vt_hi + (long long)(prow0 + lane_row0) * p.ld_vt + n : nullptr;
-    bf16_t* vt_lo = (SPLIT && p.vt_lo) ? p.vt_lo + (long long)(prow0 + lane_row0) * p.ld_vt + n : nullptr;
-    // Few wavefronts hold a target row at all (64 tokens x WTM of V rows): the common case runs without
-    // the per-element comparison.
-    const bool any_y = __builtin_amdgcn_ballot_w64(yrel >= 0 && yrel < C::WTM) != 0;
-    // Column-blocked panel: a lane's 8 bytes (4 vocabulary entries of one token) would be a 64-line scatter per
-    // store instruction.  The wavefront instead parks 32 tokens x WTM entries in a private LDS patch and writes
-    // them out as 16-byte pieces, 16 lanes per token row: every store instruction fills whole 128-byte lines.
-    constexpr int EROW = C::WTM * 2 + 16;               // patch row: one token's WTM entries + 16 bytes of padding
-    constexpr int PPT = C::WTM * 2 / 16, TPP = 64 / PPT;  // 16-byte pieces per token, tokens per store instruction
-    char* patch = smem + wave * (32 * EROW);
-    static_assert(C::NW * 32 * EROW <= C::LDS_BYTES && 64 % PPT == 0 && 32 % TPP == 0, "epilogue patch");
-    auto emit = [&](auto with_y, auto via_lds) {
+    cj[j] = (lab != -100) ? p.gtok[n] * go : 0.f;             // ignored tokens carry no gradient
+    ylab[j] = (lab >= 0 && lab < V) ? (int)lab : (int)0xC0000000;   // far below any row: never matches
+  }
+
+  // Column-blocked panel: a lane's 8 bytes (4 vocabulary entries of one token) would be a 64-line scatter per
+  // store instruction.  The wavefront instead parks 32 tokens x WTM entries in a private LDS patch and writes
+  // them out as 16-byte pieces, PPT lanes per token row: every store instruction fills whole 128-byte lines.
+  // Patch rows are unpadded; the 8-byte slots of row n are XOR-swizzled with n, so that the 32 lanes of a write
+  // (one token each) hit 32 different slots.  The patch lives behind LDS buffer 0, which the prefetch of the next
+  // tile may already be filling.
+  constexpr int ROWP = C::WTM * 2;                       // patch row: one token's WTM entries
+  constexpr int NSLOT = ROWP / 8;                        // 8-byte slots per row
+  constexpr int PPT = ROWP / 16, TPP = 64 / PPT;         // 16-byte pieces per token, tokens per store instruction
+  constexpr int PATCH = C::NW * 32 * ROWP;
+  constexpr bool kPatchBehind = C::STAGE + PATCH <= C::LDS_BYTES;
+  constexpr bool kPrefetch = kSplitPrologue<C> && kPatchBehind;
+  static_assert(PATCH <= C::LDS_BYTES && 64 % PPT == 0 && 32 % TPP == 0 && (NSLOT & (NSLOT - 1)) == 0, "epilogue patch");
+  char* patch = smem + (kPatchBehind ? C::STAGE : 0) + wave * (32 * ROWP);
+  const bool through_lds = !SPLIT && p.tv_blk != 0;
+
+  if constexpr (kPrefetch) {
+    if (vt_begin < vt_end) {
+      f32x16_t none[C::TM][C::TN];
+      gemm_mainloop_dma<C, 2>(p.g, p.v0 + vt_begin * C::BM, col0, smem, none);
+    }
+  }
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    const int prow0 = vt * C::BM;        // row inside the panel
+    const int row0 = p.v0 + prow0;       // vocabulary row
+    f32x16_t acc[C::TM][C::TN];
+    zero_acc<C>(acc);
+    if constexpr (kPrefetch) {
+      gemm_mainloop_dma<C, 1>(p.g, row0, col0, smem, acc);
+      if (vt + 1 < vt_end) gemm_mainloop_dma<C, 2>(p.g, row0 + C::BM, col0, smem, acc);
+    } else {
+      run_mainloop<C>(p.g, row0, col0, smem, acc);
+    }
+
+    // vocabulary rows past V get a logit that exponentiates to exactly 0; the bias joins the raw product
+    if (p.bias != nullptr || row0 + C::BM > V) {
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i) {
+      for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int rr0 = i * 32 + 8 * q;  // row relative to the lane's first row
-          float ds[4];
+        for (int r = 0; r < 16; ++r) {
+          const int v = row0 + acc_row<C>(wm, i, r, lane);
+          const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float pr = fast_exp2(__builtin_fmaf(acc[i][j][q * 4 + e], xs, -lse2));
-            if constexpr (decltype(with_y)::value)
-              ds[e] = __builtin_fmaf(nc, pr, (rr0 + e == yrel) ? c : 0.f);
-            else
-              ds[e] = nc * pr;
-          }
-          // [token][vocab]: four consecutive vocabulary entries = one 8-byte store
-          uint2 pk;
-          pk.x = pack_bf16x2(ds[0], ds[1]);
-          pk.y = pack_bf16x2(ds[2], ds[3]);
-          if constexpr (decltype(via_lds)::value) {
-            *(uint2*)(patch + (lane & 31) * EROW + (rr0 + 4 * (lane >> 5)) * 2) = pk;
-            continue;
-          }
-          *(uint2*)(tv_hi + rr0) = pk;
-          uint2 pl;
-          if (SPLIT) {
-            pl.x = pack_bf16x2(ds[0] - __uint_as_float(pk.x << 16), ds[1] - __uint_as_float(pk.x & 0xffff0000u));
-            pl.y = pack_bf16x2(ds[2] - __uint_as_float(pk.y << 16), ds[3] - __uint_as_float(pk.y & 0xffff0000u));
-            *(uint2*)(tv_lo + rr0) = pl;
-          }
-          // [vocab][token] (only when the consumer GEMM wants that copy): lanes hold consecutive tokens
-          if (vt_hi != nullptr) {
-            vt_hi[(long long)(rr0 + 0) * p.ld_vt] = (uint16_t)(pk.x & 0xffffu);
-            vt_hi[(long long)(rr0 + 1) * p.ld_vt] = (uint16_t)(pk.x >> 16);
-            vt_hi[(long long)(rr0 + 2) * p.ld_vt] = (uint16_t)(pk.y & 0xffffu);
-            vt_hi[(long long)(rr0 + 3) * p.ld_vt] = (uint16_t)(pk.y >> 16);
-            if (SPLIT && vt_lo != nullptr) {
-              vt_lo[(long long)(rr0 + 0) * p.ld_vt] = (uint16_t)(pl.x & 0xffffu);
-              vt_lo[(long long)(rr0 + 1) * p.ld_vt] = (uint16_t)(pl.x >> 16);
-              vt_lo[(long long)(rr0 + 2) * p.ld_vt] = (uint16_t)(pl.y & 0xffffu);
-              vt_lo[(long long)(rr0 + 3) * p.ld_vt] = (uint16_t)(pl.y >> 16);
+          for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      const int n = col0 + acc_col<C>(wn, j, lane);
+      const float c = cj[j], nc = -c, l2 = lse2[j];
+      // target row relative to this lane's first row; out of range when not in this sub-tile
+      const int yrel = ylab[j] - row0 - lane_row0;
+      // Few wavefronts hold a target row at all (64 tokens x WTM of V rows): the common case runs without
+      // the per-element comparison.
+      const bool any_y = __builtin_amdgcn_ballot_w64(yrel >= 0 && yrel < C::WTM) != 0;
+      auto emit = [&](auto with_y, auto via_lds) {
+        // The swizzled patch addresses are recomputed per tile on purpose: hoisted out of the vocabulary loop they
+        // would occupy two dozen registers across the main loop.  The empty asm makes them loop-variant.
+        int lane_v = lane;
+        asm volatile("" : "+v"(lane_v));
+        bf16_t *tv_hi = nullptr, *tv_lo = nullptr, *vt_hi = nullptr, *vt_lo = nullptr;
+        if constexpr (!decltype(via_lds)::value) {      // direct stores: plain or blocked rows, optional [vocab][token] copy
+          const long long tv_off = p.tv_blk ? (long long)vt * p.tv_blk + (long long)n * 256 + lane_row0
+                                            : (long long)n * p.ld_tv + prow0 + lane_row0;
+          tv_hi = p.tv_hi + tv_off;
+          tv_lo = SPLIT ? p.tv_lo + tv_off : nullptr;
+          vt_hi = p.vt_hi ? p.vt_hi + (long long)(prow0 + lane_row0) * p.ld_vt + n : nullptr;
+          vt_lo = (SPLIT && p.vt_lo) ? p.vt_lo + (long long)(prow0 + lane_row0) * p.ld_vt + n : nullptr;
+        }
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int rr0 = i * 32 + 8 * q;  // row relative to the lane's first row
+            float ds[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float pr = fast_exp2(__builtin_fmaf(acc[i][j][q * 4 + e], xs, -l2));
+              if constexpr (decltype(with_y)::value)
+                ds[e] = __builtin_fmaf(nc, pr, (rr0 + e == yrel) ? c : 0.f);
+              else
+                ds[e] = nc * pr;
+            }
+            // four consecutive vocabulary entries of one token = 8 bytes
+            uint2 pk;
+            pk.x = pack_bf16x2(ds[0], ds[1]);
+            pk.y = pack_bf16x2(ds[2], ds[3]);
+            if constexpr (decltype(via_lds)::value) {
+              const int slot = (rr0 >> 2) + (lane_v >> 5);             // 8-byte slot of (rr0 + 4*(lane/32)) in the row
+              *(uint2*)(patch + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3)) = pk;
+              continue;
+            }
+            *(uint2*)(tv_hi + rr0) = pk;
+            uint2 pl;
+            if (SPLIT) {
+              pl.x = pack_bf16x2(ds[0] - __uint_as_float(pk.x << 16), ds[1] - __uint_as_float(pk.x & 0xffff0000u));
+              pl.y = pack_bf16x2(ds[2] - __uint_as_float(pk.y << 16), ds[3] - __uint_as_float(pk.y & 0xffff0000u));
+              *(uint2*)(tv_lo + rr0) = pl;
+            }
+            // [vocab][token] (only when the consumer GEMM wants that copy): lanes hold consecutive tokens
+            if (vt_hi != nullptr) {
+              vt_hi[(long long)(rr0 + 0) * p.ld_vt] = (uint16_t)(pk.x & 0xffffu);
+              vt_hi[(long long)(rr0 + 1) * p.ld_vt] = (uint16_t)(pk.x >> 16);
+              vt_hi[(long long)(rr0 + 2) * p.ld_vt] = (uint16_t)(pk.y & 0xffffu);
+              vt_hi[(long long)(rr0 + 3) * p.ld_vt] = (uint16_t)(pk.y >> 16);
+              if (SPLIT && vt_lo != nullptr) {
+                vt_lo[(long long)(rr0 + 0) * p.ld_vt] = (uint16_t)(pl.x & 0xffffu);
+                vt_lo[(long long)(rr0 + 1) * p.ld_vt] = (uint16_t)(pl.x >> 16);
+                vt_lo[(long long)(rr0 + 2) * p.ld_vt] = (uint16_t)(pl.y & 0xffffu);
+                vt_lo[(long long)(rr0 + 3) * p.ld_vt] = (uint16_t)(pl.y >> 16);
+              }
             }
           }
         }
-      }
-      if constexpr (decltype(via_lds)::value) {
-        bf16_t* out = p.tv_hi + (long long)tv * p.tv_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
+        if constexpr (decltype(via_lds)::value) {
+          bf16_t* out = p.tv_hi + (long long)vt * p.tv_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
 #pragma unroll
-        for (int r = 0; r < 32 / TPP; ++r) {
-          const int tok = r * TPP + lane / PPT, piece = lane % PPT;
-          const u32x4_t v = *(const u32x4_t*)(patch + tok * EROW + piece * 16);
-          *(u32x4_t*)(out + (long long)tok * 256 + piece * 8) = v;
+          for (int r = 0; r < 32 / TPP; ++r) {
+            const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
+            const int m = tok & (NSLOT - 1);
+            u32x4_t v = *(const u32x4_t*)(patch + tok * ROWP + ((piece ^ (m >> 1)) << 4));
+            if (m & 1) v = u32x4_t{v[2], v[3], v[0], v[1]};       // odd rows hold the two slots of a piece swapped
+            *(u32x4_t*)(out + (long long)tok * 256 + piece * 8) = v;
+          }
         }
+      };
+      if (through_lds) {
+        if (any_y)
+          emit(std::true_type{}, std::true_type{});
+        else
+          emit(std::false_type{}, std::true_type{});
+      } else {
+        if (any_y)
+          emit(std::true_type{}, std::false_type{});
+        else
+          emit(std::false_type{}, std::false_type{});
       }
-    };
-    const bool through_lds = !SPLIT && p.tv_blk != 0;
-    if (through_lds) {
-      if (any_y)
-        emit(std::true_type{}, std::true_type{});
-      else
-        emit(std::false_type{}, std::true_type{});
-    } else {
-      if (any_y)
-        emit(std::true_type{}, std::false_type{});
-      else
-        emit(std::false_type{}, std::false_type{});
     }
+    if constexpr (!kPrefetch) __syncthreads();   // the patch (or the direct stores) are done before the buffers refill
   }
 }
 
