@@ -76,7 +76,7 @@ struct Tuning {
   int gemm_group_m = 4;
   int panel_cols = 32768;  // default vocabulary panel width of the backward
   int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
-  int bwd_kmajor = 1;      // 1: the dW GEMM reads dLogits and hidden in place; 2: the dH GEMM reads W in place too
+  int bwd_kmajor = 2;      // 0: transposed copies; 1: the dW GEMM reads dLogits and hidden in place; 2: the dH GEMM reads W in place too
 } g_tune;
 
 int* tuning_slot(const char* key) {

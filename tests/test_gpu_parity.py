@@ -220,7 +220,7 @@ def test_backward_operand_layout_modes_agree(dev, kmajor):
     try:
         want, got, o, g, _, _ = run_case(w, dev, "north_star", bias=bias)
     finally:
-        _lib.set_tuning(bwd_kmajor=1)
+        _lib.set_tuning(bwd_kmajor=2)
     check(want, got, o, g, f32=False)
 
 
