@@ -257,6 +257,12 @@ __device__ __forceinline__ bf16x8_t lds_read_tr_pair(uint32_t addr) {
   const u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
   return __builtin_bit_cast(bf16x8_t, v);
 }
+// 8-byte LDS store the compiler does not see either (an epilogue patch written while direct-to-LDS loads of the
+// next tile are in flight would otherwise wait for them)
+__device__ __forceinline__ void lds_write_b64_asm(uint32_t addr, uint32_t lo, uint32_t hi) {
+  const u32x2_t v = {lo, hi};
+  asm volatile("ds_write_b64 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
 template <int OFF>
 __device__ __forceinline__ bf16x8_t lds_read_b128_asm(uint32_t addr) {
   static_assert(OFF >= 0 && OFF < 65536, "DS offset field");

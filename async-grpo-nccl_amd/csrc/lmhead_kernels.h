@@ -382,7 +382,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
             pk.y = pack_bf16x2(ds[2], ds[3]);
             if constexpr (decltype(via_lds)::value) {
               const int slot = (rr0 >> 2) + (lane_v >> 5);             // 8-byte slot of (rr0 + 4*(lane/32)) in the row
-              *(uint2*)(patch + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3)) = pk;
+              lds_write_b64_asm(lds_addr(patch) + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3), pk.x, pk.y);
               continue;
             }
             *(uint2*)(tv_hi + rr0) = pk;
@@ -409,11 +409,22 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
         }
         if constexpr (decltype(via_lds)::value) {
           bf16_t* out = p.tv_hi + (long long)vt * p.tv_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
+          // inline-assembly LDS traffic (see lds_write_b64_asm): one wait for all reads, LDS operations of a
+          // wavefront complete in order, so the reads see this wavefront's writes
+          u32x4_t pv[32 / TPP];
 #pragma unroll
           for (int r = 0; r < 32 / TPP; ++r) {
             const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
             const int m = tok & (NSLOT - 1);
-            u32x4_t v = *(const u32x4_t*)(patch + tok * ROWP + ((piece ^ (m >> 1)) << 4));
+            pv[r] = __builtin_bit_cast(u32x4_t, lds_read_b128_asm<0>(lds_addr(patch) + tok * ROWP + ((piece ^ (m >> 1)) << 4)));
+          }
+          wait_lgkm<0>();
+          __builtin_amdgcn_sched_barrier(0);     // nothing that consumes pv may move above the wait
+#pragma unroll
+          for (int r = 0; r < 32 / TPP; ++r) {
+            const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
+            const int m = tok & (NSLOT - 1);
+            u32x4_t v = pv[r];
             if (m & 1) v = u32x4_t{v[2], v[3], v[0], v[1]};       // odd rows hold the two slots of a piece swapped
             *(u32x4_t*)(out + (long long)tok * 256 + piece * 8) = v;
           }
