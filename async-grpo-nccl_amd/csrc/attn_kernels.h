@@ -1,0 +1,481 @@
+// Packed variable-length attention for gfx950 (head dimension 128, bf16 operands, fp32 softmax and accumulators):
+// forward with log-sum-exp output, and the backward as two kernels (dQ by query tile, dK/dV by key tile).
+// Replaces the flash-attn varlen call of the reference's packed path (gpu_process_worker.py:265-276) with the
+// K/V head repeat of its grouped-query wrapper folded into the head index (gpu_process_worker.py:154-161).
+//
+// Tiling works on the PACKED token axis: a work-group owns 128 consecutive tokens whatever segments they
+// belong to, and every score is masked with its query's own key range [seg_start[q], q] (causal) or
+// [seg_start[q], seg_end[q]) - so no tile-to-segment map is needed and short segments share tiles.
+//
+// MFMA orientation (v_mfma_f32_32x32x16_bf16; operand lane l = row l%32, k values 8*(l/32)..+7; result lane l =
+// column l%32, rows 8*(r/4) + 4*(l/32) + r%4 for r = 0..15):
+//  * query-side kernels (forward, dQ) compute S^T = K Q^T, so that a lane owns ONE query (its column) and 32 of
+//    the 64 keys of a step: the running max/sum, the rescale of the output accumulator (kept transposed,
+//    O^T = V^T P^T) and the bf16 P all stay inside the lane - no cross-lane traffic but one 32-lane swap per
+//    step for the row max.  The fp32 P values of a lane are, as they sit in the accumulator, exactly the k
+//    values the next MFMA wants from that lane, up to a permutation of the keys that the other operand (V^T,
+//    read with ds_read_b64_tr_b16 from the [key][d] tile) simply follows.
+//  * the key-side kernel (dK/dV) computes S = Q K^T, so that a lane owns one key and P / dS feed the
+//    dV = P^T dO and dK = dS^T Q products from registers in the same way.
+// LDS tiles are [row][128] bf16 with the 16-byte chunk index XOR ((row&3)<<2 | (row>>2)&3): conflict-free both
+// for 16-byte row reads (16 consecutive rows, one chunk) and for the transposing reads (4 consecutive rows x 64 B).
+#pragma once
+#include "lmhead_kernels.h"
+
+namespace fgrpo {
+
+constexpr int kHD = 128;             // head dimension
+constexpr int kAttnBQ = 128;         // tokens per work-group (32 per wavefront)
+constexpr int kAttnBK = 64;          // tokens of the other side per step
+constexpr int kAttnRowB = kHD * 2;   // bytes of one LDS row
+constexpr int kAttnTile = kAttnBK * kAttnRowB;
+
+struct AttnParams {
+  const bf16_t* q;       // [T][Hq][128] with element strides q_st (token), q_sh (head)
+  const bf16_t* k;       // [T][Hkv][128]
+  const bf16_t* v;
+  long long q_st, q_sh, k_st, k_sh, v_st, v_sh;
+  const int* seg_start;  // [T] first token of the token's segment
+  const int* seg_end;    // [T] one past the last token of the token's segment
+  int T, Hq, Hkv;
+  float scale;
+  int causal;
+  bf16_t* out;           // [T][Hq][128] contiguous
+  float* lse;            // [Hq][T], natural log of the softmax denominator
+  // backward
+  const bf16_t* dout;    // [T][Hq][128] contiguous
+  const float* delta;    // [Hq][T] rowsum(dO * O)
+  bf16_t* dq;            // [T][Hq][128] contiguous
+  bf16_t* dk;            // [T][Hkv][128] contiguous
+  bf16_t* dv;
+};
+
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int attn_swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
+// K-contiguous fragment: the 8 values [row][8*chunk .. 8*chunk+7]
+__device__ __forceinline__ bf16x8_t attn_frag(const char* tile, int row, int chunk) {
+  return *(const bf16x8_t*)(tile + row * kAttnRowB + ((chunk ^ attn_swz(row)) << 4));
+}
+
+// K-major fragment: lane (n = lane%32, h = lane/32) receives Tile[kbase + 4h + 8*(j/4) + j%4][col0 + n] for the
+// eight slots j = 0..7 (kbase a multiple of 16, col0 of 32) - the key order in which a result accumulator
+// hands its values to the next MFMA.
+__device__ __forceinline__ bf16x8_t attn_frag_tr(const char* tile, int kbase, int col0, int lane) {
+  const int h = lane >> 5, g1 = (lane >> 4) & 1, j = lane & 15;
+  const int chunk = (col0 >> 3) + 2 * g1 + ((j & 3) >> 1);
+  const int r0 = kbase + 4 * h + (j >> 2), r1 = r0 + 8;
+  const char* p0 = tile + r0 * kAttnRowB + ((chunk ^ attn_swz(r0)) << 4) + 8 * (j & 1);
+  const char* p1 = tile + r1 * kAttnRowB + ((chunk ^ attn_swz(r1)) << 4) + 8 * (j & 1);
+  const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p0));
+  const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p1));
+  typedef short i16x8_t __attribute__((ext_vector_type(8)));
+  const i16x8_t v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
+// eight consecutive accumulator values -> one bf16 operand
+__device__ __forceinline__ bf16x8_t attn_pack8(const float* x) {
+  const u32x4_t v = {pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7])};
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
+// 64 rows x 256 bytes of one head: global -> registers (rows >= row_end read as zero) ...
+__device__ __forceinline__ void attn_fetch_rows(u32x4_t (&r)[4], const bf16_t* base, long long st, int row0, int row_end) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    const int row = row0 + (c >> 4);
+    const u32x4_t z = {0u, 0u, 0u, 0u};
+    r[i] = (row >= 0 && row < row_end) ? *(const u32x4_t*)(base + (long long)row * st + (c & 15) * 8) : z;
+  }
+}
+// ... and registers -> swizzled LDS tile
+__device__ __forceinline__ void attn_put_rows(const u32x4_t (&r)[4], char* tile) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    const int row = c >> 4;
+    *(u32x4_t*)(tile + row * kAttnRowB + (((c & 15) ^ attn_swz(row)) << 4)) = r[i];
+  }
+}
+
+// the lane's own row of one head as an MFMA operand: chunks 2s + h, s = 0..7
+__device__ __forceinline__ void attn_row_operand(bf16x8_t (&f)[8], const bf16_t* row_ptr, bool valid, int h) {
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const u32x4_t z = {0u, 0u, 0u, 0u};
+    const u32x4_t x = valid ? *(const u32x4_t*)(row_ptr + (2 * s + h) * 8) : z;
+    f[s] = __builtin_bit_cast(bf16x8_t, x);
+  }
+}
+
+__device__ __forceinline__ float attn_swap32(float x) { return __shfl_xor(x, 32, 64); }
+
+// transposed accumulator (4 blocks of 32 d x 32 tokens, the lane's token = its column) -> [token][head][128] bf16
+__device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[4], float mul, bf16_t* row_ptr, int h) {
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint2 pk;
+      pk.x = pack_bf16x2(acc[db][4 * g + 0] * mul, acc[db][4 * g + 1] * mul);
+      pk.y = pack_bf16x2(acc[db][4 * g + 2] * mul, acc[db][4 * g + 3] * mul);
+      *(uint2*)(row_ptr + 32 * db + 8 * g + 4 * h) = pk;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Forward: grid (ceil(T/128), Hq), 256 threads.
+// ---------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void varlen_attn_fwd_kernel(AttnParams p) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
+  char* kt = smem;
+  char* vt = smem + kAttnTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
+  const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
+  const int q0 = blockIdx.x * kAttnBQ;
+  const int tq = q0 + 32 * wave + (lane & 31);
+  const bool valid = tq < p.T;
+  const int lo = valid ? p.seg_start[tq] : 1;
+  const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
+  const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
+  const int k_begin = p.seg_start[q0];
+  const int k_end = p.causal ? last + 1 : p.seg_end[last];
+  // this wavefront's own key range (whole steps outside it are skipped)
+  const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = wfirst < p.T;
+  const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
+  const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
+
+  bf16x8_t qf[8];
+  attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
+
+  f32x16_t acc_o[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_o[db][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale * kLog2e;
+
+  const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
+  const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
+  u32x4_t rk[4], rv[4];
+  attn_fetch_rows(rk, kbase, p.k_st, k_begin, k_end);
+  attn_fetch_rows(rv, vbase, p.v_st, k_begin, k_end);
+  for (int kb = k_begin; kb < k_end; kb += kAttnBK) {
+    attn_put_rows(rk, kt);
+    attn_put_rows(rv, vt);
+    __syncthreads();
+    if (kb + kAttnBK < k_end) {   // next step's rows travel while this one is computed
+      attn_fetch_rows(rk, kbase, p.k_st, kb + kAttnBK, k_end);
+      attn_fetch_rows(rv, vbase, p.v_st, kb + kAttnBK, k_end);
+    }
+    if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
+      f32x16_t s[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[mb][r] = 0.f;
+#pragma unroll
+        for (int st = 0; st < 8; ++st) s[mb] = FGRPO_MFMA(attn_frag(kt, 32 * mb + (lane & 31), 2 * st + h), qf[st], s[mb]);
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
+          const float x = (key >= lo && key <= hi) ? s[mb][r] : -INFINITY;
+          s[mb][r] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, attn_swap32(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2((m_run - m_use) * c);
+      const float mc = m_use * c;
+      float sum = 0.f;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = fast_exp2(__builtin_fmaf(s[mb][r], c, -mc));
+          s[mb][r] = e;
+          sum += e;
+        }
+      l_run = l_run * alpha + sum;
+      m_run = m_new;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[db][r] *= alpha;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          float tmp[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) tmp[j] = s[mb][8 * s2 + j];
+          const bf16x8_t pf = attn_pack8(tmp);
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+            acc_o[db] = FGRPO_MFMA(attn_frag_tr(vt, 32 * mb + 16 * s2, 32 * db, lane), pf, acc_o[db]);
+        }
+    }
+    __syncthreads();
+  }
+  const float l = l_run + attn_swap32(l_run);
+  if (valid) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    attn_store_rowmajor(acc_o, inv, p.out + ((long long)tq * p.Hq + hq) * kHD, h);
+    if (h == 0) p.lse[(long long)hq * p.T + tq] = l > 0.f ? m_run * p.scale + __logf(l) : -INFINITY;
+  }
+}
+
+// delta[hq][t] = sum_d dO[t][hq][d] * O[t][hq][d]; 16 lanes per row, grid ceil(T*Hq / 16), 256 threads
+__global__ void varlen_attn_delta_kernel(const bf16_t* dout, const bf16_t* out, int T, int Hq, float* delta) {
+  const long long row = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int part = threadIdx.x & 15;
+  float a = 0.f;
+  if (row < (long long)T * Hq) {
+    const u32x4_t x = *(const u32x4_t*)(dout + row * kHD + part * 8);
+    const u32x4_t y = *(const u32x4_t*)(out + row * kHD + part * 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a += __uint_as_float(x[i] << 16) * __uint_as_float(y[i] << 16);
+      a += __uint_as_float(x[i] & 0xffff0000u) * __uint_as_float(y[i] & 0xffff0000u);
+    }
+  }
+#pragma unroll
+  for (int o = 8; o >= 1; o >>= 1) a += __shfl_xor(a, o, 64);
+  if (part == 0 && row < (long long)T * Hq) {
+    const int t = (int)(row / Hq), hq = (int)(row % Hq);
+    delta[(long long)hq * T + t] = a;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dQ: grid (ceil(T/128), Hq), 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
+// ---------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void varlen_attn_dq_kernel(AttnParams p) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
+  char* kt = smem;
+  char* vt = smem + kAttnTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
+  const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
+  const int q0 = blockIdx.x * kAttnBQ;
+  const int tq = q0 + 32 * wave + (lane & 31);
+  const bool valid = tq < p.T;
+  const int lo = valid ? p.seg_start[tq] : 1;
+  const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
+  const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
+  const int k_begin = p.seg_start[q0];
+  const int k_end = p.causal ? last + 1 : p.seg_end[last];
+  const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = wfirst < p.T;
+  const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
+  const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
+
+  bf16x8_t qf[8], dof[8];
+  attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
+  attn_row_operand(dof, p.dout + ((long long)(valid ? tq : 0) * p.Hq + hq) * kHD, valid, h);
+  const float lse2 = valid ? p.lse[(long long)hq * p.T + tq] * kLog2e : 0.f;
+  const float dl = valid ? p.delta[(long long)hq * p.T + tq] : 0.f;
+  const float c = p.scale * kLog2e;
+
+  f32x16_t acc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+
+  const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
+  const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
+  u32x4_t rk[4], rv[4];
+  attn_fetch_rows(rk, kbase, p.k_st, k_begin, k_end);
+  attn_fetch_rows(rv, vbase, p.v_st, k_begin, k_end);
+  for (int kb = k_begin; kb < k_end; kb += kAttnBK) {
+    attn_put_rows(rk, kt);
+    attn_put_rows(rv, vt);
+    __syncthreads();
+    if (kb + kAttnBK < k_end) {
+      attn_fetch_rows(rk, kbase, p.k_st, kb + kAttnBK, k_end);
+      attn_fetch_rows(rv, vbase, p.v_st, kb + kAttnBK, k_end);
+    }
+    if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+        f32x16_t s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+        for (int st = 0; st < 8; ++st) {
+          s = FGRPO_MFMA(attn_frag(kt, 32 * mb + (lane & 31), 2 * st + h), qf[st], s);
+          dp = FGRPO_MFMA(attn_frag(vt, 32 * mb + (lane & 31), 2 * st + h), dof[st], dp);
+        }
+        float ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
+          const float pr = (key >= lo && key <= hi) ? fast_exp2(__builtin_fmaf(s[r], c, -lse2)) : 0.f;
+          ds[r] = pr * (dp[r] - dl) * p.scale;
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const bf16x8_t dsf = attn_pack8(ds + 8 * s2);
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+            acc[db] = FGRPO_MFMA(attn_frag_tr(kt, 32 * mb + 16 * s2, 32 * db, lane), dsf, acc[db]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (valid) attn_store_rowmajor(acc, 1.f, p.dq + ((long long)tq * p.Hq + hq) * kHD, h);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dK, dV: grid (ceil(T/128), Hkv), 256 threads; a wavefront owns 32 keys (one per lane pair) and walks the
+// queries that can see them, for every query head of the group.
+// ---------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
+  __shared__ __attribute__((aligned(16))) float row_lse2[kAttnBK];
+  __shared__ __attribute__((aligned(16))) float row_dl[kAttnBK];
+  __shared__ __attribute__((aligned(16))) int row_lo[kAttnBK];
+  __shared__ __attribute__((aligned(16))) int row_hi[kAttnBK];
+  char* qt = smem;
+  char* dot = smem + kAttnTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
+  const int hkv = blockIdx.y, G = p.Hq / p.Hkv;
+  const int k0 = blockIdx.x * kAttnBQ;
+  const int key = k0 + 32 * wave + (lane & 31);
+  const bool valid = key < p.T;
+  const int last = (k0 + kAttnBQ - 1 < p.T ? k0 + kAttnBQ - 1 : p.T - 1);
+  // queries that can see a key of this tile
+  const int q_begin = p.causal ? k0 : p.seg_start[k0];
+  const int q_end = p.seg_end[last];
+  const int wfirst = k0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = wfirst < p.T;
+  const int wq_lo = wave_on ? (p.causal ? wfirst : p.seg_start[wfirst]) : 1;   // first / last query of interest
+  const int wq_hi = wave_on ? p.seg_end[wlast] - 1 : 0;
+
+  bf16x8_t kf[8], vf[8];
+  attn_row_operand(kf, p.k + (long long)(valid ? key : 0) * p.k_st + (long long)hkv * p.k_sh, valid, h);
+  attn_row_operand(vf, p.v + (long long)(valid ? key : 0) * p.v_st + (long long)hkv * p.v_sh, valid, h);
+  const float c = p.scale * kLog2e;
+
+  f32x16_t acc_k[4], acc_v[4];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_k[nb][r] = acc_v[nb][r] = 0.f;
+
+  for (int g = 0; g < G; ++g) {
+    const int hq = hkv * G + g;
+    const bf16_t* qbase = p.q + (long long)hq * p.q_sh;
+    const bf16_t* dobase = p.dout + (long long)hq * kHD;
+    const long long do_st = (long long)p.Hq * kHD;
+    u32x4_t rq[4], rd[4];
+    attn_fetch_rows(rq, qbase, p.q_st, q_begin, q_end);
+    attn_fetch_rows(rd, dobase, do_st, q_begin, q_end);
+    for (int qb = q_begin; qb < q_end; qb += kAttnBK) {
+      attn_put_rows(rq, qt);
+      attn_put_rows(rd, dot);
+      if (threadIdx.x < kAttnBK) {
+        const int t = qb + threadIdx.x;
+        const bool ok = t < q_end;
+        row_lse2[threadIdx.x] = ok ? p.lse[(long long)hq * p.T + t] * kLog2e : 0.f;
+        row_dl[threadIdx.x] = ok ? p.delta[(long long)hq * p.T + t] : 0.f;
+        row_lo[threadIdx.x] = ok ? p.seg_start[t] : 1;
+        row_hi[threadIdx.x] = ok ? (p.causal ? t : p.seg_end[t] - 1) : 0;
+      }
+      __syncthreads();
+      if (qb + kAttnBK < q_end) {
+        attn_fetch_rows(rq, qbase, p.q_st, qb + kAttnBK, q_end);
+        attn_fetch_rows(rd, dobase, do_st, qb + kAttnBK, q_end);
+      }
+      if (wave_on && qb <= wq_hi && qb + kAttnBK > wq_lo) {
+#pragma unroll
+        for (int mq = 0; mq < 2; ++mq) {
+          f32x16_t s, dp;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+          for (int st = 0; st < 8; ++st) {
+            s = FGRPO_MFMA(attn_frag(qt, 32 * mq + (lane & 31), 2 * st + h), kf[st], s);
+            dp = FGRPO_MFMA(attn_frag(dot, 32 * mq + (lane & 31), 2 * st + h), vf[st], dp);
+          }
+          float pr[16], ds[16];
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int row = 32 * mq + 8 * r4 + 4 * h;
+            const float4 l4 = *(const float4*)(row_lse2 + row);
+            const float4 d4 = *(const float4*)(row_dl + row);
+            const int4 lo4 = *(const int4*)(row_lo + row);
+            const int4 hi4 = *(const int4*)(row_hi + row);
+            const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
+            const int lo[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, hi[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int r = 4 * r4 + e;
+              const float pv = (key >= lo[e] && key <= hi[e]) ? fast_exp2(__builtin_fmaf(s[r], c, -ls[e])) : 0.f;
+              pr[r] = pv;
+              ds[r] = pv * (dp[r] - dd[e]) * p.scale;
+            }
+          }
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const bf16x8_t pf = attn_pack8(pr + 8 * s2);
+            const bf16x8_t dsf = attn_pack8(ds + 8 * s2);
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+              acc_v[nb] = FGRPO_MFMA(pf, attn_frag_tr(dot, 32 * mq + 16 * s2, 32 * nb, lane), acc_v[nb]);
+              acc_k[nb] = FGRPO_MFMA(dsf, attn_frag_tr(qt, 32 * mq + 16 * s2, 32 * nb, lane), acc_k[nb]);
+            }
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // result lane = column d, rows = keys of this wavefront
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kk = k0 + 32 * wave + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (kk < p.T) {
+        const long long o = ((long long)kk * p.Hkv + hkv) * kHD + 32 * nb + (lane & 31);
+        p.dk[o] = f32_to_bf16_rn(acc_k[nb][r]);
+        p.dv[o] = f32_to_bf16_rn(acc_v[nb][r]);
+      }
+    }
+}
+
+// seg_start[t], seg_end[t] from cu_seqlens (tokens outside every segment stand alone)
+__global__ void segment_bounds_kernel(const int* cu, int nseq, int T, int* seg_start, int* seg_end) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  // largest i with cu[i] <= t
+  int a = 0, b = nseq;   // invariant: answer in [a, b] if cu[0] <= t
+  if (nseq <= 0 || t < cu[0] || t >= cu[nseq]) {
+    seg_start[t] = t;
+    seg_end[t] = t + 1;
+    return;
+  }
+  while (a < b) {
+    const int mid = (a + b + 1) >> 1;
+    if (cu[mid] <= t) a = mid; else b = mid - 1;
+  }
+  // cu[a] <= t < cu[a+1] (empty segments share a start and are skipped by taking the largest i)
+  int e = a + 1;
+  while (e < nseq && cu[e] <= t) ++e;
+  seg_start[t] = cu[a] > 0 ? cu[a] : 0;
+  seg_end[t] = cu[e] < T ? cu[e] : T;
+}
+
+}  // namespace fgrpo

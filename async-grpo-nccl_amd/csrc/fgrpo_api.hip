@@ -9,6 +9,7 @@
 
 #include "../../include/fgrpo.h"
 #include "tail_kernels.h"
+#include "attn_kernels.h"
 
 using namespace fgrpo;
 
@@ -859,6 +860,90 @@ int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long lo
     return rc;
   }
   return run_store_gemm_kmajor(s, a_kmajor != 0, b_kmajor != 0, (hipStream_t)stream);
+}
+
+// ---- packed variable-length attention ------------------------------------------------------------------
+namespace {
+int check_attn(const char* who, const void* q, const void* k, const void* v, long long q_st, long long q_sh,
+               long long k_st, long long k_sh, long long v_st, long long v_sh, const int32_t* cu, int n_seq, int T,
+               int Hq, int Hkv, int D, float scale, const int32_t* bounds_ws) {
+  if (!q || !k || !v || !cu || !bounds_ws) return fail(FGRPO_ERR_BAD_ARG, "%s: null argument", who);
+  if (T <= 0 || n_seq <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0)
+    return fail(FGRPO_ERR_BAD_ARG, "%s: T=%d n_seq=%d Hq=%d Hkv=%d", who, T, n_seq, Hq, Hkv);
+  if (D != kHD) return fail(FGRPO_ERR_BAD_ARG, "%s: head dimension %d not supported (128 only)", who, D);
+  if (!(scale > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "%s: softmax scale must be positive", who);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v)) return fail(FGRPO_ERR_ALIGN, "%s: q/k/v must be 16-byte aligned", who);
+  const long long st[6] = {q_st, q_sh, k_st, k_sh, v_st, v_sh};
+  for (int i = 0; i < 6; ++i)
+    if (st[i] <= 0 || st[i] % 8 != 0) return fail(FGRPO_ERR_ALIGN, "%s: strides must be positive multiples of 8 elements", who);
+  return 0;
+}
+
+void fill_attn(AttnParams& p, const void* q, const void* k, const void* v, long long q_st, long long q_sh,
+               long long k_st, long long k_sh, long long v_st, long long v_sh, int T, int Hq, int Hkv, float scale,
+               int causal, int32_t* bounds_ws) {
+  memset(&p, 0, sizeof(p));
+  p.q = (const bf16_t*)q;
+  p.k = (const bf16_t*)k;
+  p.v = (const bf16_t*)v;
+  p.q_st = q_st, p.q_sh = q_sh, p.k_st = k_st, p.k_sh = k_sh, p.v_st = v_st, p.v_sh = v_sh;
+  p.seg_start = bounds_ws;
+  p.seg_end = bounds_ws + T;
+  p.T = T, p.Hq = Hq, p.Hkv = Hkv;
+  p.scale = scale;
+  p.causal = causal != 0;
+}
+}  // namespace
+
+int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long q_st, long long q_sh, long long k_st,
+                          long long k_sh, long long v_st, long long v_sh, const int32_t* cu, int n_seq, int T, int Hq,
+                          int Hkv, int D, float scale, int causal, void* out, float* lse, int32_t* bounds_ws,
+                          void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  int rc = check_attn("varlen_attn_fwd", q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, cu, n_seq, T, Hq, Hkv, D, scale, bounds_ws);
+  if (rc) return rc;
+  if (!out || !lse) return fail(FGRPO_ERR_BAD_ARG, "varlen_attn_fwd: null output");
+  if (!aligned16(out)) return fail(FGRPO_ERR_ALIGN, "varlen_attn_fwd: out must be 16-byte aligned");
+  AttnParams p;
+  fill_attn(p, q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, T, Hq, Hkv, scale, causal, bounds_ws);
+  p.out = (bf16_t*)out;
+  p.lse = lse;
+  hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
+  HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(varlen_attn_fwd_kernel, dim3((T + kAttnBQ - 1) / kAttnBQ, Hq), dim3(256), 0, st, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                          long long q_st, long long q_sh, long long k_st, long long k_sh, long long v_st, long long v_sh,
+                          const int32_t* cu, int n_seq, int T, int Hq, int Hkv, int D, float scale, int causal, void* dq,
+                          void* dk, void* dv, float* delta_ws, int32_t* bounds_ws, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  int rc = check_attn("varlen_attn_bwd", q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, cu, n_seq, T, Hq, Hkv, D, scale, bounds_ws);
+  if (rc) return rc;
+  if (!dout || !out || !lse || !dq || !dk || !dv || !delta_ws) return fail(FGRPO_ERR_BAD_ARG, "varlen_attn_bwd: null argument");
+  if (!aligned16(dout) || !aligned16(out) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
+    return fail(FGRPO_ERR_ALIGN, "varlen_attn_bwd: dout/out/dq/dk/dv must be 16-byte aligned");
+  AttnParams p;
+  fill_attn(p, q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, T, Hq, Hkv, scale, causal, bounds_ws);
+  p.lse = const_cast<float*>(lse);
+  p.dout = (const bf16_t*)dout;
+  p.delta = delta_ws;
+  p.dq = (bf16_t*)dq;
+  p.dk = (bf16_t*)dk;
+  p.dv = (bf16_t*)dv;
+  hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
+  HIP_TRY(hipGetLastError());
+  const long long rows = (long long)T * Hq;
+  hipLaunchKernelGGL(varlen_attn_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const bf16_t*)dout,
+                     (const bf16_t*)out, T, Hq, delta_ws);
+  HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(varlen_attn_dq_kernel, dim3((T + kAttnBQ - 1) / kAttnBQ, Hq), dim3(256), 0, st, p);
+  HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(varlen_attn_dkv_kernel, dim3((T + kAttnBQ - 1) / kAttnBQ, Hkv), dim3(256), 0, st, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
 }
 
 }  // extern "C"

@@ -556,3 +556,94 @@ def fused_grpo_loss(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp=No
     return _FusedGRPOLoss.apply(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens,
                                 float(temperature), float(clip_low), float(clip_high), float(clip_ratio_c),
                                 float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint), bool(compact))
+
+
+# --------------------------------------------------------------------------- packed variable-length attention
+def _attn_operand(t: torch.Tensor, name: str) -> torch.Tensor:
+    """[T, H, 128] bf16 view the kernels can read in place (innermost contiguous, strides multiples of 8
+    elements, 16-byte aligned base); anything else is copied once."""
+    if t.dim() != 3:
+        raise RuntimeError(f"fgrpo: {name} must be [tokens, heads, head_dim], got {tuple(t.shape)}")
+    if t.dtype != torch.bfloat16:
+        raise RuntimeError(f"fgrpo: {name} must be bf16, got {t.dtype}")
+    t = t.detach()
+    ok = t.stride(2) == 1 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0 and t.stride(0) > 0 and t.stride(1) > 0 \
+        and t.data_ptr() % 16 == 0
+    return t if ok else _aligned(t)
+
+
+def varlen_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
+                    softmax_scale: Optional[float] = None, causal: bool = True):
+    """out [T, Hq, D] bf16 and lse [Hq, T] fp32 of packed self-attention: segment i covers tokens
+    cu_seqlens[i]:cu_seqlens[i+1]; query head j reads K/V head j // (Hq // Hkv)."""
+    dev = _require_cuda(q, k, v, cu_seqlens)
+    lib = _lib.load()
+    q, k, v = _attn_operand(q, "q"), _attn_operand(k, "k"), _attn_operand(v, "v")
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != v.shape or k.shape[0] != T or k.shape[2] != D:
+        raise RuntimeError(f"fgrpo: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit together")
+    cu = cu_seqlens.to(torch.int32).contiguous()
+    scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty((Hq, T), dtype=torch.float32, device=dev)
+    if T == 0:
+        return out, lse
+    bounds = torch.empty(2 * T, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_varlen_attn_fwd(_ptr(q), _ptr(k), _ptr(v), q.stride(0), q.stride(1), k.stride(0), k.stride(1),
+                                       v.stride(0), v.stride(1), _ptr(cu), cu.numel() - 1, T, Hq, Hkv, D, scale,
+                                       int(bool(causal)), _ptr(out), _ptr(lse), _ptr(bounds), _stream())
+    _lib.check(rc, "varlen_attn_fwd")
+    return out, lse
+
+
+def varlen_attn_bwd(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
+                    lse: torch.Tensor, cu_seqlens: torch.Tensor, softmax_scale: Optional[float] = None,
+                    causal: bool = True):
+    """(dq, dk, dv) bf16, contiguous, for the forward above."""
+    dev = _require_cuda(dout, q, k, v, out, lse, cu_seqlens)
+    lib = _lib.load()
+    q, k, v = _attn_operand(q, "q"), _attn_operand(k, "k"), _attn_operand(v, "v")
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    if dout.dtype != torch.bfloat16 or tuple(dout.shape) != (T, Hq, D):
+        raise RuntimeError(f"fgrpo: dout must be bf16 {(T, Hq, D)}, got {dout.dtype} {tuple(dout.shape)}")
+    dout, out = _aligned(dout), _aligned(out)
+    lse = lse.detach().to(torch.float32).contiguous()
+    cu = cu_seqlens.to(torch.int32).contiguous()
+    scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    dq = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
+    dk = torch.empty((T, Hkv, D), dtype=torch.bfloat16, device=dev)
+    dv = torch.empty((T, Hkv, D), dtype=torch.bfloat16, device=dev)
+    if T == 0:
+        return dq, dk, dv
+    delta = torch.empty((Hq, T), dtype=torch.float32, device=dev)
+    bounds = torch.empty(2 * T, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_varlen_attn_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), q.stride(0),
+                                       q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), _ptr(cu),
+                                       cu.numel() - 1, T, Hq, Hkv, D, scale, int(bool(causal)), _ptr(dq), _ptr(dk),
+                                       _ptr(dv), _ptr(delta), _ptr(bounds), _stream())
+    _lib.check(rc, "varlen_attn_bwd")
+    return dq, dk, dv
+
+
+class _VarlenAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens, softmax_scale, causal):
+        out, lse = varlen_attn_fwd(q, k, v, cu_seqlens, softmax_scale, causal)
+        ctx.save_for_backward(q, k, v, out, lse, cu_seqlens)
+        ctx.softmax_scale, ctx.causal = softmax_scale, causal
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, cu = ctx.saved_tensors
+        dq, dk, dv = varlen_attn_bwd(dout.to(torch.bfloat16), q, k, v, out, lse, cu, ctx.softmax_scale, ctx.causal)
+        return dq, dk, dv, None, None, None
+
+
+def varlen_attention(q, k, v, cu_seqlens, softmax_scale=None, causal=True) -> torch.Tensor:
+    """Differentiable packed self-attention on the HIP kernels (bf16 in, bf16 out)."""
+    return _VarlenAttention.apply(q, k, v, cu_seqlens, softmax_scale, causal)

@@ -171,6 +171,30 @@ int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long lo
                       int a_kmajor, int b_kmajor, long long a_blk, int k_valid, const float* c_in,
                       float* c_out_f32, void* c_out_bf16, long long ldc, float alpha, void* stream);
 
+/* ---- packed variable-length attention ----------------------------------------------
+ * Replaces the flash-attn call of the reference's packed path,
+ * flash_attn_varlen_func(q, k, v, cu_seqlens_q=cu, cu_seqlens_k=cu, ..., softmax_scale, causal)
+ * (gpu_process_worker.py:265-276), with the K/V head repeat of its grouped-query wrapper
+ * (gpu_process_worker.py:154-161) done by head index: query head j reads K/V head j / (Hq/Hkv).
+ * q [T, Hq, D], k / v [T, Hkv, D] bf16, D == 128, innermost dimension contiguous, token and head
+ * strides in elements (multiples of 8), bases 16-byte aligned.  cu_seqlens [n_seq+1] int32 as built
+ * at gpu_process_worker.py:239-252 (the same vector for queries and keys).  bounds_ws: 2*T int32
+ * of scratch.  out [T, Hq, D] bf16 contiguous; lse [Hq, T] fp32 (natural log of the softmax
+ * denominator), needed by the backward.  dropout is not supported (the reference passes 0). */
+int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long q_stride_t, long long q_stride_h,
+                          long long k_stride_t, long long k_stride_h, long long v_stride_t, long long v_stride_h,
+                          const int32_t* cu_seqlens, int n_seq, int T, int Hq, int Hkv, int D, float softmax_scale,
+                          int causal, void* out, float* lse, int32_t* bounds_ws, void* stream);
+
+/* Backward of the above (autograd of flash_attn_varlen_func in the reference).  dout, out
+ * [T, Hq, D] bf16 contiguous; dq [T, Hq, D], dk / dv [T, Hkv, D] bf16 contiguous;
+ * delta_ws: Hq*T fp32 of scratch. */
+int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                          const float* lse, long long q_stride_t, long long q_stride_h, long long k_stride_t,
+                          long long k_stride_h, long long v_stride_t, long long v_stride_h, const int32_t* cu_seqlens,
+                          int n_seq, int T, int Hq, int Hkv, int D, float softmax_scale, int causal, void* dq, void* dk,
+                          void* dv, float* delta_ws, int32_t* bounds_ws, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,173 @@
+"""GPU parity of the packed variable-length attention kernels (through the C ABI) against the CPU oracle
+(oracle/attn_oracle.py, fp32 math on the same bf16-rounded inputs).
+
+Tolerances, bf16 inputs/outputs with fp32 softmax and accumulation: |d out| <= 2e-2 absolute for O(1) values
+(bf16 output rounding is 2^-8 relative, P is rounded to bf16 before P V) and mean |d out| <= 2e-3;
+|d lse| <= 2e-3; every gradient cosine >= 0.999 and max error <= 3 % of the gradient's largest entry."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import attn_oracle as A
+
+pytestmark = pytest.mark.gpu
+
+OUT_ATOL, OUT_MEAN, LSE_ATOL, COS_MIN, GRAD_REL = 2e-2, 2e-3, 2e-3, 0.999, 3e-2
+
+
+def cos(a, b):
+    return F.cosine_similarity(a.detach().float().flatten().cpu(), b.detach().float().flatten().cpu(), dim=0).item()
+
+
+def make(T, Hq, Hkv, seed, scale_in=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(T, Hq, 128, generator=g) * scale_in).bfloat16()
+    k = (torch.randn(T, Hkv, 128, generator=g) * scale_in).bfloat16()
+    v = torch.randn(T, Hkv, 128, generator=g).bfloat16()
+    do = torch.randn(T, Hq, 128, generator=g).bfloat16()
+    return q, k, v, do
+
+
+def check(dev, name, T, cu, Hq, Hkv, causal, seed=0, softmax_scale=None, backward=True):
+    from fgrpo import ops
+    print(f"[attention case] {name}: T={T} Hq={Hq} Hkv={Hkv} causal={causal} segments={len(cu) - 1}", flush=True)
+    q, k, v, do = make(T, Hq, Hkv, seed)
+    cu_t = torch.tensor(cu, dtype=torch.int32)
+    qo, ko, vo = (x.float().requires_grad_(True) for x in (q, k, v))
+    want, want_lse = A.varlen_attention(qo, ko, vo, cu_t, softmax_scale=softmax_scale, causal=causal, return_lse=True)
+    qg, kg, vg = (x.to(dev).requires_grad_(True) for x in (q, k, v))
+    got = ops.varlen_attention(qg, kg, vg, cu_t.to(dev), softmax_scale, causal)
+    _, lse = ops.varlen_attn_fwd(qg, kg, vg, cu_t.to(dev), softmax_scale, causal)
+    torch.cuda.synchronize()
+    err = (got.float().cpu() - want.detach()).abs()
+    assert err.max().item() <= OUT_ATOL, f"{name}: out max err {err.max().item()}"
+    assert err.mean().item() <= OUT_MEAN, f"{name}: out mean err {err.mean().item()}"
+    assert (lse.cpu() - want_lse).abs().max().item() <= LSE_ATOL, f"{name}: lse"
+    if not backward:
+        return
+    want.backward(do.float())
+    got.backward(do.to(dev))
+    torch.cuda.synchronize()
+    for nm, a, b in (("dq", qg.grad, qo.grad), ("dk", kg.grad, ko.grad), ("dv", vg.grad, vo.grad)):
+        if b.abs().max().item() < 1e-6:      # e.g. one-token segments: dq = dk = 0 exactly; a cosine says nothing
+            assert a.float().abs().max().item() <= 1e-3, f"{name}: {nm} should vanish"
+            continue
+        c = cos(a, b)
+        rel = (a.float().cpu() - b).abs().max().item() / max(b.abs().max().item(), 1e-12)
+        assert c >= COS_MIN, f"{name}: {nm} cosine {c}"
+        assert rel <= GRAD_REL, f"{name}: {nm} max error {rel} of the largest entry"
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_small_segments_share_a_tile(dev, causal):
+    check(dev, "short segments", 200, [0, 5, 6, 70, 71, 72, 200], 4, 2, causal, seed=1)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_segments_cross_tile_boundaries(dev, causal):
+    check(dev, "crossing tiles", 1000, [0, 130, 385, 390, 900, 1000], 4, 4, causal, seed=2)
+
+
+def test_one_long_segment(dev):
+    check(dev, "one segment", 777, [0, 777], 2, 1, True, seed=3)
+
+
+def test_grouped_query_shape_of_the_1_5b_model(dev):
+    # Qwen2.5-1.5B: 12 query heads, 2 K/V heads, head dimension 128
+    check(dev, "12/2 heads", 1536, [0, 300, 301, 900, 1536], 12, 2, True, seed=4)
+
+
+def test_single_token_segments_and_explicit_scale(dev):
+    T = 140
+    check(dev, "single tokens", T, list(range(T + 1)), 2, 2, True, seed=5)
+    check(dev, "explicit scale", 300, [0, 100, 300], 2, 1, True, seed=6, softmax_scale=0.05)
+
+
+def test_empty_segments_in_cu_seqlens(dev):
+    check(dev, "empty segments", 260, [0, 0, 100, 100, 100, 260], 2, 2, True, seed=7)
+
+
+def test_strided_operands_are_read_in_place(dev):
+    """q, k, v as slices of one fused [T, (Hq + 2 Hkv) * 128] projection, the way a fused QKV layer hands them over."""
+    from fgrpo import ops
+    T, Hq, Hkv = 500, 4, 2
+    print("[attention case] strided qkv", flush=True)
+    g = torch.Generator().manual_seed(8)
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * 128, generator=g).bfloat16().to(dev)
+    q = qkv[:, :Hq * 128].view(T, Hq, 128)
+    k = qkv[:, Hq * 128:(Hq + Hkv) * 128].view(T, Hkv, 128)
+    v = qkv[:, (Hq + Hkv) * 128:].view(T, Hkv, 128)
+    cu = torch.tensor([0, 123, 500], dtype=torch.int32, device=dev)
+    out, lse = ops.varlen_attn_fwd(q, k, v, cu)
+    out2, lse2 = ops.varlen_attn_fwd(q.contiguous(), k.contiguous(), v.contiguous(), cu)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+    do = torch.randn(T, Hq, 128, generator=g).bfloat16().to(dev)
+    g1 = ops.varlen_attn_bwd(do, q, k, v, out, lse, cu)
+    g2 = ops.varlen_attn_bwd(do, q.contiguous(), k.contiguous(), v.contiguous(), out, lse, cu)
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b)
+
+
+def test_full_size_properties(dev):
+    """T = 32768 packed like the benchmark micro-batch (too large for the oracle): size-independent properties.
+    Segments do not see each other (perturbing one segment leaves every other token bit-identical) and a
+    segment computed alone equals the same segment inside the pack."""
+    from fgrpo import ops
+    print("[attention case] full size", flush=True)
+    T, Hq, Hkv = 32768, 12, 2
+    g = torch.Generator().manual_seed(9)
+    lens = []
+    while sum(lens) < T:
+        lens.append(int(torch.randint(128, 1025, (1,), generator=g)))
+    lens[-1] -= sum(lens) - T
+    cu_l = [0]
+    for n in lens:
+        cu_l.append(cu_l[-1] + n)
+    cu = torch.tensor(cu_l, dtype=torch.int32, device=dev)
+    q = torch.randn(T, Hq, 128, generator=g).bfloat16().to(dev)
+    k = torch.randn(T, Hkv, 128, generator=g).bfloat16().to(dev)
+    v = torch.randn(T, Hkv, 128, generator=g).bfloat16().to(dev)
+    out, lse = ops.varlen_attn_fwd(q, k, v, cu)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    a, b = cu_l[3], cu_l[4]
+    k2, v2 = k.clone(), v.clone()
+    k2[a:b] += 1.0
+    v2[a:b] -= 1.0
+    out2, _ = ops.varlen_attn_fwd(q, k2, v2, cu)
+    assert torch.equal(out[:a], out2[:a]) and torch.equal(out[b:], out2[b:]) and not torch.equal(out[a:b], out2[a:b])
+    # the segment alone: same keys per query, but a different split into 64-key steps -> equal up to the
+    # rounding of the running rescale
+    alone, lse_alone = ops.varlen_attn_fwd(q[a:b], k[a:b], v[a:b], torch.tensor([0, b - a], dtype=torch.int32, device=dev))
+    assert (alone.float() - out[a:b].float()).abs().max().item() <= 2e-2
+    assert (lse_alone - lse[:, a:b]).abs().max().item() <= 1e-3
+    # one segment against the oracle
+    want, want_lse = A.varlen_attention(q[a:b].float().cpu(), k[a:b].float().cpu(), v[a:b].float().cpu(),
+                                        torch.tensor([0, b - a], dtype=torch.int32), return_lse=True)
+    assert (out[a:b].float().cpu() - want).abs().max().item() <= OUT_ATOL
+    assert (lse[:, a:b].cpu() - want_lse).abs().max().item() <= LSE_ATOL
+    # backward runs at this size and stays finite; dK/dV of a segment do not depend on the others
+    do = torch.randn(T, Hq, 128, generator=g).bfloat16().to(dev)
+    dq, dk, dv = ops.varlen_attn_bwd(do, q, k, v, out, lse, cu)
+    for t in (dq, dk, dv):
+        assert torch.isfinite(t.float()).all()
+    do2 = do.clone()
+    do2[a:b] *= 2
+    dq2, dk2, dv2 = ops.varlen_attn_bwd(do2, q, k, v, out, lse, cu)
+    for x, y in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert torch.equal(x[:a], y[:a]) and torch.equal(x[b:], y[b:])
+
+
+def test_argument_errors(dev):
+    from fgrpo import ops
+    cu = torch.tensor([0, 16], dtype=torch.int32, device=dev)
+    q64 = torch.zeros(16, 2, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="head dimension"):
+        ops.varlen_attn_fwd(q64, q64, q64, cu)
+    q = torch.zeros(16, 3, 128, dtype=torch.bfloat16, device=dev)
+    kv = torch.zeros(16, 2, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError):
+        ops.varlen_attn_fwd(q, kv, kv, cu)          # 3 query heads over 2 K/V heads
+    with pytest.raises(RuntimeError, match="bf16"):
+        ops.varlen_attn_fwd(q.float(), kv.float(), kv.float(), cu)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.varlen_attn_fwd(q.cpu(), kv.cpu(), kv.cpu(), cu.cpu())
