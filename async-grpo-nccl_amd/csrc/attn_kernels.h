@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void varlen_attn_fwd_kernel(AttnParams p) {
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = blockIdx.x * kAttnBQ;
+  const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
@@ -148,6 +148,10 @@ __global__ __launch_bounds__(256) void varlen_attn_fwd_kernel(AttnParams p) {
   const bool wave_on = wfirst < p.T;
   const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
   const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
+  // keys in [w_lo_max, w_hi_min] are visible to every query of the wavefront (only when all 32 rows exist)
+  const bool wave_full = wfirst + 31 < p.T;
+  const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
+  const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
 
   bf16x8_t qf[8];
   attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
@@ -183,15 +187,22 @@ __global__ __launch_bounds__(256) void varlen_attn_fwd_kernel(AttnParams p) {
         for (int st = 0; st < 8; ++st) s[mb] = FGRPO_MFMA(attn_frag(kt, 32 * mb + (lane & 31), 2 * st + h), qf[st], s[mb]);
       }
       float mx = -INFINITY;
+      if (kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min) {   // every pair of this step is visible
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
-          const float x = (key >= lo && key <= hi) ? s[mb][r] : -INFINITY;
-          s[mb][r] = x;
-          mx = fmaxf(mx, x);
-        }
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[mb][r]);
+      } else {
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
+            const float x = (key >= lo && key <= hi) ? s[mb][r] : -INFINITY;
+            s[mb][r] = x;
+            mx = fmaxf(mx, x);
+          }
+      }
       mx = fmaxf(mx, attn_swap32(mx));
       const float m_new = fmaxf(m_run, mx);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -266,7 +277,7 @@ __global__ __launch_bounds__(256) void varlen_attn_dq_kernel(AttnParams p) {
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = blockIdx.x * kAttnBQ;
+  const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
