@@ -171,3 +171,57 @@ def test_argument_errors(dev):
         ops.varlen_attn_fwd(q.float(), kv.float(), kv.float(), cu)
     with pytest.raises(RuntimeError, match="GPU"):
         ops.varlen_attn_fwd(q.cpu(), kv.cpu(), kv.cpu(), cu.cpu())
+
+
+def test_transformers_model_with_packed_position_ids(dev):
+    """A small random Qwen2 model (head dimension 128, 4 query heads over 2 K/V heads) on one packed row with
+    position_ids resets, attention routed through install_explicit_varlen_wrapper: logits and weight gradients
+    against the same model run segment by segment with Transformers' own eager attention."""
+    from transformers import Qwen2Config, Qwen2ForCausalLM
+    import varlen_attention as VA
+    print("[attention case] tiny Qwen2 model, packed row", flush=True)
+    cfg = Qwen2Config(vocab_size=512, hidden_size=512, intermediate_size=1024, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=1024)
+    torch.manual_seed(0)
+    model = Qwen2ForCausalLM(cfg).to(dev).to(torch.bfloat16)
+    lens = [37, 1, 200, 130]
+    T = sum(lens)
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, 512, (1, T), generator=g).to(dev)
+    pos = torch.cat([torch.arange(n) for n in lens]).unsqueeze(0).to(dev)
+    wsel = torch.randn(T, 512, generator=g).to(dev)
+
+    model.config._attn_implementation = "eager"
+    ref_logits = []
+    a = 0
+    for n in lens:
+        ref_logits.append(model(input_ids=ids[:, a:a + n], position_ids=pos[:, a:a + n]).logits[0])
+        a += n
+    ref_logits = torch.cat(ref_logits, 0).float()
+    model.zero_grad()
+    (ref_logits * wsel).mean().backward()
+    ref_grad = model.model.layers[0].self_attn.q_proj.weight.grad.float().clone()
+    ref_grad_v = model.model.layers[0].self_attn.v_proj.weight.grad.float().clone()
+
+    assert VA.install_explicit_varlen_wrapper(model) is True
+    assert model.config._attn_implementation == VA.ATTENTION_NAME
+    model.zero_grad()
+    got = model(input_ids=ids, position_ids=pos).logits[0].float()
+    (got * wsel).mean().backward()
+    torch.cuda.synchronize()
+    assert cos(got, ref_logits) >= 0.9995
+    assert (got - ref_logits).abs().max().item() <= 0.05 * ref_logits.abs().max().item()
+    assert cos(model.model.layers[0].self_attn.q_proj.weight.grad, ref_grad) >= 0.995
+    assert cos(model.model.layers[0].self_attn.v_proj.weight.grad, ref_grad_v) >= 0.995
+
+
+def test_flash_attn_varlen_func_signature(dev):
+    import varlen_attention as VA
+    q, k, v, _ = make(96, 4, 2, 11)
+    cu = torch.tensor([0, 40, 96], dtype=torch.int32)
+    want = A.varlen_attention(q.float(), k.float(), v.float(), cu, causal=True)
+    got = VA.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev).clone(), 56, 56,
+                                    dropout_p=0.0, softmax_scale=None, causal=True)
+    assert (got.float().cpu() - want).abs().max().item() <= OUT_ATOL
+    cu2, mx = VA.prepare_from_position_ids(torch.cat([torch.arange(40), torch.arange(56)]).unsqueeze(0).to(dev))
+    assert cu2.tolist() == [0, 40, 96] and mx == 56

@@ -78,3 +78,27 @@ def test_synthetic_workloads_have_the_stated_shapes():
     assert w1.T == 4096 and w1.dtype == torch.bfloat16 and int(w1.cu_seqlens[-1]) == 4096
     assert min(w1.sample_lens) >= 2
     assert set(CONFIGS) == {"cfg0", "cfg1", "cfg2", "cfg3", "cfg4"}
+
+
+def test_varlen_attention_argument_errors_and_route():
+    """Unsupported flash-attn options raise before anything touches the GPU; a model switched to the varlen
+    attention reaches the HIP op (which refuses CPU tensors: there is no fallback)."""
+    import torch
+    import varlen_attention as VA
+    q = torch.zeros(8, 2, 128, dtype=torch.bfloat16)
+    cu = torch.tensor([0, 8], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="dropout"):
+        VA.flash_attn_varlen_func(q, q, q, cu, cu, 8, 8, dropout_p=0.1)
+    with pytest.raises(RuntimeError, match="window_size"):
+        VA.flash_attn_varlen_func(q, q, q, cu, cu, 8, 8, window_size=(128, 0))
+    with pytest.raises(RuntimeError, match="share their segments"):
+        VA.flash_attn_varlen_func(q, q, q, cu, torch.tensor([0, 4, 8], dtype=torch.int32), 8, 8)
+    with pytest.raises(RuntimeError, match="GPU"):
+        VA.flash_attn_varlen_func(q, q, q, cu, cu, 8, 8, causal=True)
+    from transformers import Qwen2Config, Qwen2ForCausalLM
+    cfg = Qwen2Config(vocab_size=64, hidden_size=256, intermediate_size=256, num_hidden_layers=1,
+                      num_attention_heads=2, num_key_value_heads=1, max_position_embeddings=64)
+    model = Qwen2ForCausalLM(cfg)
+    assert VA.install_explicit_varlen_wrapper(model) is True
+    with pytest.raises(RuntimeError, match="GPU"):
+        model(input_ids=torch.zeros(1, 6, dtype=torch.long), position_ids=torch.tensor([[0, 1, 2, 0, 1, 2]]))
