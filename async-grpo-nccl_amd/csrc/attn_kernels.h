@@ -129,7 +129,7 @@ __device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[4], fl
 // ---------------------------------------------------------------------------------------------------------
 // Forward: grid (ceil(T/128), Hq), 256 threads.
 // ---------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void varlen_attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
   char* kt = smem;
   char* vt = smem + kAttnTile;
@@ -271,7 +271,7 @@ __global__ void varlen_attn_delta_kernel(const bf16_t* dout, const bf16_t* out, 
 // ---------------------------------------------------------------------------------------------------------
 // dQ: grid (ceil(T/128), Hq), 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
 // ---------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void varlen_attn_dq_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
   char* kt = smem;
   char* vt = smem + kAttnTile;
