@@ -289,6 +289,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   const bool wave_on = wfirst < p.T;
   const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
   const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
+  const bool wave_full = wfirst + 31 < p.T;
+  const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
+  const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
 
   bf16x8_t qf[8], dof[8];
   attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
@@ -328,11 +331,17 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
           dp = FGRPO_MFMA(attn_frag(vt, 32 * mb + (lane & 31), 2 * st + h), dof[st], dp);
         }
         float ds[16];
+        if (kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min) {   // every pair of this step is visible
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
-          const float pr = (key >= lo && key <= hi) ? fast_exp2(__builtin_fmaf(s[r], c, -lse2)) : 0.f;
-          ds[r] = pr * (dp[r] - dl) * p.scale;
+          for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(__builtin_fmaf(s[r], c, -lse2)) * (dp[r] - dl) * p.scale;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int vis = (int)(key >= lo) & (int)(key <= hi);
+            const float pr = fast_exp2(vis ? __builtin_fmaf(s[r], c, -lse2) : -INFINITY);
+            ds[r] = pr * (dp[r] - dl) * p.scale;
+          }
         }
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
@@ -391,35 +400,70 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
     const bf16_t* dobase = p.dout + (long long)hq * kHD;
     const long long do_st = (long long)p.Hq * kHD;
     u32x4_t rq[4], rd[4];
+    // per-query scalars of a step travel with its rows: fetched one step ahead, never waited for inside a step
+    float n_lse = 0.f, n_dl = 0.f;
+    int n_lo = 1, n_hi = 0;
+    auto fetch_row_scalars = [&](int qb) {
+      if (threadIdx.x < kAttnBK) {
+        const int t = qb + threadIdx.x;
+        const bool ok = t < q_end;
+        n_lse = ok ? p.lse[(long long)hq * p.T + t] * kLog2e : 0.f;
+        n_dl = ok ? p.delta[(long long)hq * p.T + t] : 0.f;
+        n_lo = ok ? p.seg_start[t] : 1;
+        n_hi = ok ? (p.causal ? t : p.seg_end[t] - 1) : 0;
+      }
+    };
     attn_fetch_rows(rq, qbase, p.q_st, q_begin, q_end);
     attn_fetch_rows(rd, dobase, do_st, q_begin, q_end);
+    fetch_row_scalars(q_begin);
     for (int qb = q_begin; qb < q_end; qb += kAttnBK) {
       attn_put_rows(rq, qt);
       attn_put_rows(rd, dot);
       if (threadIdx.x < kAttnBK) {
-        const int t = qb + threadIdx.x;
-        const bool ok = t < q_end;
-        row_lse2[threadIdx.x] = ok ? p.lse[(long long)hq * p.T + t] * kLog2e : 0.f;
-        row_dl[threadIdx.x] = ok ? p.delta[(long long)hq * p.T + t] : 0.f;
-        row_lo[threadIdx.x] = ok ? p.seg_start[t] : 1;
-        row_hi[threadIdx.x] = ok ? (p.causal ? t : p.seg_end[t] - 1) : 0;
+        row_lse2[threadIdx.x] = n_lse;
+        row_dl[threadIdx.x] = n_dl;
+        row_lo[threadIdx.x] = n_lo;
+        row_hi[threadIdx.x] = n_hi;
       }
       __syncthreads();
       if (qb + kAttnBK < q_end) {
         attn_fetch_rows(rq, qbase, p.q_st, qb + kAttnBK, q_end);
         attn_fetch_rows(rd, dobase, do_st, qb + kAttnBK, q_end);
+        fetch_row_scalars(qb + kAttnBK);
       }
       if (wave_on && qb <= wq_hi && qb + kAttnBK > wq_lo) {
+        // every (query, key) pair of this step visible: all 64 queries exist, the last one's segment starts at or
+        // before the wavefront's first key, the first one sees the wavefront's last key
+        const bool all_visible = wfirst + 31 < p.T && qb + kAttnBK <= q_end && row_lo[kAttnBK - 1] <= wfirst && row_hi[0] >= wlast;
+        // LDS reads are issued a phase ahead of the MFMAs that use them (one wavefront per SIMD: nothing else
+        // would cover their latency): the row fragments of sub-block mq+1 under the dV/dK products of mq, the
+        // transposed fragments of mq under its own softmax arithmetic.
+        bf16x8_t qa[8], da[8];
+#pragma unroll
+        for (int st = 0; st < 8; ++st) {
+          qa[st] = attn_frag(qt, (lane & 31), 2 * st + h);
+          da[st] = attn_frag(dot, (lane & 31), 2 * st + h);
+        }
 #pragma unroll
         for (int mq = 0; mq < 2; ++mq) {
           f32x16_t s, dp;
 #pragma unroll
           for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int st = 0; st < 8; ++st) {
-            s = FGRPO_MFMA(attn_frag(qt, 32 * mq + (lane & 31), 2 * st + h), kf[st], s);
-            dp = FGRPO_MFMA(attn_frag(dot, 32 * mq + (lane & 31), 2 * st + h), vf[st], dp);
+            s = FGRPO_MFMA(qa[st], kf[st], s);
+            dp = FGRPO_MFMA(da[st], vf[st], dp);
           }
+          bf16x8_t fdo[2][4], fq[2][4];
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+              fdo[s2][nb] = attn_frag_tr(dot, 32 * mq + 16 * s2, 32 * nb, lane);
+              fq[s2][nb] = attn_frag_tr(qt, 32 * mq + 16 * s2, 32 * nb, lane);
+            }
+          __builtin_amdgcn_sched_barrier(0);
           float pr[16], ds[16];
 #pragma unroll
           for (int r4 = 0; r4 < 4; ++r4) {
@@ -433,21 +477,34 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int r = 4 * r4 + e;
-              const float pv = (key >= lo[e] && key <= hi[e]) ? fast_exp2(__builtin_fmaf(s[r], c, -ls[e])) : 0.f;
+              // select before the exponential: a masked pair becomes exp2(-inf) = 0 without a branch
+              const int vis = (int)all_visible | ((int)(key >= lo[e]) & (int)(key <= hi[e]));
+              const float pv = fast_exp2(vis ? __builtin_fmaf(s[r], c, -ls[e]) : -INFINITY);
               pr[r] = pv;
               ds[r] = pv * (dp[r] - dd[e]) * p.scale;
             }
           }
+          bf16x8_t pf[2], dsf[2];
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2) {
-            const bf16x8_t pf = attn_pack8(pr + 8 * s2);
-            const bf16x8_t dsf = attn_pack8(ds + 8 * s2);
+            pf[s2] = attn_pack8(pr + 8 * s2);
+            dsf[s2] = attn_pack8(ds + 8 * s2);
+          }
+          if (mq == 0) {
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-              acc_v[nb] = FGRPO_MFMA(pf, attn_frag_tr(dot, 32 * mq + 16 * s2, 32 * nb, lane), acc_v[nb]);
-              acc_k[nb] = FGRPO_MFMA(dsf, attn_frag_tr(qt, 32 * mq + 16 * s2, 32 * nb, lane), acc_k[nb]);
+            for (int st = 0; st < 8; ++st) {
+              qa[st] = attn_frag(qt, 32 + (lane & 31), 2 * st + h);
+              da[st] = attn_frag(dot, 32 + (lane & 31), 2 * st + h);
             }
           }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+              acc_v[nb] = FGRPO_MFMA(pf[s2], fdo[s2][nb], acc_v[nb]);
+              acc_k[nb] = FGRPO_MFMA(dsf[s2], fq[s2][nb], acc_k[nb]);
+            }
         }
       }
       __syncthreads();

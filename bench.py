@@ -69,6 +69,67 @@ def cpu_baseline(name: str, cfg_chunk, seed: int):
                       f"fp32 math on bf16-rounded inputs, best of 2; tokens/s is linear in tokens"}
 
 
+def attention_line(args):
+    """One layer of packed variable-length attention (forward + backward) at the packing of the benchmark
+    micro-batch: T tokens in segments of 128..1024, 12 query heads over 2 K/V heads, head dimension 128
+    (the attention shape of the 1.5B model).  Algorithmic flops count the visible (query, key) pairs only:
+    forward 4*D per pair and head, backward 10*D (recomputing the scores is not counted)."""
+    import torch
+    from fgrpo import ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    T, Hq, Hkv, D = 32768, 12, 2, 128
+    g = torch.Generator().manual_seed(args.seed)
+    lens = []
+    while sum(lens) < T:
+        lens.append(int(torch.randint(128, 1025, (1,), generator=g)))
+    lens[-1] -= sum(lens) - T
+    cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+    q = torch.randn(T, Hq, D, generator=g).bfloat16().to(dev)
+    k = torch.randn(T, Hkv, D, generator=g).bfloat16().to(dev)
+    v = torch.randn(T, Hkv, D, generator=g).bfloat16().to(dev)
+    do = torch.randn(T, Hq, D, generator=g).bfloat16().to(dev)
+    pairs = sum(n * (n + 1) // 2 for n in lens)
+    f_fwd = 4.0 * D * Hq * pairs
+
+    def step():
+        out, lse = ops.varlen_attn_fwd(q, k, v, cu)
+        return ops.varlen_attn_bwd(do, q, k, v, out, lse, cu)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    t_f = t_b = 0.0
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ev[0].record()
+        out, lse = ops.varlen_attn_fwd(q, k, v, cu)
+        ev[1].record()
+        ops.varlen_attn_bwd(do, q, k, v, out, lse, cu)
+        ev[2].record()
+        torch.cuda.synchronize()
+        t_f += ev[0].elapsed_time(ev[1])
+        t_b += ev[1].elapsed_time(ev[2])
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    t_f /= args.steps
+    t_b /= args.steps
+    achieved = f_fwd / (t_f * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "packed tokens/sec of one layer's variable-length attention fwd+bwd (Qwen2.5-1.5B heads); MFMA % peak",
+        "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"attention: T={T} packed tokens in {len(lens)} segments of 128..1024, Hq={Hq}, Hkv={Hkv}, "
+                               f"D={D}, causal, forward + backward", "tokens": T, "segments": len(lens)},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "varlen_attn_fwd_kernel",
+                     "kernel_ms": t_f, "algorithmic_flops_per_launch": f_fwd},
+        "backward": {"ms": t_b, "algorithmic_flops": 2.5 * f_fwd, "achieved": 2.5 * f_fwd / (t_b * 1e-3) / 1e12,
+                     "frac": 2.5 * f_fwd / (t_b * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -79,11 +140,16 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed steps, run one 1 GiB device copy (reference point for traffic counters)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--attention", action="store_true",
+                    help="time the packed attention kernels instead (prints their own JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path shards by micro-batch, one per GPU); "
               "--gpus must be 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.attention:
+        return attention_line(args)
 
     import torch
     import grpo_loss as G
