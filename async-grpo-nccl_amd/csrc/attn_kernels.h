@@ -54,20 +54,39 @@ typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int attn_swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
-// K-contiguous fragment: the 8 values [row][8*chunk .. 8*chunk+7]
-__device__ __forceinline__ bf16x8_t attn_frag(const char* tile, int row, int chunk) {
-  return *(const bf16x8_t*)(tile + row * kAttnRowB + ((chunk ^ attn_swz(row)) << 4));
+// Per-lane LDS byte offsets of the fragment reads, computed once: everything that varies inside the loops
+// (tile, 32-row block, 16-row k block) is a compile-time offset added to one of these sixteen values.
+struct AttnLane {
+  int rowc[8];    // K-contiguous fragment of row lane%32: chunk 2*st + lane/32, swizzled
+  int tr[4][2];   // K-major fragment, column block nb: the two transposing reads (k rows 4h + j/4 and + 8)
+};
+__device__ __forceinline__ AttnLane attn_lane(int lane) {
+  AttnLane L;
+  const int h = lane >> 5, g1 = (lane >> 4) & 1, j = lane & 15, r = lane & 31;
+#pragma unroll
+  for (int st = 0; st < 8; ++st) L.rowc[st] = r * kAttnRowB + (((2 * st + h) ^ attn_swz(r)) << 4);
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int rd = 0; rd < 2; ++rd) {
+      const int row = 4 * h + (j >> 2) + 8 * rd;               // + kbase (a multiple of 16: same swizzle)
+      const int chunk = 4 * nb + 2 * g1 + ((j & 3) >> 1);
+      L.tr[nb][rd] = row * kAttnRowB + ((chunk ^ attn_swz(row)) << 4) + 8 * (j & 1);
+    }
+  return L;
 }
 
-// K-major fragment: lane (n = lane%32, h = lane/32) receives Tile[kbase + 4h + 8*(j/4) + j%4][col0 + n] for the
-// eight slots j = 0..7 (kbase a multiple of 16, col0 of 32) - the key order in which a result accumulator
-// hands its values to the next MFMA.
-__device__ __forceinline__ bf16x8_t attn_frag_tr(const char* tile, int kbase, int col0, int lane) {
-  const int h = lane >> 5, g1 = (lane >> 4) & 1, j = lane & 15;
-  const int chunk = (col0 >> 3) + 2 * g1 + ((j & 3) >> 1);
-  const int r0 = kbase + 4 * h + (j >> 2), r1 = r0 + 8;
-  const char* p0 = tile + r0 * kAttnRowB + ((chunk ^ attn_swz(r0)) << 4) + 8 * (j & 1);
-  const char* p1 = tile + r1 * kAttnRowB + ((chunk ^ attn_swz(r1)) << 4) + 8 * (j & 1);
+// K-contiguous fragment: the 8 values [32*blk + lane%32][16*st + 8*(lane/32) .. +7]
+__device__ __forceinline__ bf16x8_t attn_frag(const char* tile, const AttnLane& L, int blk, int st) {
+  return *(const bf16x8_t*)(tile + L.rowc[st] + blk * 32 * kAttnRowB);
+}
+
+// K-major fragment: lane (n = lane%32, h = lane/32) receives Tile[kbase + 4h + 8*(j/4) + j%4][32*nb + n] for the
+// eight slots j = 0..7 (kbase a multiple of 16) - the key order in which a result accumulator hands its values
+// to the next MFMA.
+__device__ __forceinline__ bf16x8_t attn_frag_tr(const char* tile, const AttnLane& L, int kbase, int nb) {
+  const char* p0 = tile + L.tr[nb][0] + kbase * kAttnRowB;
+  const char* p1 = tile + L.tr[nb][1] + kbase * kAttnRowB;
   const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p0));
   const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p1));
   typedef short i16x8_t __attribute__((ext_vector_type(8)));
@@ -81,15 +100,29 @@ __device__ __forceinline__ bf16x8_t attn_pack8(const float* x) {
   return __builtin_bit_cast(bf16x8_t, v);
 }
 
-// 64 rows x 256 bytes of one head: global -> registers (rows >= row_end read as zero) ...
-__device__ __forceinline__ void attn_fetch_rows(u32x4_t (&r)[4], const bf16_t* base, long long st, int row0, int row_end) {
+// 64 rows x 256 bytes of one head: global -> registers.  Buffer loads over a descriptor that starts at row `row0`
+// (wavefront-uniform) and ends with row `row_end - 1`: rows from row_end on read as zero, and a load costs one
+// instruction - the lane's byte offset inside the slab is a constant computed once per kernel.
+struct AttnFetch {
+  uint32_t off[4];
+};
+__device__ __forceinline__ AttnFetch attn_fetch_init(long long st) {
+  AttnFetch f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int c = threadIdx.x + 256 * i;
-    const int row = row0 + (c >> 4);
-    const u32x4_t z = {0u, 0u, 0u, 0u};
-    r[i] = (row >= 0 && row < row_end) ? *(const u32x4_t*)(base + (long long)row * st + (c & 15) * 8) : z;
+    f.off[i] = (uint32_t)(((long long)(c >> 4) * st + (c & 15) * 8) * 2);
   }
+  return f;
+}
+__device__ __forceinline__ void attn_fetch_rows(u32x4_t (&r)[4], const AttnFetch& f, const bf16_t* base, long long st, int row0,
+                                                int row_end) {
+  const long long rows = (long long)row_end - row0;
+  long long bytes = rows > 0 ? (rows - 1) * st * 2 + kAttnRowB : 0;
+  if (bytes > 0xffffffffLL) bytes = 0xffffffffLL;
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(base + (long long)row0 * st, (uint32_t)bytes);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)f.off[i], 0, 0));
 }
 // ... and registers -> swizzled LDS tile
 __device__ __forceinline__ void attn_put_rows(const u32x4_t (&r)[4], char* tile) {
@@ -134,6 +167,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   char* kt = smem;
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
+  const AttnLane L = attn_lane(lane);
   const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
   const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
   const int tq = q0 + 32 * wave + (lane & 31);
@@ -141,8 +175,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   const int lo = valid ? p.seg_start[tq] : 1;
   const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
   const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
-  const int k_begin = p.seg_start[q0];
-  const int k_end = p.causal ? last + 1 : p.seg_end[last];
+  const int k_begin = __builtin_amdgcn_readfirstlane(p.seg_start[q0]);          // wavefront-uniform loop bounds
+  const int k_end = __builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]);
   // this wavefront's own key range (whole steps outside it are skipped)
   const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
   const bool wave_on = wfirst < p.T;
@@ -167,15 +201,16 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
   const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
   u32x4_t rk[4], rv[4];
-  attn_fetch_rows(rk, kbase, p.k_st, k_begin, k_end);
-  attn_fetch_rows(rv, vbase, p.v_st, k_begin, k_end);
+  const AttnFetch fk = attn_fetch_init(p.k_st), fv = attn_fetch_init(p.v_st);
+  attn_fetch_rows(rk, fk, kbase, p.k_st, k_begin, k_end);
+  attn_fetch_rows(rv, fv, vbase, p.v_st, k_begin, k_end);
   for (int kb = k_begin; kb < k_end; kb += kAttnBK) {
     attn_put_rows(rk, kt);
     attn_put_rows(rv, vt);
     __syncthreads();
     if (kb + kAttnBK < k_end) {   // next step's rows travel while this one is computed
-      attn_fetch_rows(rk, kbase, p.k_st, kb + kAttnBK, k_end);
-      attn_fetch_rows(rv, vbase, p.v_st, kb + kAttnBK, k_end);
+      attn_fetch_rows(rk, fk, kbase, p.k_st, kb + kAttnBK, k_end);
+      attn_fetch_rows(rv, fv, vbase, p.v_st, kb + kAttnBK, k_end);
     }
     if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
       f32x16_t s[2];
@@ -184,7 +219,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[mb][r] = 0.f;
 #pragma unroll
-        for (int st = 0; st < 8; ++st) s[mb] = FGRPO_MFMA(attn_frag(kt, 32 * mb + (lane & 31), 2 * st + h), qf[st], s[mb]);
+        for (int st = 0; st < 8; ++st) s[mb] = FGRPO_MFMA(attn_frag(kt, L, mb, st), qf[st], s[mb]);
       }
       float mx = -INFINITY;
       if (kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min) {   // every pair of this step is visible
@@ -233,7 +268,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
           const bf16x8_t pf = attn_pack8(tmp);
 #pragma unroll
           for (int db = 0; db < 4; ++db)
-            acc_o[db] = FGRPO_MFMA(attn_frag_tr(vt, 32 * mb + 16 * s2, 32 * db, lane), pf, acc_o[db]);
+            acc_o[db] = FGRPO_MFMA(attn_frag_tr(vt, L, 32 * mb + 16 * s2, db), pf, acc_o[db]);
         }
     }
     __syncthreads();
@@ -276,6 +311,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   char* kt = smem;
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
+  const AttnLane L = attn_lane(lane);
   const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
   const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
   const int tq = q0 + 32 * wave + (lane & 31);
@@ -283,8 +319,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   const int lo = valid ? p.seg_start[tq] : 1;
   const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
   const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
-  const int k_begin = p.seg_start[q0];
-  const int k_end = p.causal ? last + 1 : p.seg_end[last];
+  const int k_begin = __builtin_amdgcn_readfirstlane(p.seg_start[q0]);          // wavefront-uniform loop bounds
+  const int k_end = __builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]);
   const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
   const bool wave_on = wfirst < p.T;
   const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
@@ -309,15 +345,16 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
   const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
   u32x4_t rk[4], rv[4];
-  attn_fetch_rows(rk, kbase, p.k_st, k_begin, k_end);
-  attn_fetch_rows(rv, vbase, p.v_st, k_begin, k_end);
+  const AttnFetch fk = attn_fetch_init(p.k_st), fv = attn_fetch_init(p.v_st);
+  attn_fetch_rows(rk, fk, kbase, p.k_st, k_begin, k_end);
+  attn_fetch_rows(rv, fv, vbase, p.v_st, k_begin, k_end);
   for (int kb = k_begin; kb < k_end; kb += kAttnBK) {
     attn_put_rows(rk, kt);
     attn_put_rows(rv, vt);
     __syncthreads();
     if (kb + kAttnBK < k_end) {
-      attn_fetch_rows(rk, kbase, p.k_st, kb + kAttnBK, k_end);
-      attn_fetch_rows(rv, vbase, p.v_st, kb + kAttnBK, k_end);
+      attn_fetch_rows(rk, fk, kbase, p.k_st, kb + kAttnBK, k_end);
+      attn_fetch_rows(rv, fv, vbase, p.v_st, kb + kAttnBK, k_end);
     }
     if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
 #pragma unroll
@@ -327,8 +364,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
         for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
 #pragma unroll
         for (int st = 0; st < 8; ++st) {
-          s = FGRPO_MFMA(attn_frag(kt, 32 * mb + (lane & 31), 2 * st + h), qf[st], s);
-          dp = FGRPO_MFMA(attn_frag(vt, 32 * mb + (lane & 31), 2 * st + h), dof[st], dp);
+          s = FGRPO_MFMA(attn_frag(kt, L, mb, st), qf[st], s);
+          dp = FGRPO_MFMA(attn_frag(vt, L, mb, st), dof[st], dp);
         }
         float ds[16];
         if (kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min) {   // every pair of this step is visible
@@ -348,7 +385,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
           const bf16x8_t dsf = attn_pack8(ds + 8 * s2);
 #pragma unroll
           for (int db = 0; db < 4; ++db)
-            acc[db] = FGRPO_MFMA(attn_frag_tr(kt, 32 * mb + 16 * s2, 32 * db, lane), dsf, acc[db]);
+            acc[db] = FGRPO_MFMA(attn_frag_tr(kt, L, 32 * mb + 16 * s2, db), dsf, acc[db]);
         }
       }
     }
@@ -370,14 +407,15 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
   char* qt = smem;
   char* dot = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
+  const AttnLane L = attn_lane(lane);
   const int hkv = blockIdx.y, G = p.Hq / p.Hkv;
   const int k0 = blockIdx.x * kAttnBQ;
   const int key = k0 + 32 * wave + (lane & 31);
   const bool valid = key < p.T;
   const int last = (k0 + kAttnBQ - 1 < p.T ? k0 + kAttnBQ - 1 : p.T - 1);
   // queries that can see a key of this tile
-  const int q_begin = p.causal ? k0 : p.seg_start[k0];
-  const int q_end = p.seg_end[last];
+  const int q_begin = __builtin_amdgcn_readfirstlane(p.causal ? k0 : p.seg_start[k0]);   // wavefront-uniform loop bounds
+  const int q_end = __builtin_amdgcn_readfirstlane(p.seg_end[last]);
   const int wfirst = k0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
   const bool wave_on = wfirst < p.T;
   const int wq_lo = wave_on ? (p.causal ? wfirst : p.seg_start[wfirst]) : 1;   // first / last query of interest
@@ -394,6 +432,7 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc_k[nb][r] = acc_v[nb][r] = 0.f;
 
+  const AttnFetch fq_ = attn_fetch_init(p.q_st), fd_ = attn_fetch_init((long long)p.Hq * kHD);
   for (int g = 0; g < G; ++g) {
     const int hq = hkv * G + g;
     const bf16_t* qbase = p.q + (long long)hq * p.q_sh;
@@ -413,8 +452,8 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
         n_hi = ok ? (p.causal ? t : p.seg_end[t] - 1) : 0;
       }
     };
-    attn_fetch_rows(rq, qbase, p.q_st, q_begin, q_end);
-    attn_fetch_rows(rd, dobase, do_st, q_begin, q_end);
+    attn_fetch_rows(rq, fq_, qbase, p.q_st, q_begin, q_end);
+    attn_fetch_rows(rd, fd_, dobase, do_st, q_begin, q_end);
     fetch_row_scalars(q_begin);
     for (int qb = q_begin; qb < q_end; qb += kAttnBK) {
       attn_put_rows(rq, qt);
@@ -427,8 +466,8 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
       }
       __syncthreads();
       if (qb + kAttnBK < q_end) {
-        attn_fetch_rows(rq, qbase, p.q_st, qb + kAttnBK, q_end);
-        attn_fetch_rows(rd, dobase, do_st, qb + kAttnBK, q_end);
+        attn_fetch_rows(rq, fq_, qbase, p.q_st, qb + kAttnBK, q_end);
+        attn_fetch_rows(rd, fd_, dobase, do_st, qb + kAttnBK, q_end);
         fetch_row_scalars(qb + kAttnBK);
       }
       if (wave_on && qb <= wq_hi && qb + kAttnBK > wq_lo) {
@@ -441,8 +480,8 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
         bf16x8_t qa[8], da[8];
 #pragma unroll
         for (int st = 0; st < 8; ++st) {
-          qa[st] = attn_frag(qt, (lane & 31), 2 * st + h);
-          da[st] = attn_frag(dot, (lane & 31), 2 * st + h);
+          qa[st] = attn_frag(qt, L, 0, st);
+          da[st] = attn_frag(dot, L, 0, st);
         }
 #pragma unroll
         for (int mq = 0; mq < 2; ++mq) {
@@ -460,8 +499,8 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
           for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
-              fdo[s2][nb] = attn_frag_tr(dot, 32 * mq + 16 * s2, 32 * nb, lane);
-              fq[s2][nb] = attn_frag_tr(qt, 32 * mq + 16 * s2, 32 * nb, lane);
+              fdo[s2][nb] = attn_frag_tr(dot, L, 32 * mq + 16 * s2, nb);
+              fq[s2][nb] = attn_frag_tr(qt, L, 32 * mq + 16 * s2, nb);
             }
           __builtin_amdgcn_sched_barrier(0);
           float pr[16], ds[16];
@@ -493,8 +532,8 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
           if (mq == 0) {
 #pragma unroll
             for (int st = 0; st < 8; ++st) {
-              qa[st] = attn_frag(qt, 32 + (lane & 31), 2 * st + h);
-              da[st] = attn_frag(dot, 32 + (lane & 31), 2 * st + h);
+              qa[st] = attn_frag(qt, L, 1, st);
+              da[st] = attn_frag(dot, L, 1, st);
             }
           }
           __builtin_amdgcn_sched_barrier(0);

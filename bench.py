@@ -78,12 +78,15 @@ def attention_line(args):
     from fgrpo import ops
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    T, Hq, Hkv, D = 32768, 12, 2, 128
+    T, D = 32768, 128
     g = torch.Generator().manual_seed(args.seed)
-    lens = []
-    while sum(lens) < T:
-        lens.append(int(torch.randint(128, 1025, (1,), generator=g)))
-    lens[-1] -= sum(lens) - T
+    if args.attention_shape == "long":      # the 7B model's heads on four 8192-token samples
+        Hq, Hkv, lens = 28, 4, [8192] * 4
+    else:                                   # the 1.5B model's heads on the benchmark packing
+        Hq, Hkv, lens = 12, 2, []
+        while sum(lens) < T:
+            lens.append(int(torch.randint(128, 1025, (1,), generator=g)))
+        lens[-1] -= sum(lens) - T
     cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
     q = torch.randn(T, Hq, D, generator=g).bfloat16().to(dev)
     k = torch.randn(T, Hkv, D, generator=g).bfloat16().to(dev)
@@ -116,11 +119,11 @@ def attention_line(args):
     t_b /= args.steps
     achieved = f_fwd / (t_f * 1e-3) / 1e12
     print(json.dumps({
-        "metric": "packed tokens/sec of one layer's variable-length attention fwd+bwd (Qwen2.5-1.5B heads); MFMA % peak",
+        "metric": "packed tokens/sec of one layer's variable-length attention fwd+bwd; MFMA % peak",
         "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"attention: T={T} packed tokens in {len(lens)} segments of 128..1024, Hq={Hq}, Hkv={Hkv}, "
+        "config": {"workload": f"attention: T={T} packed tokens in {len(lens)} segments of {min(lens)}..{max(lens)}, Hq={Hq}, Hkv={Hkv}, "
                                f"D={D}, causal, forward + backward", "tokens": T, "segments": len(lens)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "varlen_attn_fwd_kernel",
@@ -142,6 +145,7 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--attention", action="store_true",
                     help="time the packed attention kernels instead (prints their own JSON line)")
+    ap.add_argument("--attention-shape", choices=["cfg1", "long"], default="cfg1")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path shards by micro-batch, one per GPU); "
