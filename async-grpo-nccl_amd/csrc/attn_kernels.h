@@ -19,6 +19,12 @@
 //    dV = P^T dO and dK = dS^T Q products from registers in the same way.
 // LDS tiles are [row][128] bf16 with the 16-byte chunk index XOR ((row&3)<<2 | (row>>2)&3): conflict-free both
 // for 16-byte row reads (16 consecutive rows, one chunk) and for the transposing reads (4 consecutive rows x 64 B).
+// Tiles travel global -> registers (bounds-checked buffer loads, issued one step ahead) -> LDS; masks are applied
+// only on steps that can hold a masked pair, and without branches (select before the exponential).
+// Registers: the forward and dQ kernels fit 256 registers and run two wavefronts per SIMD, which is what overlaps
+// one wavefront's softmax arithmetic with the other's MFMAs.  The dK/dV kernel holds two accumulator sets
+// (128 registers) plus its K and V operands and runs one wavefront per SIMD; splitting it into a dV and a dK
+// launch (two wavefronts per SIMD each, S computed twice) measured slower, as did a second LDS buffer.
 #pragma once
 #include "lmhead_kernels.h"
 
