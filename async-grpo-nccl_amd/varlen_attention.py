@@ -18,6 +18,7 @@ There is no fallback: inputs the kernels do not cover (dropout, sliding windows,
 dimensions other than 128, CPU tensors) raise."""
 from __future__ import annotations
 
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -26,16 +27,18 @@ from fgrpo import ops
 
 ATTENTION_NAME = "fgrpo_varlen"
 
-_cu_cache = {"key": None, "value": None}
+# (weak reference to the position_ids tensor, its version counter, result) of the last call
+_cu_cache = {"ref": None, "version": None, "value": None}
 
 
 def prepare_from_position_ids(position_ids: torch.Tensor) -> Tuple[torch.Tensor, int]:
     """``(cu_seqlens int32 [n+1], max_seqlen)`` for ``position_ids`` of shape ``[B, L]`` (or ``[L]``): a segment
     starts wherever the position is 0 and at the start of every row; the last entry is ``B * L``.  Follows
-    reference ``gpu_process_worker.py:239-252``.  The result is remembered for the tensor it was computed
-    from, so that the layers of one forward pass pay for it once."""
-    key = (position_ids.data_ptr(), tuple(position_ids.shape), position_ids._version, position_ids.device)
-    if _cu_cache["key"] == key:
+    reference ``gpu_process_worker.py:239-252``.  The result is remembered for the tensor OBJECT it was computed
+    from (weak reference + version counter; an address would be reused by the next batch), so that the layers of
+    one forward pass pay for it once."""
+    ref = _cu_cache["ref"]
+    if ref is not None and ref() is position_ids and _cu_cache["version"] == position_ids._version:
         return _cu_cache["value"]
     pos = position_ids if position_ids.dim() == 2 else position_ids.reshape(1, -1)
     if pos.shape[0] > 1:                       # a row start is a boundary whatever its first position says
@@ -45,7 +48,7 @@ def prepare_from_position_ids(position_ids: torch.Tensor) -> Tuple[torch.Tensor,
     if int(cu[0].item()) != 0:                 # tokens before the first reset form a segment of their own
         cu = torch.cat([torch.zeros(1, dtype=torch.int32, device=cu.device), cu])
     max_seqlen = int((cu[1:] - cu[:-1]).max().item())
-    _cu_cache["key"], _cu_cache["value"] = key, (cu, max_seqlen)
+    _cu_cache["ref"], _cu_cache["version"], _cu_cache["value"] = weakref.ref(position_ids), position_ids._version, (cu, max_seqlen)
     return cu, max_seqlen
 
 

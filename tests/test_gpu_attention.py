@@ -223,8 +223,17 @@ def test_flash_attn_varlen_func_signature(dev):
     got = VA.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev).clone(), 56, 56,
                                     dropout_p=0.0, softmax_scale=None, causal=True)
     assert (got.float().cpu() - want).abs().max().item() <= OUT_ATOL
-    cu2, mx = VA.prepare_from_position_ids(torch.cat([torch.arange(40), torch.arange(56)]).unsqueeze(0).to(dev))
+    pos = torch.cat([torch.arange(40), torch.arange(56)]).unsqueeze(0).to(dev)
+    cu2, mx = VA.prepare_from_position_ids(pos)
     assert cu2.tolist() == [0, 40, 96] and mx == 56
+    assert VA.prepare_from_position_ids(pos)[0] is cu2                     # same tensor object: remembered
+    ptr = pos.data_ptr()
+    del pos
+    pos = torch.cat([torch.arange(10), torch.arange(86)]).unsqueeze(0).to(dev)   # typically lands on the same address
+    cu3, mx3 = VA.prepare_from_position_ids(pos)
+    assert cu3.tolist() == [0, 10, 96] and mx3 == 86, (ptr == pos.data_ptr())
+    pos[0, 50] = 0                                                          # in-place edit bumps the version
+    assert VA.prepare_from_position_ids(pos)[0].tolist() == [0, 10, 50, 96]
 
 
 def test_workers_on_a_transformers_model_end_to_end(dev):
