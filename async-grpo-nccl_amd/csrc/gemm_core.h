@@ -301,8 +301,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 //   s_waitcnt lgkmcnt(n) itself (LDS operations return in order).
 // The fragments of the following sub-step are requested between the MFMA row groups of the current one, in the
 // order a0, b0 .. b(TN-1), a1 .. a(TM-1) (row group 0 needs a0 and every b), so that the LDS sees a steady
-// trickle of reads next to the direct-to-LDS stream instead of a burst per sub-step.
-constexpr bool kTrickleReads = true;   // false: all fragments of a sub-step requested in one burst (measured equal or slower)
+// trickle of reads next to the direct-to-LDS stream instead of a burst per sub-step (a burst measured equal or
+// slower).
 template <int N>
 __device__ __forceinline__ void wait_lgkm() {
   static_assert(N >= 0, "wait count");
@@ -318,7 +318,7 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
   constexpr int NSLOT = kLoadPhases * TM;         // MFMA groups over which one step's loads are spread
   // fragment order and bookkeeping (all compile time)
   struct Ord {
-    static constexpr int cum(int i) { return kTrickleReads ? (i * NR + TM - 1) / TM : (i > 0 ? NR : 0); }  // entries requested before row group i ends.. starts
+    static constexpr int cum(int i) { return (i * NR + TM - 1) / TM; }  // entries requested before row group i ends.. starts
     static constexpr int instrs(int n) {              // LDS instructions of the first n entries
       int c = 0;
       for (int e = 0; e < n; ++e) c += (e == 0 || e > TN) ? RA : RB;
@@ -379,39 +379,42 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
       // phase of the load spreading this sub-step belongs to: 0 = last sub-step, then 1, 2 .. from the top
       constexpr int phase = last ? 0 : kk + 1;
       const bool loads_here = STEADY || (active && phase < kLoadPhases && (phase > 0 || next));
-      if constexpr (!kTrickleReads) {                 // burst: every fragment of the next sub-step up front
-        if (issuing) static_for<NR>([&](auto e) { request(src, e, std::integral_constant<int, kn>{}, std::integral_constant<int, nbuf>{}); });
-        if (issuing) wait_lgkm<Ord::instrs(NR)>(); else wait_lgkm<0>();
-      }
       __builtin_amdgcn_sched_barrier(0);
       static_for<TM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        if constexpr (kTrickleReads) {
-          if constexpr (!last) {
-            wait_lgkm<Ord::allowed(i, true)>();
-          } else {
-            if (next) wait_lgkm<Ord::allowed(i, true)>(); else wait_lgkm<Ord::allowed(i, false)>();
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
-        if constexpr (kTrickleReads) {
-          if (issuing) {
-            static_for<Ord::cum(i + 1) - Ord::cum(i)>([&](auto d) {
-              request(src, std::integral_constant<int, Ord::cum(i) + decltype(d)::value>{}, std::integral_constant<int, kn>{},
-                      std::integral_constant<int, nbuf>{});
-            });
-          }
-        }
-        if constexpr (phase < kLoadPhases) {
-          if (loads_here) {
-            static_for<LPT>([&](auto q) {
-              if constexpr (decltype(q)::value * NSLOT / LPT == phase * TM + i) issue_one(tgt, decltype(q)::value);
-            });
-          }
+        if constexpr (!last) {
+          wait_lgkm<Ord::allowed(i, true)>();
+        } else {
+          if (next) wait_lgkm<Ord::allowed(i, true)>(); else wait_lgkm<Ord::allowed(i, false)>();
         }
         __builtin_amdgcn_sched_barrier(0);
+        {
+          // the group's fragment requests and loads go BETWEEN its MFMAs (after MFMA j the extras x with
+          // x*TN/X == j): an MFMA keeps the matrix pipe busy for 32 cycles but issues in 4, so whatever is
+          // issued right behind it is free - what is issued after the last one delays the next group.
+          constexpr int R = Ord::cum(i + 1) - Ord::cum(i);
+          constexpr int slot = phase * TM + i;
+          constexpr int q_lo = (phase < kLoadPhases) ? (slot * LPT + NSLOT - 1) / NSLOT : 0;
+          constexpr int q_hi = (phase < kLoadPhases) ? ((slot + 1) * LPT + NSLOT - 1) / NSLOT : 0;   // loads q_lo .. q_hi-1
+          constexpr int X = R + (q_hi - q_lo);
+          static_for<TN>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            acc[i][j] = FGRPO_MFMA(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
+            static_for<X>([&](auto xc) {
+              constexpr int x = decltype(xc)::value;
+              if constexpr (x * TN / (X > 0 ? X : 1) == j) {
+                if constexpr (x < R) {
+                  if (issuing)
+                    request(src, std::integral_constant<int, Ord::cum(i) + x>{}, std::integral_constant<int, kn>{},
+                            std::integral_constant<int, nbuf>{});
+                } else {
+                  if (loads_here) issue_one(tgt, q_lo + (x - R));
+                }
+              }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+          });
+        }
       });
     });
     cur ^= 1;
