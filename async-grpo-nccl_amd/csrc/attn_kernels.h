@@ -376,14 +376,14 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
         float ds[16];
         if (kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min) {   // every pair of this step is visible
 #pragma unroll
-          for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(__builtin_fmaf(s[r], c, -lse2)) * (dp[r] - dl) * p.scale;
+          for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(__builtin_fmaf(s[r], c, -lse2)) * (dp[r] - dl);
         } else {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
             const int vis = (int)(key >= lo) & (int)(key <= hi);
             const float pr = fast_exp2(vis ? __builtin_fmaf(s[r], c, -lse2) : -INFINITY);
-            ds[r] = pr * (dp[r] - dl) * p.scale;
+            ds[r] = pr * (dp[r] - dl);
           }
         }
 #pragma unroll
@@ -397,7 +397,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
     }
     __syncthreads();
   }
-  if (valid) attn_store_rowmajor(acc, 1.f, p.dq + ((long long)tq * p.Hq + hq) * kHD, h);
+  if (valid) attn_store_rowmajor(acc, p.scale, p.dq + ((long long)tq * p.Hq + hq) * kHD, h);   // dS was kept / scale
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -509,24 +509,42 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
               fq[s2][nb] = attn_frag_tr(qt, L, 32 * mq + 16 * s2, nb);
             }
           __builtin_amdgcn_sched_barrier(0);
+          // P and dS / scale (the scale is applied once, to the dK accumulators, at the end)
           float pr[16], ds[16];
+          if (all_visible) {
 #pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const int row = 32 * mq + 8 * r4 + 4 * h;
-            const float4 l4 = *(const float4*)(row_lse2 + row);
-            const float4 d4 = *(const float4*)(row_dl + row);
-            const int4 lo4 = *(const int4*)(row_lo + row);
-            const int4 hi4 = *(const int4*)(row_hi + row);
-            const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
-            const int lo[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, hi[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
+            for (int r4 = 0; r4 < 4; ++r4) {
+              const int row = 32 * mq + 8 * r4 + 4 * h;
+              const float4 l4 = *(const float4*)(row_lse2 + row);
+              const float4 d4 = *(const float4*)(row_dl + row);
+              const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int r = 4 * r4 + e;
-              // select before the exponential: a masked pair becomes exp2(-inf) = 0 without a branch
-              const int vis = (int)all_visible | ((int)(key >= lo[e]) & (int)(key <= hi[e]));
-              const float pv = fast_exp2(vis ? __builtin_fmaf(s[r], c, -ls[e]) : -INFINITY);
-              pr[r] = pv;
-              ds[r] = pv * (dp[r] - dd[e]) * p.scale;
+              for (int e = 0; e < 4; ++e) {
+                const int r = 4 * r4 + e;
+                const float pv = fast_exp2(__builtin_fmaf(s[r], c, -ls[e]));
+                pr[r] = pv;
+                ds[r] = pv * (dp[r] - dd[e]);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+              const int row = 32 * mq + 8 * r4 + 4 * h;
+              const float4 l4 = *(const float4*)(row_lse2 + row);
+              const float4 d4 = *(const float4*)(row_dl + row);
+              const int4 lo4 = *(const int4*)(row_lo + row);
+              const int4 hi4 = *(const int4*)(row_hi + row);
+              const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
+              const int lo[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, hi[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int r = 4 * r4 + e;
+                // select before the exponential: a masked pair becomes exp2(-inf) = 0 without a branch
+                const int vis = (int)(key >= lo[e]) & (int)(key <= hi[e]);
+                const float pv = fast_exp2(vis ? __builtin_fmaf(s[r], c, -ls[e]) : -INFINITY);
+                pr[r] = pv;
+                ds[r] = pv * (dp[r] - dd[e]);
+              }
             }
           }
           bf16x8_t pf[2], dsf[2];
@@ -563,7 +581,7 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
       const int kk = k0 + 32 * wave + 8 * (r >> 2) + 4 * h + (r & 3);
       if (kk < p.T) {
         const long long o = ((long long)kk * p.Hkv + hkv) * kHD + 32 * nb + (lane & 31);
-        p.dk[o] = f32_to_bf16_rn(acc_k[nb][r]);
+        p.dk[o] = f32_to_bf16_rn(acc_k[nb][r] * p.scale);
         p.dv[o] = f32_to_bf16_rn(acc_v[nb][r]);
       }
     }
