@@ -260,10 +260,12 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
         }
       l_run = l_run * alpha + sum;
       m_run = m_new;
+      if (__any(alpha != 1.f)) {      // once the running maxima have settled no lane rescales any more
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc_o[db][r] *= alpha;
+          for (int r = 0; r < 16; ++r) acc_o[db][r] *= alpha;
+      }
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
