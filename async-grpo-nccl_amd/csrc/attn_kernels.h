@@ -482,27 +482,21 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
         // every (query, key) pair of this step visible: all 64 queries exist, the last one's segment starts at or
         // before the wavefront's first key, the first one sees the wavefront's last key
         const bool all_visible = wfirst + 31 < p.T && qb + kAttnBK <= q_end && row_lo[kAttnBK - 1] <= wfirst && row_hi[0] >= wlast;
-        // LDS reads are issued a phase ahead of the MFMAs that use them (one wavefront per SIMD: nothing else
-        // would cover their latency): the row fragments of sub-block mq+1 under the dV/dK products of mq, the
-        // transposed fragments of mq under its own softmax arithmetic.
-        bf16x8_t qa[8], da[8];
-#pragma unroll
-        for (int st = 0; st < 8; ++st) {
-          qa[st] = attn_frag(qt, L, 0, st);
-          da[st] = attn_frag(dot, L, 0, st);
-        }
-#pragma unroll
-        for (int mq = 0; mq < 2; ++mq) {
-          f32x16_t s, dp;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
-          __builtin_amdgcn_sched_barrier(0);
+        // One wavefront per SIMD: only this wavefront's own instruction order can overlap the softmax arithmetic
+        // with the matrix pipe (an MFMA occupies the pipe for 32 cycles but issues in 4).  The step's two 32-query
+        // sub-blocks are therefore software-pipelined by hand, one MFMA per softmax element:
+        //   S,dP(0) | S,dP(1) + softmax(0) | dV,dK(0) + softmax(1) | dV,dK(1)
+        // and LDS fragments are requested a phase before the MFMAs that use them.
+        bf16x8_t qa[8], da[8], fdo[2][4], fq[2][4], pf[2][2], dsf[2][2];
+        f32x16_t s[2], dp[2];
+        auto load_rows = [&](int mq) {
 #pragma unroll
           for (int st = 0; st < 8; ++st) {
-            s = FGRPO_MFMA(qa[st], kf[st], s);
-            dp = FGRPO_MFMA(da[st], vf[st], dp);
+            qa[st] = attn_frag(qt, L, mq, st);
+            da[st] = attn_frag(dot, L, mq, st);
           }
-          bf16x8_t fdo[2][4], fq[2][4];
+        };
+        auto load_tr = [&](int mq) {
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
@@ -510,67 +504,99 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
               fdo[s2][nb] = attn_frag_tr(dot, L, 32 * mq + 16 * s2, nb);
               fq[s2][nb] = attn_frag_tr(qt, L, 32 * mq + 16 * s2, nb);
             }
-          __builtin_amdgcn_sched_barrier(0);
-          // P and dS / scale (the scale is applied once, to the dK accumulators, at the end)
-          float pr[16], ds[16];
-          if (all_visible) {
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-              const int row = 32 * mq + 8 * r4 + 4 * h;
-              const float4 l4 = *(const float4*)(row_lse2 + row);
-              const float4 d4 = *(const float4*)(row_dl + row);
-              const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int r = 4 * r4 + e;
-                const float pv = fast_exp2(__builtin_fmaf(s[r], c, -ls[e]));
-                pr[r] = pv;
-                ds[r] = pv * (dp[r] - dd[e]);
-              }
-            }
-          } else {
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-              const int row = 32 * mq + 8 * r4 + 4 * h;
-              const float4 l4 = *(const float4*)(row_lse2 + row);
-              const float4 d4 = *(const float4*)(row_dl + row);
-              const int4 lo4 = *(const int4*)(row_lo + row);
-              const int4 hi4 = *(const int4*)(row_hi + row);
-              const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
-              const int lo[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, hi[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int r = 4 * r4 + e;
-                // select before the exponential: a masked pair becomes exp2(-inf) = 0 without a branch
-                const int vis = (int)(key >= lo[e]) & (int)(key <= hi[e]);
-                const float pv = fast_exp2(vis ? __builtin_fmaf(s[r], c, -ls[e]) : -INFINITY);
-                pr[r] = pv;
-                ds[r] = pv * (dp[r] - dd[e]);
-              }
+        };
+        auto score_mfma = [&](int mq, int j) {      // MFMA j of 16: two chains of eight
+          if (j & 1) dp[mq] = FGRPO_MFMA(da[j >> 1], vf[j >> 1], dp[mq]);
+          else s[mq] = FGRPO_MFMA(qa[j >> 1], kf[j >> 1], s[mq]);
+        };
+        auto grad_mfma = [&](int mq, int j) {       // MFMA j of 16: eight accumulators
+          const int s2 = j >> 3, nb = (j >> 1) & 3;
+          if (j & 1) acc_k[nb] = FGRPO_MFMA(dsf[mq][s2], fq[s2][nb], acc_k[nb]);
+          else acc_v[nb] = FGRPO_MFMA(pf[mq][s2], fdo[s2][nb], acc_v[nb]);
+        };
+        // softmax element r of sub-block mq: P and dS / scale (the scale is applied once, to the dK accumulators)
+        float pr[16], ds[16];
+        float4 l4, d4;
+        int4 lo4 = {0, 0, 0, 0}, hi4 = {0, 0, 0, 0};
+        auto element = [&](int mq, int r, bool masked) {
+          if ((r & 3) == 0) {                       // the four queries of this register group
+            const int row = 32 * mq + 8 * (r >> 2) + 4 * h;
+            l4 = *(const float4*)(row_lse2 + row);
+            d4 = *(const float4*)(row_dl + row);
+            if (masked) {
+              lo4 = *(const int4*)(row_lo + row);
+              hi4 = *(const int4*)(row_hi + row);
             }
           }
-          bf16x8_t pf[2], dsf[2];
+          const int e = r & 3;
+          const float ls = e == 0 ? l4.x : e == 1 ? l4.y : e == 2 ? l4.z : l4.w;
+          const float dd = e == 0 ? d4.x : e == 1 ? d4.y : e == 2 ? d4.z : d4.w;
+          float x = __builtin_fmaf(s[mq][r], c, -ls);
+          if (masked) {
+            const int lo = e == 0 ? lo4.x : e == 1 ? lo4.y : e == 2 ? lo4.z : lo4.w;
+            const int hi = e == 0 ? hi4.x : e == 1 ? hi4.y : e == 2 ? hi4.z : hi4.w;
+            // select before the exponential: a masked pair becomes exp2(-inf) = 0 without a branch
+            x = ((int)(key >= lo) & (int)(key <= hi)) ? x : -INFINITY;
+          }
+          const float pv = fast_exp2(x);
+          pr[r] = pv;
+          ds[r] = pv * (dp[mq][r] - dd);
+        };
+        auto pack = [&](int mq) {
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2) {
-            pf[s2] = attn_pack8(pr + 8 * s2);
-            dsf[s2] = attn_pack8(ds + 8 * s2);
+            pf[mq][s2] = attn_pack8(pr + 8 * s2);
+            dsf[mq][s2] = attn_pack8(ds + 8 * s2);
           }
-          if (mq == 0) {
+        };
 #pragma unroll
-            for (int st = 0; st < 8; ++st) {
-              qa[st] = attn_frag(qt, L, 1, st);
-              da[st] = attn_frag(dot, L, 1, st);
-            }
+        for (int mq = 0; mq < 2; ++mq)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[mq][r] = dp[mq][r] = 0.f;
+
+        load_rows(0);
+        load_tr(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) score_mfma(0, j);
+        load_rows(1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (all_visible) {
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            score_mfma(1, j);
+            element(0, j, false);
+            __builtin_amdgcn_sched_barrier(0);
           }
+          pack(0);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2)
+          for (int j = 0; j < 16; ++j) {
+            grad_mfma(0, j);
+            element(1, j, false);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        } else {
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-              acc_v[nb] = FGRPO_MFMA(pf[s2], fdo[s2][nb], acc_v[nb]);
-              acc_k[nb] = FGRPO_MFMA(dsf[s2], fq[s2][nb], acc_k[nb]);
-            }
+          for (int j = 0; j < 16; ++j) {
+            score_mfma(1, j);
+            element(0, j, true);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          pack(0);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            grad_mfma(0, j);
+            element(1, j, true);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
+        pack(1);
+        load_tr(1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) grad_mfma(1, j);
       }
       __syncthreads();
     }
