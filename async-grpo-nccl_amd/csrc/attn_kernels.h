@@ -516,19 +516,26 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
         };
         // softmax element r of sub-block mq: P and dS / scale (the scale is applied once, to the dK accumulators)
         float pr[16], ds[16];
-        float4 l4, d4;
-        int4 lo4 = {0, 0, 0, 0}, hi4 = {0, 0, 0, 0};
-        auto element = [&](int mq, int r, bool masked) {
-          if ((r & 3) == 0) {                       // the four queries of this register group
-            const int row = 32 * mq + 8 * (r >> 2) + 4 * h;
-            l4 = *(const float4*)(row_lse2 + row);
-            d4 = *(const float4*)(row_dl + row);
-            if (masked) {
-              lo4 = *(const int4*)(row_lo + row);
-              hi4 = *(const int4*)(row_hi + row);
-            }
+        // per-query scalars of a register group (four queries), read one group ahead of their use
+        float4 l4s[2], d4s[2];
+        int4 lo4s[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}}, hi4s[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+        auto read_group = [&](int mq, int grp, bool masked) {     // -> set grp % 2
+          const int row = 32 * mq + 8 * grp + 4 * h;
+          l4s[grp & 1] = *(const float4*)(row_lse2 + row);
+          d4s[grp & 1] = *(const float4*)(row_dl + row);
+          if (masked) {
+            lo4s[grp & 1] = *(const int4*)(row_lo + row);
+            hi4s[grp & 1] = *(const int4*)(row_hi + row);
           }
-          const int e = r & 3;
+        };
+        auto element = [&](int mq, int r, bool masked) {
+          if ((r & 3) == 0) {
+            if (r + 4 < 16) read_group(mq, (r >> 2) + 1, masked);
+            else if (mq == 0) read_group(1, 0, masked);          // first group of the other sub-block
+          }
+          const int e = r & 3, st = (r >> 2) & 1;
+          const float4 l4 = l4s[st], d4 = d4s[st];
+          const int4 lo4 = lo4s[st], hi4 = hi4s[st];
           const float ls = e == 0 ? l4.x : e == 1 ? l4.y : e == 2 ? l4.z : l4.w;
           const float dd = e == 0 ? d4.x : e == 1 ? d4.y : e == 2 ? d4.z : d4.w;
           float x = __builtin_fmaf(s[mq][r], c, -ls);
@@ -556,6 +563,7 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
 
         load_rows(0);
         load_tr(0);
+        read_group(0, 0, !all_visible);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 16; ++j) score_mfma(0, j);
