@@ -23,8 +23,9 @@
 // only on steps that can hold a masked pair, and without branches (select before the exponential).
 // Registers: the forward and dQ kernels fit 256 registers and run two wavefronts per SIMD, which is what overlaps
 // one wavefront's softmax arithmetic with the other's MFMAs.  The dK/dV kernel holds two accumulator sets
-// (128 registers) plus its K and V operands and runs one wavefront per SIMD; splitting it into a dV and a dK
-// launch (two wavefronts per SIMD each, S computed twice) measured slower, as did a second LDS buffer.
+// (128 registers) plus its K and V operands and runs one wavefront per SIMD, so its step is software-pipelined
+// by hand (one MFMA per softmax element); splitting it into a dV and a dK launch (two wavefronts per SIMD each,
+// S computed twice) measured slower, as did a second LDS buffer.
 #pragma once
 #include "lmhead_kernels.h"
 
