@@ -51,7 +51,8 @@ struct AttnParams {
   float* lse;            // [Hq][T], natural log of the softmax denominator
   // backward
   const bf16_t* dout;    // [T][Hq][128] contiguous
-  const float* delta;    // [Hq][T] rowsum(dO * O)
+  float* delta;          // [Hq][T] rowsum(dO * O): written by the dQ kernel, read by the dK/dV kernel
+  const bf16_t* out_fwd; // [T][Hq][128] the forward's output (backward only)
   bf16_t* dq;            // [T][Hq][128] contiguous
   bf16_t* dk;            // [T][Hkv][128] contiguous
   bf16_t* dv;
@@ -290,30 +291,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   }
 }
 
-// delta[hq][t] = sum_d dO[t][hq][d] * O[t][hq][d]; 16 lanes per row, grid ceil(T*Hq / 16), 256 threads
-__global__ void varlen_attn_delta_kernel(const bf16_t* dout, const bf16_t* out, int T, int Hq, float* delta) {
-  const long long row = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
-  const int part = threadIdx.x & 15;
-  float a = 0.f;
-  if (row < (long long)T * Hq) {
-    const u32x4_t x = *(const u32x4_t*)(dout + row * kHD + part * 8);
-    const u32x4_t y = *(const u32x4_t*)(out + row * kHD + part * 8);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      a += __uint_as_float(x[i] << 16) * __uint_as_float(y[i] << 16);
-      a += __uint_as_float(x[i] & 0xffff0000u) * __uint_as_float(y[i] & 0xffff0000u);
-    }
-  }
-#pragma unroll
-  for (int o = 8; o >= 1; o >>= 1) a += __shfl_xor(a, o, 64);
-  if (part == 0 && row < (long long)T * Hq) {
-    const int t = (int)(row / Hq), hq = (int)(row % Hq);
-    delta[(long long)hq * T + t] = a;
-  }
-}
-
 // ---------------------------------------------------------------------------------------------------------
 // dQ: grid (ceil(T/128), Hq), 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
+// Also produces delta[hq][t] = sum_d dO[t][hq][d] * O[t][hq][d] (each lane already holds its query's dO row).
 // ---------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
@@ -342,7 +322,23 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
   attn_row_operand(dof, p.dout + ((long long)(valid ? tq : 0) * p.Hq + hq) * kHD, valid, h);
   const float lse2 = valid ? p.lse[(long long)hq * p.T + tq] * kLog2e : 0.f;
-  const float dl = valid ? p.delta[(long long)hq * p.T + tq] : 0.f;
+  // delta = rowsum(dO * O) of the lane's query: each lane half holds alternate 8-element pieces of the row
+  float dl = 0.f;
+  {
+    bf16x8_t of[8];
+    attn_row_operand(of, p.out_fwd + ((long long)(valid ? tq : 0) * p.Hq + hq) * kHD, valid, h);
+#pragma unroll
+    for (int st = 0; st < 8; ++st) {
+      const u32x4_t x = __builtin_bit_cast(u32x4_t, dof[st]), y = __builtin_bit_cast(u32x4_t, of[st]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        dl += __uint_as_float(x[i] << 16) * __uint_as_float(y[i] << 16);
+        dl += __uint_as_float(x[i] & 0xffff0000u) * __uint_as_float(y[i] & 0xffff0000u);
+      }
+    }
+    dl += attn_swap32(dl);
+    if (valid && h == 0) p.delta[(long long)hq * p.T + tq] = dl;    // for the dK/dV kernel, launched after this one
+  }
   const float c = p.scale * kLog2e;
 
   f32x16_t acc[4];

@@ -930,14 +930,11 @@ int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const 
   p.lse = const_cast<float*>(lse);
   p.dout = (const bf16_t*)dout;
   p.delta = delta_ws;
+  p.out_fwd = (const bf16_t*)out;
   p.dq = (bf16_t*)dq;
   p.dk = (bf16_t*)dk;
   p.dv = (bf16_t*)dv;
   hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
-  HIP_TRY(hipGetLastError());
-  const long long rows = (long long)T * Hq;
-  hipLaunchKernelGGL(varlen_attn_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const bf16_t*)dout,
-                     (const bf16_t*)out, T, Hq, delta_ws);
   HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(varlen_attn_dq_kernel, dim3((T + kAttnBQ - 1) / kAttnBQ, Hq), dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());
