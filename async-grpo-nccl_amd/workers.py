@@ -4,7 +4,8 @@ in the reference: ``TrainerGPUWorker.compute_gradients``
 ``LogProbGPUWorker.compute_log_probs_from_samples``
 (gpu_process_worker.py:1662-1709).  Ray, FSDP and the weight sync around them
 are not reproduced; the model is any module patched by
-``grpo_loss.make_grpo_forward``."""
+``grpo_loss.make_grpo_forward`` (``prepare_actor_module`` does what the reference does at
+load time: attention wrapper, then the forward patch)."""
 from __future__ import annotations
 
 from types import SimpleNamespace
@@ -12,8 +13,22 @@ from typing import List
 
 import torch
 
-from grpo_loss import compute_dual_clip_grpo_loss
+from grpo_loss import compute_dual_clip_grpo_loss, make_grpo_forward
 from sample_processing_utils import post_process_batch
+
+
+def prepare_actor_module(model, config=None, mode: str = "training", use_varlen_attention: bool = True):
+    """What the reference does to a freshly loaded actor before using it (gpu_process_worker.py:657-693): install the
+    packed-attention wrapper when flattened packing is used (``:657-668``), then patch ``forward`` with
+    ``make_grpo_forward`` in 'training' or 'eval' mode with the configured temperature and ``loss_chunksize``
+    (``:676-693``).  Returns the model."""
+    if use_varlen_attention:
+        from varlen_attention import install_explicit_varlen_wrapper
+        install_explicit_varlen_wrapper(model)
+    make_grpo_forward(model, temperature=float(getattr(config, "temperature", 1.0)), mode=mode,
+                      use_torch_compile=bool(getattr(config, "use_torch_compile", True)),
+                      loss_chunksize=getattr(config, "loss_chunksize", None))
+    return model
 
 
 class TrainerHarness:

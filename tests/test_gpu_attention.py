@@ -274,8 +274,9 @@ def test_workers_on_a_transformers_model_end_to_end(dev):
             lp = torch.log_softmax(logits, -1).gather(-1, lab.clamp(min=0)[:, None])[:, 0] * (lab != -100)
             want.append(lp.cpu())
 
-    assert VA.install_explicit_varlen_wrapper(model)
-    G.make_grpo_forward(model, temperature=1.0, mode="eval")
+    from workers import prepare_actor_module
+    prepare_actor_module(model, SimpleNamespace(temperature=1.0), mode="eval")
+    assert model.config._attn_implementation == VA.ATTENTION_NAME
     res = LogProbHarness(model, dev).compute_log_probs_from_samples(samples)
     for r, w_lp in zip(res, want):
         got = torch.tensor(r["logprobs"])
