@@ -1,4 +1,4 @@
-// Packed variable-length attention for gfx950 (head dimension 128, bf16 operands, fp32 softmax and accumulators):
+// Packed variable-length attention for gfx950 (head dimension 128 or 64, bf16 operands, fp32 softmax and accumulators):
 // forward with log-sum-exp output, and the backward as two kernels (dQ by query tile, dK/dV by key tile).
 // Replaces the flash-attn varlen call of the reference's packed path (gpu_process_worker.py:265-276) with the
 // K/V head repeat of its grouped-query wrapper folded into the head index (gpu_process_worker.py:154-161).
@@ -31,15 +31,14 @@
 
 namespace fgrpo {
 
-constexpr int kHD = 128;             // head dimension
+// Every kernel is a template on the head dimension HD (128 or 64): LDS rows of 2*HD bytes in HD/8 16-byte chunks,
+// HD/16 MFMA k-steps per score, HD/32 output blocks of 32 columns.
 constexpr int kAttnBQ = 128;         // tokens per work-group (32 per wavefront)
 constexpr int kAttnBK = 64;          // tokens of the other side per step
-constexpr int kAttnRowB = kHD * 2;   // bytes of one LDS row
-constexpr int kAttnTile = kAttnBK * kAttnRowB;
 
 struct AttnParams {
-  const bf16_t* q;       // [T][Hq][128] with element strides q_st (token), q_sh (head)
-  const bf16_t* k;       // [T][Hkv][128]
+  const bf16_t* q;       // [T][Hq][HD] with element strides q_st (token), q_sh (head)
+  const bf16_t* k;       // [T][Hkv][HD]
   const bf16_t* v;
   long long q_st, q_sh, k_st, k_sh, v_st, v_sh;
   const int* seg_start;  // [T] first token of the token's segment
@@ -47,54 +46,65 @@ struct AttnParams {
   int T, Hq, Hkv;
   float scale;
   int causal;
-  bf16_t* out;           // [T][Hq][128] contiguous
+  bf16_t* out;           // [T][Hq][HD] contiguous
   float* lse;            // [Hq][T], natural log of the softmax denominator
   // backward
-  const bf16_t* dout;    // [T][Hq][128] contiguous
+  const bf16_t* dout;    // [T][Hq][HD] contiguous
   float* delta;          // [Hq][T] rowsum(dO * O): written by the dQ kernel, read by the dK/dV kernel
-  const bf16_t* out_fwd; // [T][Hq][128] the forward's output (backward only)
-  bf16_t* dq;            // [T][Hq][128] contiguous
-  bf16_t* dk;            // [T][Hkv][128] contiguous
+  const bf16_t* out_fwd; // [T][Hq][HD] the forward's output (backward only)
+  bf16_t* dq;            // [T][Hq][HD] contiguous
+  bf16_t* dk;            // [T][Hkv][HD] contiguous
   bf16_t* dv;
 };
 
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ int attn_swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+// chunk-index XOR of an LDS row.  HD = 128 (16 chunks, one row = all 64 banks): (row&3)<<2 | (row>>2)&3.
+// HD = 64 (8 chunks, two rows share the banks): (row>>1&1)<<2 | (row>>2)&3.  Both are conflict-free for 16-byte
+// reads of 16 consecutive rows at one chunk and for the transposing reads (4 consecutive rows x 64 bytes).
+template <int HD>
+__device__ __forceinline__ int attn_swz(int row) {
+  static_assert(HD == 128 || HD == 64, "head dimension");
+  return HD == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+}
 
 // Per-lane LDS byte offsets of the fragment reads, computed once: everything that varies inside the loops
 // (tile, 32-row block, 16-row k block) is a compile-time offset added to one of these sixteen values.
+template <int HD>
 struct AttnLane {
-  int rowc[8];    // K-contiguous fragment of row lane%32: chunk 2*st + lane/32, swizzled
-  int tr[4][2];   // K-major fragment, column block nb: the two transposing reads (k rows 4h + j/4 and + 8)
+  int rowc[HD / 16];    // K-contiguous fragment of row lane%32: chunk 2*st + lane/32, swizzled
+  int tr[HD / 32][2];   // K-major fragment, column block nb: the two transposing reads (k rows 4h + j/4 and + 8)
 };
-__device__ __forceinline__ AttnLane attn_lane(int lane) {
-  AttnLane L;
+template <int HD>
+__device__ __forceinline__ AttnLane<HD> attn_lane(int lane) {
+  AttnLane<HD> L;
   const int h = lane >> 5, g1 = (lane >> 4) & 1, j = lane & 15, r = lane & 31;
 #pragma unroll
-  for (int st = 0; st < 8; ++st) L.rowc[st] = r * kAttnRowB + (((2 * st + h) ^ attn_swz(r)) << 4);
+  for (int st = 0; st < HD / 16; ++st) L.rowc[st] = r * (HD * 2) + (((2 * st + h) ^ attn_swz<HD>(r)) << 4);
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
+  for (int nb = 0; nb < HD / 32; ++nb)
 #pragma unroll
     for (int rd = 0; rd < 2; ++rd) {
       const int row = 4 * h + (j >> 2) + 8 * rd;               // + kbase (a multiple of 16: same swizzle)
       const int chunk = 4 * nb + 2 * g1 + ((j & 3) >> 1);
-      L.tr[nb][rd] = row * kAttnRowB + ((chunk ^ attn_swz(row)) << 4) + 8 * (j & 1);
+      L.tr[nb][rd] = row * (HD * 2) + ((chunk ^ attn_swz<HD>(row)) << 4) + 8 * (j & 1);
     }
   return L;
 }
 
 // K-contiguous fragment: the 8 values [32*blk + lane%32][16*st + 8*(lane/32) .. +7]
-__device__ __forceinline__ bf16x8_t attn_frag(const char* tile, const AttnLane& L, int blk, int st) {
-  return *(const bf16x8_t*)(tile + L.rowc[st] + blk * 32 * kAttnRowB);
+template <int HD>
+__device__ __forceinline__ bf16x8_t attn_frag(const char* tile, const AttnLane<HD>& L, int blk, int st) {
+  return *(const bf16x8_t*)(tile + L.rowc[st] + blk * 32 * (HD * 2));
 }
 
 // K-major fragment: lane (n = lane%32, h = lane/32) receives Tile[kbase + 4h + 8*(j/4) + j%4][32*nb + n] for the
 // eight slots j = 0..7 (kbase a multiple of 16) - the key order in which a result accumulator hands its values
 // to the next MFMA.
-__device__ __forceinline__ bf16x8_t attn_frag_tr(const char* tile, const AttnLane& L, int kbase, int nb) {
-  const char* p0 = tile + L.tr[nb][0] + kbase * kAttnRowB;
-  const char* p1 = tile + L.tr[nb][1] + kbase * kAttnRowB;
+template <int HD>
+__device__ __forceinline__ bf16x8_t attn_frag_tr(const char* tile, const AttnLane<HD>& L, int kbase, int nb) {
+  const char* p0 = tile + L.tr[nb][0] + kbase * (HD * 2);
+  const char* p1 = tile + L.tr[nb][1] + kbase * (HD * 2);
   const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p0));
   const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p1));
   typedef short i16x8_t __attribute__((ext_vector_type(8)));
@@ -111,41 +121,47 @@ __device__ __forceinline__ bf16x8_t attn_pack8(const float* x) {
 // 64 rows x 256 bytes of one head: global -> registers.  Buffer loads over a descriptor that starts at row `row0`
 // (wavefront-uniform) and ends with row `row_end - 1`: rows from row_end on read as zero, and a load costs one
 // instruction - the lane's byte offset inside the slab is a constant computed once per kernel.
+template <int HD>
 struct AttnFetch {
-  uint32_t off[4];
+  uint32_t off[HD / 32];      // 64 rows x HD/8 chunks over 256 threads
 };
-__device__ __forceinline__ AttnFetch attn_fetch_init(long long st) {
-  AttnFetch f;
+template <int HD>
+__device__ __forceinline__ AttnFetch<HD> attn_fetch_init(long long st) {
+  AttnFetch<HD> f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < HD / 32; ++i) {
     const int c = threadIdx.x + 256 * i;
-    f.off[i] = (uint32_t)(((long long)(c >> 4) * st + (c & 15) * 8) * 2);
+    f.off[i] = (uint32_t)(((long long)(c / (HD / 8)) * st + (c % (HD / 8)) * 8) * 2);
   }
   return f;
 }
-__device__ __forceinline__ void attn_fetch_rows(u32x4_t (&r)[4], const AttnFetch& f, const bf16_t* base, long long st, int row0,
-                                                int row_end) {
+template <int HD>
+__device__ __forceinline__ void attn_fetch_rows(u32x4_t (&r)[HD / 32], const AttnFetch<HD>& f, const bf16_t* base, long long st,
+                                                int row0, int row_end) {
   const long long rows = (long long)row_end - row0;
-  long long bytes = rows > 0 ? (rows - 1) * st * 2 + kAttnRowB : 0;
+  long long bytes = rows > 0 ? (rows - 1) * st * 2 + HD * 2 : 0;
   if (bytes > 0xffffffffLL) bytes = 0xffffffffLL;
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(base + (long long)row0 * st, (uint32_t)bytes);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) r[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)f.off[i], 0, 0));
+  for (int i = 0; i < HD / 32; ++i)
+    r[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)f.off[i], 0, 0));
 }
 // ... and registers -> swizzled LDS tile
-__device__ __forceinline__ void attn_put_rows(const u32x4_t (&r)[4], char* tile) {
+template <int HD>
+__device__ __forceinline__ void attn_put_rows(const u32x4_t (&r)[HD / 32], char* tile) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < HD / 32; ++i) {
     const int c = threadIdx.x + 256 * i;
-    const int row = c >> 4;
-    *(u32x4_t*)(tile + row * kAttnRowB + (((c & 15) ^ attn_swz(row)) << 4)) = r[i];
+    const int row = c / (HD / 8);
+    *(u32x4_t*)(tile + row * (HD * 2) + (((c % (HD / 8)) ^ attn_swz<HD>(row)) << 4)) = r[i];
   }
 }
 
 // the lane's own row of one head as an MFMA operand: chunks 2s + h, s = 0..7
-__device__ __forceinline__ void attn_row_operand(bf16x8_t (&f)[8], const bf16_t* row_ptr, bool valid, int h) {
+template <int KS>
+__device__ __forceinline__ void attn_row_operand(bf16x8_t (&f)[KS], const bf16_t* row_ptr, bool valid, int h) {
 #pragma unroll
-  for (int s = 0; s < 8; ++s) {
+  for (int s = 0; s < KS; ++s) {
     const u32x4_t z = {0u, 0u, 0u, 0u};
     const u32x4_t x = valid ? *(const u32x4_t*)(row_ptr + (2 * s + h) * 8) : z;
     f[s] = __builtin_bit_cast(bf16x8_t, x);
@@ -155,9 +171,10 @@ __device__ __forceinline__ void attn_row_operand(bf16x8_t (&f)[8], const bf16_t*
 __device__ __forceinline__ float attn_swap32(float x) { return __shfl_xor(x, 32, 64); }
 
 // transposed accumulator (4 blocks of 32 d x 32 tokens, the lane's token = its column) -> [token][head][128] bf16
-__device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[4], float mul, bf16_t* row_ptr, int h) {
+template <int DB>
+__device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[DB], float mul, bf16_t* row_ptr, int h) {
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       uint2 pk;
@@ -170,12 +187,14 @@ __device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[4], fl
 // ---------------------------------------------------------------------------------------------------------
 // Forward: grid (ceil(T/128), Hq), 256 threads.
 // ---------------------------------------------------------------------------------------------------------
+template <int HD>
 __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
+  constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD;
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
   char* kt = smem;
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
-  const AttnLane L = attn_lane(lane);
+  const AttnLane<HD> L = attn_lane<HD>(lane);
   const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
   const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
   const int tq = q0 + 32 * wave + (lane & 31);
@@ -195,12 +214,12 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
   const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
 
-  bf16x8_t qf[8];
+  bf16x8_t qf[KS];
   attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
 
-  f32x16_t acc_o[4];
+  f32x16_t acc_o[DB];
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc_o[db][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
@@ -208,13 +227,13 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
 
   const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
   const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
-  u32x4_t rk[4], rv[4];
-  const AttnFetch fk = attn_fetch_init(p.k_st), fv = attn_fetch_init(p.v_st);
+  u32x4_t rk[DB], rv[DB];
+  const AttnFetch<HD> fk = attn_fetch_init<HD>(p.k_st), fv = attn_fetch_init<HD>(p.v_st);
   attn_fetch_rows(rk, fk, kbase, p.k_st, k_begin, k_end);
   attn_fetch_rows(rv, fv, vbase, p.v_st, k_begin, k_end);
   for (int kb = k_begin; kb < k_end; kb += kAttnBK) {
-    attn_put_rows(rk, kt);
-    attn_put_rows(rv, vt);
+    attn_put_rows<HD>(rk, kt);
+    attn_put_rows<HD>(rv, vt);
     __syncthreads();
     if (kb + kAttnBK < k_end) {   // next step's rows travel while this one is computed
       attn_fetch_rows(rk, fk, kbase, p.k_st, kb + kAttnBK, k_end);
@@ -227,7 +246,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[mb][r] = 0.f;
 #pragma unroll
-        for (int st = 0; st < 8; ++st) s[mb] = FGRPO_MFMA(attn_frag(kt, L, mb, st), qf[st], s[mb]);
+        for (int st = 0; st < KS; ++st) s[mb] = FGRPO_MFMA(attn_frag(kt, L, mb, st), qf[st], s[mb]);
       }
       float mx = -INFINITY;
       if (kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min) {   // every pair of this step is visible
@@ -264,7 +283,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
       m_run = m_new;
       if (__any(alpha != 1.f)) {      // once the running maxima have settled no lane rescales any more
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc_o[db][r] *= alpha;
       }
@@ -277,7 +296,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
           for (int j = 0; j < 8; ++j) tmp[j] = s[mb][8 * s2 + j];
           const bf16x8_t pf = attn_pack8(tmp);
 #pragma unroll
-          for (int db = 0; db < 4; ++db)
+          for (int db = 0; db < DB; ++db)
             acc_o[db] = FGRPO_MFMA(attn_frag_tr(vt, L, 32 * mb + 16 * s2, db), pf, acc_o[db]);
         }
     }
@@ -295,12 +314,14 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
 // dQ: grid (ceil(T/128), Hq), 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
 // Also produces delta[hq][t] = sum_d dO[t][hq][d] * O[t][hq][d] (each lane already holds its query's dO row).
 // ---------------------------------------------------------------------------------------------------------
+template <int HD>
 __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
+  constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD;
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
   char* kt = smem;
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
-  const AttnLane L = attn_lane(lane);
+  const AttnLane<HD> L = attn_lane<HD>(lane);
   const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
   const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
   const int tq = q0 + 32 * wave + (lane & 31);
@@ -318,17 +339,17 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
   const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
 
-  bf16x8_t qf[8], dof[8];
+  bf16x8_t qf[KS], dof[KS];
   attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
   attn_row_operand(dof, p.dout + ((long long)(valid ? tq : 0) * p.Hq + hq) * kHD, valid, h);
   const float lse2 = valid ? p.lse[(long long)hq * p.T + tq] * kLog2e : 0.f;
   // delta = rowsum(dO * O) of the lane's query: each lane half holds alternate 8-element pieces of the row
   float dl = 0.f;
   {
-    bf16x8_t of[8];
+    bf16x8_t of[KS];
     attn_row_operand(of, p.out_fwd + ((long long)(valid ? tq : 0) * p.Hq + hq) * kHD, valid, h);
 #pragma unroll
-    for (int st = 0; st < 8; ++st) {
+    for (int st = 0; st < KS; ++st) {
       const u32x4_t x = __builtin_bit_cast(u32x4_t, dof[st]), y = __builtin_bit_cast(u32x4_t, of[st]);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -341,21 +362,21 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   }
   const float c = p.scale * kLog2e;
 
-  f32x16_t acc[4];
+  f32x16_t acc[DB];
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
 
   const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
   const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
-  u32x4_t rk[4], rv[4];
-  const AttnFetch fk = attn_fetch_init(p.k_st), fv = attn_fetch_init(p.v_st);
+  u32x4_t rk[DB], rv[DB];
+  const AttnFetch<HD> fk = attn_fetch_init<HD>(p.k_st), fv = attn_fetch_init<HD>(p.v_st);
   attn_fetch_rows(rk, fk, kbase, p.k_st, k_begin, k_end);
   attn_fetch_rows(rv, fv, vbase, p.v_st, k_begin, k_end);
   for (int kb = k_begin; kb < k_end; kb += kAttnBK) {
-    attn_put_rows(rk, kt);
-    attn_put_rows(rv, vt);
+    attn_put_rows<HD>(rk, kt);
+    attn_put_rows<HD>(rv, vt);
     __syncthreads();
     if (kb + kAttnBK < k_end) {
       attn_fetch_rows(rk, fk, kbase, p.k_st, kb + kAttnBK, k_end);
@@ -368,7 +389,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
 #pragma unroll
-        for (int st = 0; st < 8; ++st) {
+        for (int st = 0; st < KS; ++st) {
           s = FGRPO_MFMA(attn_frag(kt, L, mb, st), qf[st], s);
           dp = FGRPO_MFMA(attn_frag(vt, L, mb, st), dof[st], dp);
         }
@@ -389,7 +410,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
         for (int s2 = 0; s2 < 2; ++s2) {
           const bf16x8_t dsf = attn_pack8(ds + 8 * s2);
 #pragma unroll
-          for (int db = 0; db < 4; ++db)
+          for (int db = 0; db < DB; ++db)
             acc[db] = FGRPO_MFMA(attn_frag_tr(kt, L, 32 * mb + 16 * s2, db), dsf, acc[db]);
         }
       }
@@ -403,7 +424,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
 // dK, dV: grid (ceil(T/128), Hkv), 256 threads; a wavefront owns 32 keys (one per lane pair) and walks the
 // queries that can see them, for every query head of the group.
 // ---------------------------------------------------------------------------------------------------------
+template <int HD>
 __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
+  constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD;
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
   __shared__ __attribute__((aligned(16))) float row_lse2[kAttnBK];
   __shared__ __attribute__((aligned(16))) float row_dl[kAttnBK];
@@ -412,7 +435,7 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
   char* qt = smem;
   char* dot = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
-  const AttnLane L = attn_lane(lane);
+  const AttnLane<HD> L = attn_lane<HD>(lane);
   const int hkv = blockIdx.y, G = p.Hq / p.Hkv;
   const int k0 = blockIdx.x * kAttnBQ;
   const int key = k0 + 32 * wave + (lane & 31);
@@ -426,24 +449,24 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
   const int wq_lo = wave_on ? (p.causal ? wfirst : p.seg_start[wfirst]) : 1;   // first / last query of interest
   const int wq_hi = wave_on ? p.seg_end[wlast] - 1 : 0;
 
-  bf16x8_t kf[8], vf[8];
+  bf16x8_t kf[KS], vf[KS];
   attn_row_operand(kf, p.k + (long long)(valid ? key : 0) * p.k_st + (long long)hkv * p.k_sh, valid, h);
   attn_row_operand(vf, p.v + (long long)(valid ? key : 0) * p.v_st + (long long)hkv * p.v_sh, valid, h);
   const float c = p.scale * kLog2e;
 
-  f32x16_t acc_k[4], acc_v[4];
+  f32x16_t acc_k[DB], acc_v[DB];
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
+  for (int nb = 0; nb < DB; ++nb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc_k[nb][r] = acc_v[nb][r] = 0.f;
 
-  const AttnFetch fq_ = attn_fetch_init(p.q_st), fd_ = attn_fetch_init((long long)p.Hq * kHD);
+  const AttnFetch<HD> fq_ = attn_fetch_init<HD>(p.q_st), fd_ = attn_fetch_init<HD>((long long)p.Hq * kHD);
   for (int g = 0; g < G; ++g) {
     const int hq = hkv * G + g;
     const bf16_t* qbase = p.q + (long long)hq * p.q_sh;
     const bf16_t* dobase = p.dout + (long long)hq * kHD;
     const long long do_st = (long long)p.Hq * kHD;
-    u32x4_t rq[4], rd[4];
+    u32x4_t rq[DB], rd[DB];
     // per-query scalars of a step travel with its rows: fetched one step ahead, never waited for inside a step
     float n_lse = 0.f, n_dl = 0.f;
     int n_lo = 1, n_hi = 0;
@@ -461,8 +484,8 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
     attn_fetch_rows(rd, fd_, dobase, do_st, q_begin, q_end);
     fetch_row_scalars(q_begin);
     for (int qb = q_begin; qb < q_end; qb += kAttnBK) {
-      attn_put_rows(rq, qt);
-      attn_put_rows(rd, dot);
+      attn_put_rows<HD>(rq, qt);
+      attn_put_rows<HD>(rd, dot);
       if (threadIdx.x < kAttnBK) {
         row_lse2[threadIdx.x] = n_lse;
         row_dl[threadIdx.x] = n_dl;
@@ -484,11 +507,11 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
         // sub-blocks are therefore software-pipelined by hand, one MFMA per softmax element:
         //   S,dP(0) | S,dP(1) + softmax(0) | dV,dK(0) + softmax(1) | dV,dK(1)
         // and LDS fragments are requested a phase before the MFMAs that use them.
-        bf16x8_t qa[8], da[8], fdo[2][4], fq[2][4], pf[2][2], dsf[2][2];
+        bf16x8_t qa[KS], da[KS], fdo[2][DB], fq[2][DB], pf[2][2], dsf[2][2];
         f32x16_t s[2], dp[2];
         auto load_rows = [&](int mq) {
 #pragma unroll
-          for (int st = 0; st < 8; ++st) {
+          for (int st = 0; st < KS; ++st) {
             qa[st] = attn_frag(qt, L, mq, st);
             da[st] = attn_frag(dot, L, mq, st);
           }
@@ -497,18 +520,19 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
+            for (int nb = 0; nb < DB; ++nb) {
               fdo[s2][nb] = attn_frag_tr(dot, L, 32 * mq + 16 * s2, nb);
               fq[s2][nb] = attn_frag_tr(qt, L, 32 * mq + 16 * s2, nb);
             }
         };
-        auto score_mfma = [&](int mq, int j) {      // MFMA j of 16: two chains of eight
-          if (j & 1) dp[mq] = FGRPO_MFMA(da[j >> 1], vf[j >> 1], dp[mq]);
-          else s[mq] = FGRPO_MFMA(qa[j >> 1], kf[j >> 1], s[mq]);
+        constexpr int NM = 2 * KS;                  // MFMAs of a phase (16 for HD = 128): one per 16 / NM softmax elements
+        auto score_mfma = [&](int mq, int m) {      // MFMA m of NM: two chains (S, dP) of KS
+          if (m & 1) dp[mq] = FGRPO_MFMA(da[m >> 1], vf[m >> 1], dp[mq]);
+          else s[mq] = FGRPO_MFMA(qa[m >> 1], kf[m >> 1], s[mq]);
         };
-        auto grad_mfma = [&](int mq, int j) {       // MFMA j of 16: eight accumulators
-          const int s2 = j >> 3, nb = (j >> 1) & 3;
-          if (j & 1) acc_k[nb] = FGRPO_MFMA(dsf[mq][s2], fq[s2][nb], acc_k[nb]);
+        auto grad_mfma = [&](int mq, int m) {       // MFMA m of NM: 2 * DB accumulators, two 16-query halves
+          const int s2 = (m >> 1) / DB, nb = (m >> 1) % DB;
+          if (m & 1) acc_k[nb] = FGRPO_MFMA(dsf[mq][s2], fq[s2][nb], acc_k[nb]);
           else acc_v[nb] = FGRPO_MFMA(pf[mq][s2], fdo[s2][nb], acc_v[nb]);
         };
         // softmax element r of sub-block mq: P and dS / scale (the scale is applied once, to the dK accumulators)
@@ -563,13 +587,13 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
         read_group(0, 0, !all_visible);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < 16; ++j) score_mfma(0, j);
+        for (int m = 0; m < NM; ++m) score_mfma(0, m);
         load_rows(1);
         __builtin_amdgcn_sched_barrier(0);
         if (all_visible) {
 #pragma unroll
           for (int j = 0; j < 16; ++j) {
-            score_mfma(1, j);
+            if (j % (16 / NM) == 0) score_mfma(1, j / (16 / NM));
             element(0, j, false);
             __builtin_amdgcn_sched_barrier(0);
           }
@@ -577,14 +601,14 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int j = 0; j < 16; ++j) {
-            grad_mfma(0, j);
+            if (j % (16 / NM) == 0) grad_mfma(0, j / (16 / NM));
             element(1, j, false);
             __builtin_amdgcn_sched_barrier(0);
           }
         } else {
 #pragma unroll
           for (int j = 0; j < 16; ++j) {
-            score_mfma(1, j);
+            if (j % (16 / NM) == 0) score_mfma(1, j / (16 / NM));
             element(0, j, true);
             __builtin_amdgcn_sched_barrier(0);
           }
@@ -592,7 +616,7 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int j = 0; j < 16; ++j) {
-            grad_mfma(0, j);
+            if (j % (16 / NM) == 0) grad_mfma(0, j / (16 / NM));
             element(1, j, true);
             __builtin_amdgcn_sched_barrier(0);
           }
@@ -601,14 +625,14 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
         load_tr(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < 16; ++j) grad_mfma(1, j);
+        for (int m = 0; m < NM; ++m) grad_mfma(1, m);
       }
       __syncthreads();
     }
   }
   // result lane = column d, rows = keys of this wavefront
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
+  for (int nb = 0; nb < DB; ++nb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int kk = k0 + 32 * wave + 8 * (r >> 2) + 4 * h + (r & 3);

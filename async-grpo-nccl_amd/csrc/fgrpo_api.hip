@@ -870,7 +870,7 @@ int check_attn(const char* who, const void* q, const void* k, const void* v, lon
   if (!q || !k || !v || !cu || !bounds_ws) return fail(FGRPO_ERR_BAD_ARG, "%s: null argument", who);
   if (T <= 0 || n_seq <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0)
     return fail(FGRPO_ERR_BAD_ARG, "%s: T=%d n_seq=%d Hq=%d Hkv=%d", who, T, n_seq, Hq, Hkv);
-  if (D != kHD) return fail(FGRPO_ERR_BAD_ARG, "%s: head dimension %d not supported (128 only)", who, D);
+  if (D != 128 && D != 64) return fail(FGRPO_ERR_BAD_ARG, "%s: head dimension %d not supported (128 or 64)", who, D);
   if (!(scale > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "%s: softmax scale must be positive", who);
   if (!aligned16(q) || !aligned16(k) || !aligned16(v)) return fail(FGRPO_ERR_ALIGN, "%s: q/k/v must be 16-byte aligned", who);
   const long long st[6] = {q_st, q_sh, k_st, k_sh, v_st, v_sh};
@@ -910,7 +910,9 @@ int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long
   p.lse = lse;
   hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
   HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(varlen_attn_fwd_kernel, dim3((T + kAttnBQ - 1) / kAttnBQ, Hq), dim3(256), 0, st, p);
+  const dim3 grid((T + kAttnBQ - 1) / kAttnBQ, Hq);
+  if (D == 128) hipLaunchKernelGGL(varlen_attn_fwd_kernel<128>, grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(varlen_attn_fwd_kernel<64>, grid, dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -936,9 +938,12 @@ int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const 
   p.dv = (bf16_t*)dv;
   hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
   HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(varlen_attn_dq_kernel, dim3((T + kAttnBQ - 1) / kAttnBQ, Hq), dim3(256), 0, st, p);
+  const dim3 grid_q((T + kAttnBQ - 1) / kAttnBQ, Hq), grid_k((T + kAttnBQ - 1) / kAttnBQ, Hkv);
+  if (D == 128) hipLaunchKernelGGL(varlen_attn_dq_kernel<128>, grid_q, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(varlen_attn_dq_kernel<64>, grid_q, dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(varlen_attn_dkv_kernel, dim3((T + kAttnBQ - 1) / kAttnBQ, Hkv), dim3(256), 0, st, p);
+  if (D == 128) hipLaunchKernelGGL(varlen_attn_dkv_kernel<128>, grid_k, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(varlen_attn_dkv_kernel<64>, grid_k, dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());
   return 0;
 }

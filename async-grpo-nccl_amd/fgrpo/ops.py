@@ -560,7 +560,7 @@ def fused_grpo_loss(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp=No
 
 # --------------------------------------------------------------------------- packed variable-length attention
 def _attn_operand(t: torch.Tensor, name: str) -> torch.Tensor:
-    """[T, H, 128] bf16 view the kernels can read in place (innermost contiguous, strides multiples of 8
+    """[T, H, D] bf16 view the kernels can read in place (innermost contiguous, strides multiples of 8
     elements, 16-byte aligned base); anything else is copied once."""
     if t.dim() != 3:
         raise RuntimeError(f"fgrpo: {name} must be [tokens, heads, head_dim], got {tuple(t.shape)}")

@@ -15,7 +15,7 @@ Mirrors, for this path, what the reference gets from flash-attn and from its loc
   (``gpu_process_worker.py:110``): makes a model use the callable above; returns ``True`` when installed.
 
 There is no fallback: inputs the kernels do not cover (dropout, sliding windows, padding masks, head
-dimensions other than 128, CPU tensors) raise."""
+dimensions other than 128 and 64, CPU tensors) raise."""
 from __future__ import annotations
 
 import weakref

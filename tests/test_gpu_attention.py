@@ -19,19 +19,19 @@ def cos(a, b):
     return F.cosine_similarity(a.detach().float().flatten().cpu(), b.detach().float().flatten().cpu(), dim=0).item()
 
 
-def make(T, Hq, Hkv, seed, scale_in=1.0):
+def make(T, Hq, Hkv, seed, scale_in=1.0, D=128):
     g = torch.Generator().manual_seed(seed)
-    q = (torch.randn(T, Hq, 128, generator=g) * scale_in).bfloat16()
-    k = (torch.randn(T, Hkv, 128, generator=g) * scale_in).bfloat16()
-    v = torch.randn(T, Hkv, 128, generator=g).bfloat16()
-    do = torch.randn(T, Hq, 128, generator=g).bfloat16()
+    q = (torch.randn(T, Hq, D, generator=g) * scale_in).bfloat16()
+    k = (torch.randn(T, Hkv, D, generator=g) * scale_in).bfloat16()
+    v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+    do = torch.randn(T, Hq, D, generator=g).bfloat16()
     return q, k, v, do
 
 
-def check(dev, name, T, cu, Hq, Hkv, causal, seed=0, softmax_scale=None, backward=True):
+def check(dev, name, T, cu, Hq, Hkv, causal, seed=0, softmax_scale=None, backward=True, D=128):
     from fgrpo import ops
-    print(f"[attention case] {name}: T={T} Hq={Hq} Hkv={Hkv} causal={causal} segments={len(cu) - 1}", flush=True)
-    q, k, v, do = make(T, Hq, Hkv, seed)
+    print(f"[attention case] {name}: T={T} Hq={Hq} Hkv={Hkv} D={D} causal={causal} segments={len(cu) - 1}", flush=True)
+    q, k, v, do = make(T, Hq, Hkv, seed, D=D)
     cu_t = torch.tensor(cu, dtype=torch.int32)
     qo, ko, vo = (x.float().requires_grad_(True) for x in (q, k, v))
     want, want_lse = A.varlen_attention(qo, ko, vo, cu_t, softmax_scale=softmax_scale, causal=causal, return_lse=True)
@@ -66,6 +66,13 @@ def test_small_segments_share_a_tile(dev, causal):
 @pytest.mark.parametrize("causal", [True, False])
 def test_segments_cross_tile_boundaries(dev, causal):
     check(dev, "crossing tiles", 1000, [0, 130, 385, 390, 900, 1000], 4, 4, causal, seed=2)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_head_dimension_64(dev, causal):
+    # 14 query heads over 2 K/V heads of 64: the attention shape of Qwen2.5-0.5B
+    check(dev, "head dim 64, short segments", 200, [0, 5, 6, 70, 71, 72, 200], 4, 2, causal, seed=21, D=64)
+    check(dev, "head dim 64, crossing tiles", 1000, [0, 130, 385, 390, 900, 1000], 14, 2, causal, seed=22, D=64)
 
 
 def test_one_long_segment(dev):
@@ -160,9 +167,9 @@ def test_full_size_properties(dev):
 def test_argument_errors(dev):
     from fgrpo import ops
     cu = torch.tensor([0, 16], dtype=torch.int32, device=dev)
-    q64 = torch.zeros(16, 2, 64, dtype=torch.bfloat16, device=dev)
+    q96 = torch.zeros(16, 2, 96, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError, match="head dimension"):
-        ops.varlen_attn_fwd(q64, q64, q64, cu)
+        ops.varlen_attn_fwd(q96, q96, q96, cu)
     q = torch.zeros(16, 3, 128, dtype=torch.bfloat16, device=dev)
     kv = torch.zeros(16, 2, 128, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError):
