@@ -300,3 +300,21 @@ def test_workers_on_a_transformers_model_end_to_end(dev):
     for p_ in (model.model.layers[0].self_attn.q_proj.weight, model.model.layers[1].self_attn.v_proj.weight,
                model.lm_head.weight):
         assert p_.grad is not None and torch.isfinite(p_.grad.float()).all() and p_.grad.float().abs().max().item() > 0
+
+
+def test_random_shapes_and_segmentations(dev):
+    """Seeded sweep over awkward sizes (T = 1, tile edges +-1), both head dimensions, grouped-query ratios up to 7,
+    empty and one-token segments, causal and full attention - forward and backward against the oracle."""
+    import random
+    rnd = random.Random(0)
+    for case in range(30):
+        T = rnd.choice([1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 255, 256, 257, 300, 511])
+        D = rnd.choice([64, 128])
+        Hkv = rnd.choice([1, 2, 3])
+        Hq = Hkv * rnd.choice([1, 2, 4, 7])
+        causal = rnd.random() < 0.7
+        cuts = sorted(set(rnd.sample(range(1, T), min(T - 1, rnd.randint(0, 6))))) if T > 1 else []
+        cu = [0] + cuts + [T]
+        if rnd.random() < 0.3:
+            cu = cu[:1] + [cu[1]] + cu[1:]                  # an empty segment
+        check(dev, f"random {case}", T, cu, Hq, Hkv, causal, seed=100 + case, D=D)
