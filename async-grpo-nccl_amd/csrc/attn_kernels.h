@@ -43,6 +43,8 @@ struct AttnParams {
   long long q_st, q_sh, k_st, k_sh, v_st, v_sh;
   const int* seg_start;  // [T] first token of the token's segment
   const int* seg_end;    // [T] one past the last token of the token's segment
+  const int* order_q;    // [ceil(T/128)] query tiles, most keys first
+  const int* order_k;    // [ceil(T/128)] key tiles, most queries first
   int T, Hq, Hkv;
   float scale;
   int causal;
@@ -185,7 +187,7 @@ __device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[DB], f
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Forward: grid (ceil(T/128), Hq), 256 threads.
+// Forward: grid (Hq, ceil(T/128)), 256 threads.
 // ---------------------------------------------------------------------------------------------------------
 template <int HD>
 __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
@@ -195,8 +197,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const AttnLane<HD> L = attn_lane<HD>(lane);
-  const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
+  // grid (heads, tiles): heads are the fast index, so the tiles start in the order of the list - most work first
+  const int hq = blockIdx.x, hkv = hq / (p.Hq / p.Hkv);
+  const int q0 = p.order_q[blockIdx.y] * kAttnBQ;
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
@@ -311,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// dQ: grid (ceil(T/128), Hq), 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
+// dQ: grid (Hq, ceil(T/128)), 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
 // Also produces delta[hq][t] = sum_d dO[t][hq][d] * O[t][hq][d] (each lane already holds its query's dO row).
 // ---------------------------------------------------------------------------------------------------------
 template <int HD>
@@ -322,8 +325,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const AttnLane<HD> L = attn_lane<HD>(lane);
-  const int hq = blockIdx.y, hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * kAttnBQ;   // late tiles see the most keys: start them first
+  // grid (heads, tiles): heads are the fast index, so the tiles start in the order of the list - most work first
+  const int hq = blockIdx.x, hkv = hq / (p.Hq / p.Hkv);
+  const int q0 = p.order_q[blockIdx.y] * kAttnBQ;
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
@@ -421,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// dK, dV: grid (ceil(T/128), Hkv), 256 threads; a wavefront owns 32 keys (one per lane pair) and walks the
+// dK, dV: grid (Hkv, ceil(T/128)), 256 threads; a wavefront owns 32 keys (one per lane pair) and walks the
 // queries that can see them, for every query head of the group.
 // ---------------------------------------------------------------------------------------------------------
 template <int HD>
@@ -436,8 +440,8 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
   char* dot = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const AttnLane<HD> L = attn_lane<HD>(lane);
-  const int hkv = blockIdx.y, G = p.Hq / p.Hkv;
-  const int k0 = blockIdx.x * kAttnBQ;
+  const int hkv = blockIdx.x, G = p.Hq / p.Hkv;
+  const int k0 = p.order_k[blockIdx.y] * kAttnBQ;
   const int key = k0 + 32 * wave + (lane & 31);
   const bool valid = key < p.T;
   const int last = (k0 + kAttnBQ - 1 < p.T ? k0 + kAttnBQ - 1 : p.T - 1);
@@ -664,6 +668,40 @@ __global__ void segment_bounds_kernel(const int* cu, int nseq, int T, int* seg_s
   while (e < nseq && cu[e] <= t) ++e;
   seg_start[t] = cu[a] > 0 ? cu[a] : 0;
   seg_end[t] = cu[e] < T ? cu[e] : T;
+}
+
+// Work-group start order: tiles sorted by the number of steps they will walk, most first (ties by index), so that
+// the long tiles of long segments do not end up alone at the tail of the launch.  One work-group of 1024 threads;
+// rank by counting (n <= kAttnMaxSorted tiles), otherwise the plain guess (late query tiles / early key tiles first).
+constexpr int kAttnMaxSorted = 2048;
+__global__ void attn_tile_order_kernel(const int* seg_start, const int* seg_end, int T, int causal, int* order_q,
+                                       int* order_k) {
+  __shared__ int wq[kAttnMaxSorted], wk[kAttnMaxSorted];
+  const int n = (T + kAttnBQ - 1) / kAttnBQ;
+  if (n > kAttnMaxSorted) {
+    for (int t = threadIdx.x; t < n; t += blockDim.x) {
+      order_q[t] = n - 1 - t;
+      order_k[t] = t;
+    }
+    return;
+  }
+  for (int t = threadIdx.x; t < n; t += blockDim.x) {
+    const int first = t * kAttnBQ, last = (first + kAttnBQ - 1 < T ? first + kAttnBQ - 1 : T - 1);
+    wq[t] = (causal ? last + 1 : seg_end[last]) - seg_start[first];          // keys a query tile walks
+    wk[t] = seg_end[last] - (causal ? first : seg_start[first]);             // queries a key tile walks
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < n; t += blockDim.x) {
+    const int a = wq[t], b = wk[t];
+    int ra = 0, rb = 0;
+    for (int u = 0; u < n; ++u) {
+      const int x = wq[u], y = wk[u];
+      ra += (x > a) | ((x == a) & (u < t));
+      rb += (y > b) | ((y == b) & (u < t));
+    }
+    order_q[ra] = t;
+    order_k[rb] = t;
+  }
 }
 
 }  // namespace fgrpo

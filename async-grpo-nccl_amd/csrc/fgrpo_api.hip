@@ -889,6 +889,8 @@ void fill_attn(AttnParams& p, const void* q, const void* k, const void* v, long 
   p.q_st = q_st, p.q_sh = q_sh, p.k_st = k_st, p.k_sh = k_sh, p.v_st = v_st, p.v_sh = v_sh;
   p.seg_start = bounds_ws;
   p.seg_end = bounds_ws + T;
+  p.order_q = bounds_ws + 2 * (long long)T;
+  p.order_k = p.order_q + (T + kAttnBQ - 1) / kAttnBQ;
   p.T = T, p.Hq = Hq, p.Hkv = Hkv;
   p.scale = scale;
   p.causal = causal != 0;
@@ -910,7 +912,10 @@ int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long
   p.lse = lse;
   hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
   HIP_TRY(hipGetLastError());
-  const dim3 grid((T + kAttnBQ - 1) / kAttnBQ, Hq);
+  hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
+                     const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
+  HIP_TRY(hipGetLastError());
+  const dim3 grid(Hq, (T + kAttnBQ - 1) / kAttnBQ);
   if (D == 128) hipLaunchKernelGGL(varlen_attn_fwd_kernel<128>, grid, dim3(256), 0, st, p);
   else hipLaunchKernelGGL(varlen_attn_fwd_kernel<64>, grid, dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());
@@ -938,7 +943,10 @@ int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const 
   p.dv = (bf16_t*)dv;
   hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
   HIP_TRY(hipGetLastError());
-  const dim3 grid_q((T + kAttnBQ - 1) / kAttnBQ, Hq), grid_k((T + kAttnBQ - 1) / kAttnBQ, Hkv);
+  hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
+                     const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
+  HIP_TRY(hipGetLastError());
+  const dim3 grid_q(Hq, (T + kAttnBQ - 1) / kAttnBQ), grid_k(Hkv, (T + kAttnBQ - 1) / kAttnBQ);
   if (D == 128) hipLaunchKernelGGL(varlen_attn_dq_kernel<128>, grid_q, dim3(256), 0, st, p);
   else hipLaunchKernelGGL(varlen_attn_dq_kernel<64>, grid_q, dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());

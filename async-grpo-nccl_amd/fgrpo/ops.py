@@ -589,7 +589,7 @@ def varlen_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlen
     lse = torch.empty((Hq, T), dtype=torch.float32, device=dev)
     if T == 0:
         return out, lse
-    bounds = torch.empty(2 * T, dtype=torch.int32, device=dev)
+    bounds = torch.empty(2 * T + 2 * ((T + 127) // 128), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         rc = lib.fgrpo_varlen_attn_fwd(_ptr(q), _ptr(k), _ptr(v), q.stride(0), q.stride(1), k.stride(0), k.stride(1),
                                        v.stride(0), v.stride(1), _ptr(cu), cu.numel() - 1, T, Hq, Hkv, D, scale,
@@ -619,7 +619,7 @@ def varlen_attn_bwd(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
     if T == 0:
         return dq, dk, dv
     delta = torch.empty((Hq, T), dtype=torch.float32, device=dev)
-    bounds = torch.empty(2 * T, dtype=torch.int32, device=dev)
+    bounds = torch.empty(2 * T + 2 * ((T + 127) // 128), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         rc = lib.fgrpo_varlen_attn_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), q.stride(0),
                                        q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), _ptr(cu),
