@@ -187,7 +187,7 @@ __device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[DB], f
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Forward: grid (Hq, ceil(T/128)), 256 threads.
+// Forward: 1-D grid of round_up(ceil(T/128) * Hkv, 8) * (Hq / Hkv) work-groups, 256 threads.
 // ---------------------------------------------------------------------------------------------------------
 template <int HD>
 __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
@@ -197,9 +197,15 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const AttnLane<HD> L = attn_lane<HD>(lane);
-  // grid (heads, tiles): heads are the fast index, so the tiles start in the order of the list - most work first
-  const int hq = blockIdx.x, hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = p.order_q[blockIdx.y] * kAttnBQ;
+  // 1-D grid over (tile rank, K/V head, query head of the group), most work first.  Work-groups go to the 8 XCDs
+  // round-robin (work-group b runs on XCD b % 8, each with its own L2): the query heads of one K/V group - which
+  // stream the same K and V rows - are given consecutive slots of ONE XCD, and whole groups go round the XCDs.
+  const int G = p.Hq / p.Hkv;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int unit = (slot / G) * 8 + xcd;                  // (tile rank, K/V head)
+  if (unit >= (int)((p.T + kAttnBQ - 1) / kAttnBQ) * p.Hkv) return;
+  const int hkv = unit % p.Hkv, hq = hkv * G + slot % G;
+  const int q0 = p.order_q[unit / p.Hkv] * kAttnBQ;
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
@@ -314,7 +320,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// dQ: grid (Hq, ceil(T/128)), 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
+// dQ: same grid as the forward, 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
 // Also produces delta[hq][t] = sum_d dO[t][hq][d] * O[t][hq][d] (each lane already holds its query's dO row).
 // ---------------------------------------------------------------------------------------------------------
 template <int HD>
@@ -325,9 +331,15 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   char* vt = smem + kAttnTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const AttnLane<HD> L = attn_lane<HD>(lane);
-  // grid (heads, tiles): heads are the fast index, so the tiles start in the order of the list - most work first
-  const int hq = blockIdx.x, hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = p.order_q[blockIdx.y] * kAttnBQ;
+  // 1-D grid over (tile rank, K/V head, query head of the group), most work first.  Work-groups go to the 8 XCDs
+  // round-robin (work-group b runs on XCD b % 8, each with its own L2): the query heads of one K/V group - which
+  // stream the same K and V rows - are given consecutive slots of ONE XCD, and whole groups go round the XCDs.
+  const int G = p.Hq / p.Hkv;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int unit = (slot / G) * 8 + xcd;                  // (tile rank, K/V head)
+  if (unit >= (int)((p.T + kAttnBQ - 1) / kAttnBQ) * p.Hkv) return;
+  const int hkv = unit % p.Hkv, hq = hkv * G + slot % G;
+  const int q0 = p.order_q[unit / p.Hkv] * kAttnBQ;
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;

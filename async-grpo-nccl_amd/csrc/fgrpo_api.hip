@@ -915,7 +915,8 @@ int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long
   hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
                      const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
   HIP_TRY(hipGetLastError());
-  const dim3 grid(Hq, (T + kAttnBQ - 1) / kAttnBQ);
+  const long long units = (long long)((T + kAttnBQ - 1) / kAttnBQ) * Hkv;       // (tile, K/V head)
+  const dim3 grid((unsigned)(((units + 7) / 8 * 8) * (Hq / Hkv)));
   if (D == 128) hipLaunchKernelGGL(varlen_attn_fwd_kernel<128>, grid, dim3(256), 0, st, p);
   else hipLaunchKernelGGL(varlen_attn_fwd_kernel<64>, grid, dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());
@@ -946,7 +947,8 @@ int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const 
   hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
                      const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
   HIP_TRY(hipGetLastError());
-  const dim3 grid_q(Hq, (T + kAttnBQ - 1) / kAttnBQ), grid_k(Hkv, (T + kAttnBQ - 1) / kAttnBQ);
+  const long long units = (long long)((T + kAttnBQ - 1) / kAttnBQ) * Hkv;       // (tile, K/V head)
+  const dim3 grid_q((unsigned)(((units + 7) / 8 * 8) * (Hq / Hkv))), grid_k(Hkv, (T + kAttnBQ - 1) / kAttnBQ);
   if (D == 128) hipLaunchKernelGGL(varlen_attn_dq_kernel<128>, grid_q, dim3(256), 0, st, p);
   else hipLaunchKernelGGL(varlen_attn_dq_kernel<64>, grid_q, dim3(256), 0, st, p);
   HIP_TRY(hipGetLastError());
