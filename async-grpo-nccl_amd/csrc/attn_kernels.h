@@ -205,14 +205,15 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   const int unit = (slot / G) * 8 + xcd;                  // (tile rank, K/V head)
   if (unit >= (int)((p.T + kAttnBQ - 1) / kAttnBQ) * p.Hkv) return;
   const int hkv = unit % p.Hkv, hq = hkv * G + slot % G;
-  const int q0 = p.order_q[unit / p.Hkv] * kAttnBQ;
+  const int ntile = (p.T + kAttnBQ - 1) / kAttnBQ;
+  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * kAttnBQ;    // clamped: the list may come from the caller
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
   const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
   const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
-  const int k_begin = __builtin_amdgcn_readfirstlane(p.seg_start[q0]);          // wavefront-uniform loop bounds
-  const int k_end = __builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]);
+  const int k_begin = max(__builtin_amdgcn_readfirstlane(p.seg_start[q0]), 0);   // wavefront-uniform loop bounds, inside [0, T]
+  const int k_end = min(__builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]), p.T);
   // this wavefront's own key range (whole steps outside it are skipped)
   const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
   const bool wave_on = wfirst < p.T;
@@ -339,14 +340,15 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   const int unit = (slot / G) * 8 + xcd;                  // (tile rank, K/V head)
   if (unit >= (int)((p.T + kAttnBQ - 1) / kAttnBQ) * p.Hkv) return;
   const int hkv = unit % p.Hkv, hq = hkv * G + slot % G;
-  const int q0 = p.order_q[unit / p.Hkv] * kAttnBQ;
+  const int ntile = (p.T + kAttnBQ - 1) / kAttnBQ;
+  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * kAttnBQ;    // clamped: the list may come from the caller
   const int tq = q0 + 32 * wave + (lane & 31);
   const bool valid = tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
   const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
   const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
-  const int k_begin = __builtin_amdgcn_readfirstlane(p.seg_start[q0]);          // wavefront-uniform loop bounds
-  const int k_end = __builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]);
+  const int k_begin = max(__builtin_amdgcn_readfirstlane(p.seg_start[q0]), 0);   // wavefront-uniform loop bounds, inside [0, T]
+  const int k_end = min(__builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]), p.T);
   const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
   const bool wave_on = wfirst < p.T;
   const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
@@ -453,13 +455,13 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const AttnLane<HD> L = attn_lane<HD>(lane);
   const int hkv = blockIdx.x, G = p.Hq / p.Hkv;
-  const int k0 = p.order_k[blockIdx.y] * kAttnBQ;
+  const int k0 = min(max(p.order_k[blockIdx.y], 0), (int)gridDim.y - 1) * kAttnBQ;   // clamped: the list may come from the caller
   const int key = k0 + 32 * wave + (lane & 31);
   const bool valid = key < p.T;
   const int last = (k0 + kAttnBQ - 1 < p.T ? k0 + kAttnBQ - 1 : p.T - 1);
   // queries that can see a key of this tile
-  const int q_begin = __builtin_amdgcn_readfirstlane(p.causal ? k0 : p.seg_start[k0]);   // wavefront-uniform loop bounds
-  const int q_end = __builtin_amdgcn_readfirstlane(p.seg_end[last]);
+  const int q_begin = max(__builtin_amdgcn_readfirstlane(p.causal ? k0 : p.seg_start[k0]), 0);   // wavefront-uniform loop bounds, inside [0, T]
+  const int q_end = min(__builtin_amdgcn_readfirstlane(p.seg_end[last]), p.T);
   const int wfirst = k0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
   const bool wave_on = wfirst < p.T;
   const int wq_lo = wave_on ? (p.causal ? wfirst : p.seg_start[wfirst]) : 1;   // first / last query of interest
@@ -703,16 +705,28 @@ __global__ void attn_tile_order_kernel(const int* seg_start, const int* seg_end,
     wk[t] = seg_end[last] - (causal ? first : seg_start[first]);             // queries a key tile walks
   }
   __syncthreads();
-  for (int t = threadIdx.x; t < n; t += blockDim.x) {
+  // rank by counting, PARTS threads per tile each scanning 1/PARTS of the list
+  __shared__ int rq[kAttnMaxSorted], rk[kAttnMaxSorted];
+  for (int t = threadIdx.x; t < n; t += blockDim.x) rq[t] = rk[t] = 0;
+  __syncthreads();
+  const int parts = (int)blockDim.x / n > 1 ? (int)blockDim.x / n : 1;
+  const int span = (n + parts - 1) / parts;
+  for (int w = threadIdx.x; w < n * parts; w += blockDim.x) {
+    const int t = w / parts, u0 = (w % parts) * span, u1 = (u0 + span < n ? u0 + span : n);
     const int a = wq[t], b = wk[t];
     int ra = 0, rb = 0;
-    for (int u = 0; u < n; ++u) {
+    for (int u = u0; u < u1; ++u) {
       const int x = wq[u], y = wk[u];
       ra += (x > a) | ((x == a) & (u < t));
       rb += (y > b) | ((y == b) & (u < t));
     }
-    order_q[ra] = t;
-    order_k[rb] = t;
+    atomicAdd(&rq[t], ra);      // integer counts: the order of the additions does not matter
+    atomicAdd(&rk[t], rb);
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < n; t += blockDim.x) {
+    order_q[rq[t]] = t;
+    order_k[rk[t]] = t;
   }
 }
 

@@ -926,7 +926,7 @@ int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long
 int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
                           long long q_st, long long q_sh, long long k_st, long long k_sh, long long v_st, long long v_sh,
                           const int32_t* cu, int n_seq, int T, int Hq, int Hkv, int D, float scale, int causal, void* dq,
-                          void* dk, void* dv, float* delta_ws, int32_t* bounds_ws, void* stream) {
+                          void* dk, void* dv, float* delta_ws, int32_t* bounds_ws, int bounds_valid, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   int rc = check_attn("varlen_attn_bwd", q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, cu, n_seq, T, Hq, Hkv, D, scale, bounds_ws);
   if (rc) return rc;
@@ -942,11 +942,13 @@ int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const 
   p.dq = (bf16_t*)dq;
   p.dk = (bf16_t*)dk;
   p.dv = (bf16_t*)dv;
-  hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
-  HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
-                     const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
-  HIP_TRY(hipGetLastError());
+  if (!bounds_valid) {   // else bounds_ws still holds what a forward or backward call with the same segments wrote
+    hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
+    HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
+                       const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
+    HIP_TRY(hipGetLastError());
+  }
   const long long units = (long long)((T + kAttnBQ - 1) / kAttnBQ) * Hkv;       // (tile, K/V head)
   const dim3 grid_q((unsigned)(((units + 7) / 8 * 8) * (Hq / Hkv))), grid_k(Hkv, (T + kAttnBQ - 1) / kAttnBQ);
   if (D == 128) hipLaunchKernelGGL(varlen_attn_dq_kernel<128>, grid_q, dim3(256), 0, st, p);

@@ -43,7 +43,7 @@ SIGNATURES = {
     "fgrpo_varlen_attn_fwd": (_i, [_vp, _vp, _vp, _ll, _ll, _ll, _ll, _ll, _ll, _vp, _i, _i, _i, _i, _i, _f, _i,
                                    _vp, _vp, _vp, _vp]),
     "fgrpo_varlen_attn_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _ll, _ll, _ll, _ll, _ll, _ll, _vp, _i, _i, _i, _i, _i,
-                                   _f, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
+                                   _f, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
 }
 
 _lib = None

@@ -573,9 +573,10 @@ def _attn_operand(t: torch.Tensor, name: str) -> torch.Tensor:
 
 
 def varlen_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
-                    softmax_scale: Optional[float] = None, causal: bool = True):
+                    softmax_scale: Optional[float] = None, causal: bool = True, return_bounds: bool = False):
     """out [T, Hq, D] bf16 and lse [Hq, T] fp32 of packed self-attention: segment i covers tokens
-    cu_seqlens[i]:cu_seqlens[i+1]; query head j reads K/V head j // (Hq // Hkv)."""
+    cu_seqlens[i]:cu_seqlens[i+1]; query head j reads K/V head j // (Hq // Hkv).  ``return_bounds``: also the int32
+    scratch (per-token segment bounds, tile order) that ``varlen_attn_bwd`` can take over instead of rebuilding it."""
     dev = _require_cuda(q, k, v, cu_seqlens)
     lib = _lib.load()
     q, k, v = _attn_operand(q, "q"), _attn_operand(k, "k"), _attn_operand(v, "v")
@@ -587,21 +588,22 @@ def varlen_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlen
     scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
     out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
     lse = torch.empty((Hq, T), dtype=torch.float32, device=dev)
-    if T == 0:
-        return out, lse
     bounds = torch.empty(2 * T + 2 * ((T + 127) // 128), dtype=torch.int32, device=dev)
+    if T == 0:
+        return (out, lse, bounds) if return_bounds else (out, lse)
     with torch.cuda.device(dev):
         rc = lib.fgrpo_varlen_attn_fwd(_ptr(q), _ptr(k), _ptr(v), q.stride(0), q.stride(1), k.stride(0), k.stride(1),
                                        v.stride(0), v.stride(1), _ptr(cu), cu.numel() - 1, T, Hq, Hkv, D, scale,
                                        int(bool(causal)), _ptr(out), _ptr(lse), _ptr(bounds), _stream())
     _lib.check(rc, "varlen_attn_fwd")
-    return out, lse
+    return (out, lse, bounds) if return_bounds else (out, lse)
 
 
 def varlen_attn_bwd(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
                     lse: torch.Tensor, cu_seqlens: torch.Tensor, softmax_scale: Optional[float] = None,
-                    causal: bool = True):
-    """(dq, dk, dv) bf16, contiguous, for the forward above."""
+                    causal: bool = True, bounds: Optional[torch.Tensor] = None):
+    """(dq, dk, dv) bf16, contiguous, for the forward above.  ``bounds``: the scratch the forward returned for the
+    same ``cu_seqlens`` and ``causal``."""
     dev = _require_cuda(dout, q, k, v, out, lse, cu_seqlens)
     lib = _lib.load()
     q, k, v = _attn_operand(q, "q"), _attn_operand(k, "k"), _attn_operand(v, "v")
@@ -619,12 +621,17 @@ def varlen_attn_bwd(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
     if T == 0:
         return dq, dk, dv
     delta = torch.empty((Hq, T), dtype=torch.float32, device=dev)
-    bounds = torch.empty(2 * T + 2 * ((T + 127) // 128), dtype=torch.int32, device=dev)
+    n_bounds = 2 * T + 2 * ((T + 127) // 128)
+    bounds_valid = bounds is not None
+    if bounds_valid and (bounds.dtype != torch.int32 or bounds.numel() != n_bounds or bounds.device != dev):
+        raise RuntimeError("fgrpo: bounds does not come from a forward call of this shape")
+    if not bounds_valid:
+        bounds = torch.empty(n_bounds, dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         rc = lib.fgrpo_varlen_attn_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), q.stride(0),
                                        q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), _ptr(cu),
                                        cu.numel() - 1, T, Hq, Hkv, D, scale, int(bool(causal)), _ptr(dq), _ptr(dk),
-                                       _ptr(dv), _ptr(delta), _ptr(bounds), _stream())
+                                       _ptr(dv), _ptr(delta), _ptr(bounds), int(bounds_valid), _stream())
     _lib.check(rc, "varlen_attn_bwd")
     return dq, dk, dv
 
@@ -632,15 +639,15 @@ def varlen_attn_bwd(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
 class _VarlenAttention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens, softmax_scale, causal):
-        out, lse = varlen_attn_fwd(q, k, v, cu_seqlens, softmax_scale, causal)
-        ctx.save_for_backward(q, k, v, out, lse, cu_seqlens)
+        out, lse, bounds = varlen_attn_fwd(q, k, v, cu_seqlens, softmax_scale, causal, return_bounds=True)
+        ctx.save_for_backward(q, k, v, out, lse, cu_seqlens, bounds)
         ctx.softmax_scale, ctx.causal = softmax_scale, causal
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, out, lse, cu = ctx.saved_tensors
-        dq, dk, dv = varlen_attn_bwd(dout.to(torch.bfloat16), q, k, v, out, lse, cu, ctx.softmax_scale, ctx.causal)
+        q, k, v, out, lse, cu, bounds = ctx.saved_tensors
+        dq, dk, dv = varlen_attn_bwd(dout.to(torch.bfloat16), q, k, v, out, lse, cu, ctx.softmax_scale, ctx.causal, bounds)
         return dq, dk, dv, None, None, None
 
 

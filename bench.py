@@ -95,9 +95,9 @@ def attention_line(args):
     pairs = sum(n * (n + 1) // 2 for n in lens)
     f_fwd = 4.0 * D * Hq * pairs
 
-    def step():
-        out, lse = ops.varlen_attn_fwd(q, k, v, cu)
-        return ops.varlen_attn_bwd(do, q, k, v, out, lse, cu)
+    def step():       # what the autograd function does: the backward takes over the forward's segment scratch
+        out, lse, bounds = ops.varlen_attn_fwd(q, k, v, cu, return_bounds=True)
+        return ops.varlen_attn_bwd(do, q, k, v, out, lse, cu, bounds=bounds)
 
     for _ in range(args.warmup):
         step()
@@ -107,9 +107,9 @@ def attention_line(args):
     t0 = time.perf_counter()
     for _ in range(args.steps):
         ev[0].record()
-        out, lse = ops.varlen_attn_fwd(q, k, v, cu)
+        out, lse, bounds = ops.varlen_attn_fwd(q, k, v, cu, return_bounds=True)
         ev[1].record()
-        ops.varlen_attn_bwd(do, q, k, v, out, lse, cu)
+        ops.varlen_attn_bwd(do, q, k, v, out, lse, cu, bounds=bounds)
         ev[2].record()
         torch.cuda.synchronize()
         t_f += ev[0].elapsed_time(ev[1])

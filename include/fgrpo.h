@@ -188,12 +188,13 @@ int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long
 
 /* Backward of the above (autograd of flash_attn_varlen_func in the reference).  dout, out
  * [T, Hq, D] bf16 contiguous; dq [T, Hq, D], dk / dv [T, Hkv, D] bf16 contiguous;
- * delta_ws: Hq*T fp32 of scratch. */
+ * delta_ws: Hq*T fp32 of scratch.  bounds_valid != 0: bounds_ws is the buffer a forward (or backward) call
+ * with the same cu_seqlens, T and causal flag filled, and is used as it is. */
 int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
                           const float* lse, long long q_stride_t, long long q_stride_h, long long k_stride_t,
                           long long k_stride_h, long long v_stride_t, long long v_stride_h, const int32_t* cu_seqlens,
                           int n_seq, int T, int Hq, int Hkv, int D, float softmax_scale, int causal, void* dq, void* dk,
-                          void* dv, float* delta_ws, int32_t* bounds_ws, void* stream);
+                          void* dv, float* delta_ws, int32_t* bounds_ws, int bounds_valid, void* stream);
 
 #ifdef __cplusplus
 }
