@@ -897,10 +897,22 @@ void fill_attn(AttnParams& p, const void* q, const void* k, const void* v, long 
 }
 }  // namespace
 
+int fgrpo_varlen_attn_bounds(const int32_t* cu, int n_seq, int T, int causal, int32_t* bounds_ws, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!cu || !bounds_ws || T <= 0 || n_seq <= 0) return fail(FGRPO_ERR_BAD_ARG, "varlen_attn_bounds: bad argument");
+  int32_t* order_q = bounds_ws + 2 * (long long)T;
+  hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
+  HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, bounds_ws, bounds_ws + T, T, causal != 0, order_q,
+                     order_q + (T + kAttnBQ - 1) / kAttnBQ);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long q_st, long long q_sh, long long k_st,
                           long long k_sh, long long v_st, long long v_sh, const int32_t* cu, int n_seq, int T, int Hq,
                           int Hkv, int D, float scale, int causal, void* out, float* lse, int32_t* bounds_ws,
-                          void* stream) {
+                          int bounds_valid, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   int rc = check_attn("varlen_attn_fwd", q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, cu, n_seq, T, Hq, Hkv, D, scale, bounds_ws);
   if (rc) return rc;
@@ -910,11 +922,10 @@ int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long
   fill_attn(p, q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, T, Hq, Hkv, scale, causal, bounds_ws);
   p.out = (bf16_t*)out;
   p.lse = lse;
-  hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
-  HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
-                     const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
-  HIP_TRY(hipGetLastError());
+  if (!bounds_valid) {   // else bounds_ws still holds what an earlier call with the same segments wrote
+    rc = fgrpo_varlen_attn_bounds(cu, n_seq, T, causal, bounds_ws, stream);
+    if (rc) return rc;
+  }
   const long long units = (long long)((T + kAttnBQ - 1) / kAttnBQ) * Hkv;       // (tile, K/V head)
   const dim3 grid((unsigned)(((units + 7) / 8 * 8) * (Hq / Hkv)));
   if (D == 128) hipLaunchKernelGGL(varlen_attn_fwd_kernel<128>, grid, dim3(256), 0, st, p);
@@ -942,12 +953,9 @@ int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const 
   p.dq = (bf16_t*)dq;
   p.dk = (bf16_t*)dk;
   p.dv = (bf16_t*)dv;
-  if (!bounds_valid) {   // else bounds_ws still holds what a forward or backward call with the same segments wrote
-    hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
-    HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(attn_tile_order_kernel, dim3(1), dim3(1024), 0, st, p.seg_start, p.seg_end, T, p.causal,
-                       const_cast<int*>(p.order_q), const_cast<int*>(p.order_k));
-    HIP_TRY(hipGetLastError());
+  if (!bounds_valid) {   // else bounds_ws still holds what an earlier call with the same segments wrote
+    rc = fgrpo_varlen_attn_bounds(cu, n_seq, T, causal, bounds_ws, stream);
+    if (rc) return rc;
   }
   const long long units = (long long)((T + kAttnBQ - 1) / kAttnBQ) * Hkv;       // (tile, K/V head)
   const dim3 grid_q((unsigned)(((units + 7) / 8 * 8) * (Hq / Hkv))), grid_k(Hkv, (T + kAttnBQ - 1) / kAttnBQ);

@@ -572,11 +572,23 @@ def _attn_operand(t: torch.Tensor, name: str) -> torch.Tensor:
     return t if ok else _aligned(t)
 
 
+def _attn_bounds(bounds: Optional[torch.Tensor], T: int, dev):
+    """(buffer, already filled?) for the int32 segment scratch of the attention kernels."""
+    n = 2 * T + 2 * ((T + 127) // 128)
+    if bounds is None:
+        return torch.empty(n, dtype=torch.int32, device=dev), False
+    if bounds.dtype != torch.int32 or bounds.numel() != n or bounds.device != dev or not bounds.is_contiguous():
+        raise RuntimeError("fgrpo: bounds does not come from an attention call of this shape")
+    return bounds, True
+
+
 def varlen_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
-                    softmax_scale: Optional[float] = None, causal: bool = True, return_bounds: bool = False):
+                    softmax_scale: Optional[float] = None, causal: bool = True, return_bounds: bool = False,
+                    bounds: Optional[torch.Tensor] = None):
     """out [T, Hq, D] bf16 and lse [Hq, T] fp32 of packed self-attention: segment i covers tokens
     cu_seqlens[i]:cu_seqlens[i+1]; query head j reads K/V head j // (Hq // Hkv).  ``return_bounds``: also the int32
-    scratch (per-token segment bounds, tile order) that ``varlen_attn_bwd`` can take over instead of rebuilding it."""
+    scratch (per-token segment bounds, tile order) that ``varlen_attn_bwd`` - or the next layer's forward, through
+    ``bounds`` - can take over instead of rebuilding it (same ``cu_seqlens``, ``T`` and ``causal``)."""
     dev = _require_cuda(q, k, v, cu_seqlens)
     lib = _lib.load()
     q, k, v = _attn_operand(q, "q"), _attn_operand(k, "k"), _attn_operand(v, "v")
@@ -588,13 +600,13 @@ def varlen_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlen
     scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
     out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
     lse = torch.empty((Hq, T), dtype=torch.float32, device=dev)
-    bounds = torch.empty(2 * T + 2 * ((T + 127) // 128), dtype=torch.int32, device=dev)
+    bounds, bounds_valid = _attn_bounds(bounds, T, dev)
     if T == 0:
         return (out, lse, bounds) if return_bounds else (out, lse)
     with torch.cuda.device(dev):
         rc = lib.fgrpo_varlen_attn_fwd(_ptr(q), _ptr(k), _ptr(v), q.stride(0), q.stride(1), k.stride(0), k.stride(1),
                                        v.stride(0), v.stride(1), _ptr(cu), cu.numel() - 1, T, Hq, Hkv, D, scale,
-                                       int(bool(causal)), _ptr(out), _ptr(lse), _ptr(bounds), _stream())
+                                       int(bool(causal)), _ptr(out), _ptr(lse), _ptr(bounds), int(bounds_valid), _stream())
     _lib.check(rc, "varlen_attn_fwd")
     return (out, lse, bounds) if return_bounds else (out, lse)
 
@@ -621,12 +633,7 @@ def varlen_attn_bwd(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
     if T == 0:
         return dq, dk, dv
     delta = torch.empty((Hq, T), dtype=torch.float32, device=dev)
-    n_bounds = 2 * T + 2 * ((T + 127) // 128)
-    bounds_valid = bounds is not None
-    if bounds_valid and (bounds.dtype != torch.int32 or bounds.numel() != n_bounds or bounds.device != dev):
-        raise RuntimeError("fgrpo: bounds does not come from a forward call of this shape")
-    if not bounds_valid:
-        bounds = torch.empty(n_bounds, dtype=torch.int32, device=dev)
+    bounds, bounds_valid = _attn_bounds(bounds, T, dev)
     with torch.cuda.device(dev):
         rc = lib.fgrpo_varlen_attn_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), q.stride(0),
                                        q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), _ptr(cu),
@@ -638,8 +645,8 @@ def varlen_attn_bwd(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
 
 class _VarlenAttention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, cu_seqlens, softmax_scale, causal):
-        out, lse, bounds = varlen_attn_fwd(q, k, v, cu_seqlens, softmax_scale, causal, return_bounds=True)
+    def forward(ctx, q, k, v, cu_seqlens, softmax_scale, causal, bounds=None):
+        out, lse, bounds = varlen_attn_fwd(q, k, v, cu_seqlens, softmax_scale, causal, return_bounds=True, bounds=bounds)
         ctx.save_for_backward(q, k, v, out, lse, cu_seqlens, bounds)
         ctx.softmax_scale, ctx.causal = softmax_scale, causal
         return out
@@ -648,9 +655,25 @@ class _VarlenAttention(torch.autograd.Function):
     def backward(ctx, dout):
         q, k, v, out, lse, cu, bounds = ctx.saved_tensors
         dq, dk, dv = varlen_attn_bwd(dout.to(torch.bfloat16), q, k, v, out, lse, cu, ctx.softmax_scale, ctx.causal, bounds)
-        return dq, dk, dv, None, None, None
+        return dq, dk, dv, None, None, None, None
 
 
-def varlen_attention(q, k, v, cu_seqlens, softmax_scale=None, causal=True) -> torch.Tensor:
-    """Differentiable packed self-attention on the HIP kernels (bf16 in, bf16 out)."""
-    return _VarlenAttention.apply(q, k, v, cu_seqlens, softmax_scale, causal)
+def varlen_attention(q, k, v, cu_seqlens, softmax_scale=None, causal=True, bounds=None) -> torch.Tensor:
+    """Differentiable packed self-attention on the HIP kernels (bf16 in, bf16 out).  ``bounds``: segment scratch of an
+    earlier call with the same ``cu_seqlens`` and ``causal`` (see ``attention_bounds``)."""
+    return _VarlenAttention.apply(q, k, v, cu_seqlens, softmax_scale, causal, bounds)
+
+
+def attention_bounds(cu_seqlens: torch.Tensor, T: int, causal: bool = True) -> torch.Tensor:
+    """The int32 segment scratch of the attention kernels for one packed batch, built once so that every layer can
+    pass it as ``bounds``."""
+    dev = _require_cuda(cu_seqlens)
+    lib = _lib.load()
+    cu = cu_seqlens.to(torch.int32).contiguous()
+    bounds, _ = _attn_bounds(None, T, dev)
+    if T > 0:
+        with torch.cuda.device(dev):
+            rc = lib.fgrpo_varlen_attn_bounds(_ptr(cu), cu.numel() - 1, T, int(bool(causal)), _ptr(bounds), _stream())
+        _lib.check(rc, "varlen_attn_bounds")
+    return bounds
+

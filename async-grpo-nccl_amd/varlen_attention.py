@@ -29,6 +29,18 @@ ATTENTION_NAME = "fgrpo_varlen"
 
 # (weak reference to the position_ids tensor, its version counter, result) of the last call
 _cu_cache = {"ref": None, "version": None, "value": None}
+# segment scratch of the attention kernels for the cu_seqlens tensor above: (weak reference, causal, buffer)
+_bounds_cache = {"ref": None, "causal": None, "value": None}
+
+
+def _bounds_for(cu: torch.Tensor, total: int, causal: bool):
+    """The kernels' int32 segment scratch, or None when it has to be built: the layers of one forward pass share
+    the ``cu_seqlens`` tensor object, so the first layer's scratch serves the others."""
+    ref = _bounds_cache["ref"]
+    if ref is not None and ref() is cu and _bounds_cache["causal"] == causal and \
+            _bounds_cache["value"].numel() == 2 * total + 2 * ((total + 127) // 128):
+        return _bounds_cache["value"]
+    return None
 
 
 def prepare_from_position_ids(position_ids: torch.Tensor) -> Tuple[torch.Tensor, int]:
@@ -103,7 +115,12 @@ def varlen_attention_forward(module, query: torch.Tensor, key: torch.Tensor, val
     dt = q.dtype
     if dt != torch.bfloat16:
         q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
-    out = ops.varlen_attention(q, k, v, cu, scaling, bool(is_causal))
+    causal = bool(is_causal)
+    bounds = _bounds_for(cu, B * L, causal) if position_ids is not None else None
+    if bounds is None and position_ids is not None:
+        bounds = ops.attention_bounds(cu, B * L, causal)
+        _bounds_cache["ref"], _bounds_cache["causal"], _bounds_cache["value"] = weakref.ref(cu), causal, bounds
+    out = ops.varlen_attention(q, k, v, cu, scaling, causal, bounds)
     return out.view(B, L, Hq, D).to(dt), None
 
 

@@ -180,11 +180,17 @@ int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long lo
  * strides in elements (multiples of 8), bases 16-byte aligned.  cu_seqlens [n_seq+1] int32 as built
  * at gpu_process_worker.py:239-252 (the same vector for queries and keys).  bounds_ws: 2*T + 2*ceil(T/128) int32
  * of scratch.  out [T, Hq, D] bf16 contiguous; lse [Hq, T] fp32 (natural log of the softmax
- * denominator), needed by the backward.  dropout is not supported (the reference passes 0). */
+ * denominator), needed by the backward.  dropout is not supported (the reference passes 0).
+ * bounds_valid != 0: bounds_ws was filled by an earlier call with the same cu_seqlens, T and causal flag (another
+ * layer of the same batch, or the forward of this backward) and is used as it is; 0: it is (re)built first.
+ * fgrpo_varlen_attn_bounds builds it alone (per-token segment bounds as the wrapper derives them from cu_seqlens,
+ * gpu_process_worker.py:239-252, and the launch order of the tiles). */
+int fgrpo_varlen_attn_bounds(const int32_t* cu_seqlens, int n_seq, int T, int causal, int32_t* bounds_ws,
+                             void* stream);
 int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long q_stride_t, long long q_stride_h,
                           long long k_stride_t, long long k_stride_h, long long v_stride_t, long long v_stride_h,
                           const int32_t* cu_seqlens, int n_seq, int T, int Hq, int Hkv, int D, float softmax_scale,
-                          int causal, void* out, float* lse, int32_t* bounds_ws, void* stream);
+                          int causal, void* out, float* lse, int32_t* bounds_ws, int bounds_valid, void* stream);
 
 /* Backward of the above (autograd of flash_attn_varlen_func in the reference).  dout, out
  * [T, Hq, D] bf16 contiguous; dq [T, Hq, D], dk / dv [T, Hkv, D] bf16 contiguous;

@@ -318,3 +318,21 @@ def test_random_shapes_and_segmentations(dev):
         if rnd.random() < 0.3:
             cu = cu[:1] + [cu[1]] + cu[1:]                  # an empty segment
         check(dev, f"random {case}", T, cu, Hq, Hkv, causal, seed=100 + case, D=D)
+
+
+def test_shared_segment_scratch_gives_identical_results(dev):
+    """The segment scratch built once (ops.attention_bounds) and handed to forward and backward gives bit-identical
+    results to calls that build their own; a scratch of another shape is refused."""
+    from fgrpo import ops
+    q, k, v, do = (x.to(dev) for x in make(700, 4, 2, 31))
+    cu = torch.tensor([0, 5, 300, 301, 700], dtype=torch.int32, device=dev)
+    for causal in (True, False):
+        bounds = ops.attention_bounds(cu, 700, causal)
+        o1, l1 = ops.varlen_attn_fwd(q, k, v, cu, None, causal)
+        o2, l2 = ops.varlen_attn_fwd(q, k, v, cu, None, causal, bounds=bounds)
+        assert torch.equal(o1, o2) and torch.equal(l1, l2)
+        g1 = ops.varlen_attn_bwd(do, q, k, v, o1, l1, cu, None, causal)
+        g2 = ops.varlen_attn_bwd(do, q, k, v, o1, l1, cu, None, causal, bounds=bounds)
+        assert all(torch.equal(a, b) for a, b in zip(g1, g2))
+    with pytest.raises(RuntimeError, match="bounds"):
+        ops.varlen_attn_fwd(q, k, v, cu, None, True, bounds=bounds[:-1])
