@@ -17,7 +17,7 @@
 //    read with ds_read_b64_tr_b16 from the [key][d] tile) simply follows.
 //  * the key-side kernel (dK/dV) computes S = Q K^T, so that a lane owns one key and P / dS feed the
 //    dV = P^T dO and dK = dS^T Q products from registers in the same way.
-// LDS tiles are [row][128] bf16 with the 16-byte chunk index XOR ((row&3)<<2 | (row>>2)&3): conflict-free both
+// LDS tiles are [row][HD] bf16 with the 16-byte chunk index XOR-swizzled by the row (attn_swz): conflict-free both
 // for 16-byte row reads (16 consecutive rows, one chunk) and for the transposing reads (4 consecutive rows x 64 B).
 // Tiles travel global -> registers (bounds-checked buffer loads, issued one step ahead) -> LDS; masks are applied
 // only on steps that can hold a masked pair, and without branches (select before the exponential).
@@ -26,6 +26,8 @@
 // (128 registers) plus its K and V operands and runs one wavefront per SIMD, so its step is software-pipelined
 // by hand (one MFMA per softmax element); splitting it into a dV and a dK launch (two wavefronts per SIMD each,
 // S computed twice) measured slower, as did a second LDS buffer.
+// Launch order: work-groups start in the order of a device-built list, tiles with the most steps first (a third of
+// a launch was tail before), and in the query-side kernels the query heads of one K/V group share an XCD.
 #pragma once
 #include "lmhead_kernels.h"
 
