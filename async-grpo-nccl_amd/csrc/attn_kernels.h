@@ -6,6 +6,9 @@
 // Tiling works on the PACKED token axis: a work-group owns 128 consecutive tokens whatever segments they
 // belong to, and every score is masked with its query's own key range [seg_start[q], q] (causal) or
 // [seg_start[q], seg_end[q]) - so no tile-to-segment map is needed and short segments share tiles.
+// The query-side kernels have a second template argument HB (1, 2 or 4): the four wavefronts of a work-group
+// take HB query heads of one K/V group over 128/HB consecutive tokens, so that one K/V tile in LDS serves several
+// heads and short segments waste fewer masked pairs; HB = 1 is the shape for long segments.
 //
 // MFMA orientation (v_mfma_f32_32x32x16_bf16; operand lane l = row l%32, k values 8*(l/32)..+7; result lane l =
 // column l%32, rows 8*(r/4) + 4*(l/32) + r%4 for r = 0..15):
@@ -45,7 +48,7 @@ struct AttnParams {
   long long q_st, q_sh, k_st, k_sh, v_st, v_sh;
   const int* seg_start;  // [T] first token of the token's segment
   const int* seg_end;    // [T] one past the last token of the token's segment
-  const int* order_q;    // [ceil(T/128)] query tiles, most keys first
+  const int* order_q;    // query tiles (of the launch's tile size: 128, 64 or 32 tokens), most keys first
   const int* order_k;    // [ceil(T/128)] key tiles, most queries first
   int T, Hq, Hkv;
   float scale;
@@ -191,7 +194,7 @@ __device__ __forceinline__ void attn_store_rowmajor(const f32x16_t (&acc)[DB], f
 // ---------------------------------------------------------------------------------------------------------
 // Forward: 1-D grid of round_up(ceil(T/128) * Hkv, 8) * (Hq / Hkv) work-groups, 256 threads.
 // ---------------------------------------------------------------------------------------------------------
-template <int HD>
+template <int HD, int HB>
 __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD;
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
@@ -202,27 +205,33 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
   // 1-D grid over (tile rank, K/V head, query head of the group), most work first.  Work-groups go to the 8 XCDs
   // round-robin (work-group b runs on XCD b % 8, each with its own L2): the query heads of one K/V group - which
   // stream the same K and V rows - are given consecutive slots of ONE XCD, and whole groups go round the XCDs.
-  const int G = p.Hq / p.Hkv;
+  // HB query heads of the group share the work-group (4 / HB wavefronts = RB = 128 / HB tokens each): K and V tiles
+  // are loaded once for all of them, and short tiles waste less on the diagonal and at segment boundaries.
+  constexpr int WPH = 4 / HB, RB = 32 * WPH;
+  const int G = p.Hq / p.Hkv, NB = (G + HB - 1) / HB;     // work-groups per (tile, K/V head)
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int unit = (slot / G) * 8 + xcd;                  // (tile rank, K/V head)
-  if (unit >= (int)((p.T + kAttnBQ - 1) / kAttnBQ) * p.Hkv) return;
-  const int hkv = unit % p.Hkv, hq = hkv * G + slot % G;
-  const int ntile = (p.T + kAttnBQ - 1) / kAttnBQ;
-  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * kAttnBQ;    // clamped: the list may come from the caller
-  const int tq = q0 + 32 * wave + (lane & 31);
-  const bool valid = tq < p.T;
+  const int unit = (slot / NB) * 8 + xcd;                 // (tile rank, K/V head)
+  const int ntile = (p.T + RB - 1) / RB;
+  if (unit >= ntile * p.Hkv) return;
+  const int hkv = unit % p.Hkv;
+  const int head_g = (slot % NB) * HB + wave / WPH;       // this wavefront's query head inside the group
+  const bool head_ok = head_g < G;
+  const int hq = hkv * G + (head_ok ? head_g : G - 1);
+  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * RB;    // clamped: the list may come from the caller
+  const int tq = q0 + 32 * (wave % WPH) + (lane & 31);
+  const bool valid = head_ok && tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
   const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
-  const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
+  const int last = (q0 + RB - 1 < p.T ? q0 + RB - 1 : p.T - 1);
   const int k_begin = max(__builtin_amdgcn_readfirstlane(p.seg_start[q0]), 0);   // wavefront-uniform loop bounds, inside [0, T]
   const int k_end = min(__builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]), p.T);
   // this wavefront's own key range (whole steps outside it are skipped)
-  const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
-  const bool wave_on = wfirst < p.T;
+  const int wfirst = q0 + 32 * (wave % WPH), wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = head_ok && wfirst < p.T;
   const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
   const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
   // keys in [w_lo_max, w_hi_min] are visible to every query of the wavefront (only when all 32 rows exist)
-  const bool wave_full = wfirst + 31 < p.T;
+  const bool wave_full = wave_on && wfirst + 31 < p.T;
   const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
   const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
 
@@ -326,7 +335,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd_kernel(AttnParams p) {
 // dQ: same grid as the forward, 256 threads.  Same walk as the forward; P is rebuilt from the saved log-sum-exp.
 // Also produces delta[hq][t] = sum_d dO[t][hq][d] * O[t][hq][d] (each lane already holds its query's dO row).
 // ---------------------------------------------------------------------------------------------------------
-template <int HD>
+template <int HD, int HB>
 __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD;
   __shared__ __attribute__((aligned(16))) char smem[2 * kAttnTile];
@@ -337,25 +346,31 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq_kernel(AttnParams p) {
   // 1-D grid over (tile rank, K/V head, query head of the group), most work first.  Work-groups go to the 8 XCDs
   // round-robin (work-group b runs on XCD b % 8, each with its own L2): the query heads of one K/V group - which
   // stream the same K and V rows - are given consecutive slots of ONE XCD, and whole groups go round the XCDs.
-  const int G = p.Hq / p.Hkv;
+  // HB query heads of the group share the work-group (4 / HB wavefronts = RB = 128 / HB tokens each): K and V tiles
+  // are loaded once for all of them, and short tiles waste less on the diagonal and at segment boundaries.
+  constexpr int WPH = 4 / HB, RB = 32 * WPH;
+  const int G = p.Hq / p.Hkv, NB = (G + HB - 1) / HB;     // work-groups per (tile, K/V head)
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int unit = (slot / G) * 8 + xcd;                  // (tile rank, K/V head)
-  if (unit >= (int)((p.T + kAttnBQ - 1) / kAttnBQ) * p.Hkv) return;
-  const int hkv = unit % p.Hkv, hq = hkv * G + slot % G;
-  const int ntile = (p.T + kAttnBQ - 1) / kAttnBQ;
-  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * kAttnBQ;    // clamped: the list may come from the caller
-  const int tq = q0 + 32 * wave + (lane & 31);
-  const bool valid = tq < p.T;
+  const int unit = (slot / NB) * 8 + xcd;                 // (tile rank, K/V head)
+  const int ntile = (p.T + RB - 1) / RB;
+  if (unit >= ntile * p.Hkv) return;
+  const int hkv = unit % p.Hkv;
+  const int head_g = (slot % NB) * HB + wave / WPH;       // this wavefront's query head inside the group
+  const bool head_ok = head_g < G;
+  const int hq = hkv * G + (head_ok ? head_g : G - 1);
+  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * RB;    // clamped: the list may come from the caller
+  const int tq = q0 + 32 * (wave % WPH) + (lane & 31);
+  const bool valid = head_ok && tq < p.T;
   const int lo = valid ? p.seg_start[tq] : 1;
   const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
-  const int last = (q0 + kAttnBQ - 1 < p.T ? q0 + kAttnBQ - 1 : p.T - 1);
+  const int last = (q0 + RB - 1 < p.T ? q0 + RB - 1 : p.T - 1);
   const int k_begin = max(__builtin_amdgcn_readfirstlane(p.seg_start[q0]), 0);   // wavefront-uniform loop bounds, inside [0, T]
   const int k_end = min(__builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]), p.T);
-  const int wfirst = q0 + 32 * wave, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
-  const bool wave_on = wfirst < p.T;
+  const int wfirst = q0 + 32 * (wave % WPH), wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = head_ok && wfirst < p.T;
   const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
   const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
-  const bool wave_full = wfirst + 31 < p.T;
+  const bool wave_full = wave_on && wfirst + 31 < p.T;
   const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
   const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
 
@@ -687,49 +702,55 @@ __global__ void segment_bounds_kernel(const int* cu, int nseq, int T, int* seg_s
 }
 
 // Work-group start order: tiles sorted by the number of steps they will walk, most first (ties by index), so that
-// the long tiles of long segments do not end up alone at the tail of the launch.  One work-group of 1024 threads;
-// rank by counting (n <= kAttnMaxSorted tiles), otherwise the plain guess (late query tiles / early key tiles first).
+// the long tiles of long segments do not end up alone at the tail of the launch.  Four lists, one work-group of
+// 1024 threads per eighth of a list: key tiles of 128 tokens, query tiles of 128, 64 and 32 tokens.  Rank by counting
+// (n <= kAttnMaxSorted tiles), otherwise the plain guess (late query tiles / early key tiles first).
+// Layout behind the 2*T per-token bounds: order_k [c128], order_q128 [c128], order_q64 [c64], order_q32 [c32],
+// cX = ceil(T / X).
 constexpr int kAttnMaxSorted = 2048;
-__global__ void attn_tile_order_kernel(const int* seg_start, const int* seg_end, int T, int causal, int* order_q,
-                                       int* order_k) {
-  __shared__ int wq[kAttnMaxSorted], wk[kAttnMaxSorted];
-  const int n = (T + kAttnBQ - 1) / kAttnBQ;
+__host__ __device__ inline long long attn_order_offset(int T, int list) {     // list 0: keys; 1, 2, 3: queries 128 / 64 / 32
+  const long long c128 = (T + 127) / 128, c64 = (T + 63) / 64;
+  return 2LL * T + (list == 0 ? 0 : list == 1 ? c128 : list == 2 ? 2 * c128 : 2 * c128 + c64);
+}
+__host__ __device__ inline long long attn_bounds_elems(int T) { return attn_order_offset(T, 3) + (T + 31) / 32; }
+
+constexpr int kAttnOrderSlices = 8;      // work-groups per list: each ranks 1/8 of the list's tiles
+__global__ void attn_tile_order_kernel(const int* seg_start, const int* seg_end, int T, int causal, int* ws) {
+  __shared__ int wk[kAttnMaxSorted], rk[kAttnMaxSorted / kAttnOrderSlices];
+  const int list = blockIdx.x;                       // 0: keys; 1, 2, 3: queries 128 / 64 / 32
+  const bool keys = list == 0;
+  const int ts = list <= 1 ? 128 : list == 2 ? 64 : 32;
+  int* order = ws + attn_order_offset(T, list);
+  const int n = (T + ts - 1) / ts;
+  const int per = (n + kAttnOrderSlices - 1) / kAttnOrderSlices;
+  const int t0 = blockIdx.y * per, t1 = (t0 + per < n ? t0 + per : n), m = t1 - t0;
+  if (m <= 0) return;
   if (n > kAttnMaxSorted) {
-    for (int t = threadIdx.x; t < n; t += blockDim.x) {
-      order_q[t] = n - 1 - t;
-      order_k[t] = t;
-    }
+    for (int t = t0 + threadIdx.x; t < t1; t += blockDim.x) order[t] = keys ? t : n - 1 - t;
     return;
   }
   for (int t = threadIdx.x; t < n; t += blockDim.x) {
-    const int first = t * kAttnBQ, last = (first + kAttnBQ - 1 < T ? first + kAttnBQ - 1 : T - 1);
-    wq[t] = (causal ? last + 1 : seg_end[last]) - seg_start[first];          // keys a query tile walks
-    wk[t] = seg_end[last] - (causal ? first : seg_start[first]);             // queries a key tile walks
+    const int first = t * ts, last = (first + ts - 1 < T ? first + ts - 1 : T - 1);
+    wk[t] = keys ? seg_end[last] - (causal ? first : seg_start[first])            // queries a key tile walks
+                 : (causal ? last + 1 : seg_end[last]) - seg_start[first];        // keys a query tile walks
   }
+  for (int t = threadIdx.x; t < m; t += blockDim.x) rk[t] = 0;
   __syncthreads();
-  // rank by counting, PARTS threads per tile each scanning 1/PARTS of the list
-  __shared__ int rq[kAttnMaxSorted], rk[kAttnMaxSorted];
-  for (int t = threadIdx.x; t < n; t += blockDim.x) rq[t] = rk[t] = 0;
-  __syncthreads();
-  const int parts = (int)blockDim.x / n > 1 ? (int)blockDim.x / n : 1;
+  // rank by counting, `parts` threads per tile of this slice, each scanning 1/parts of the whole list
+  const int parts = (int)blockDim.x / m > 1 ? (int)blockDim.x / m : 1;
   const int span = (n + parts - 1) / parts;
-  for (int w = threadIdx.x; w < n * parts; w += blockDim.x) {
-    const int t = w / parts, u0 = (w % parts) * span, u1 = (u0 + span < n ? u0 + span : n);
-    const int a = wq[t], b = wk[t];
-    int ra = 0, rb = 0;
+  for (int w = threadIdx.x; w < m * parts; w += blockDim.x) {
+    const int t = t0 + w / parts, u0 = (w % parts) * span, u1 = (u0 + span < n ? u0 + span : n);
+    const int a = wk[t];
+    int r = 0;
     for (int u = u0; u < u1; ++u) {
-      const int x = wq[u], y = wk[u];
-      ra += (x > a) | ((x == a) & (u < t));
-      rb += (y > b) | ((y == b) & (u < t));
+      const int x = wk[u];
+      r += (x > a) | ((x == a) & (u < t));
     }
-    atomicAdd(&rq[t], ra);      // integer counts: the order of the additions does not matter
-    atomicAdd(&rk[t], rb);
+    atomicAdd(&rk[t - t0], r);       // integer counts: the order of the additions does not matter
   }
   __syncthreads();
-  for (int t = threadIdx.x; t < n; t += blockDim.x) {
-    order_q[rq[t]] = t;
-    order_k[rk[t]] = t;
-  }
+  for (int t = threadIdx.x; t < m; t += blockDim.x) order[rk[t]] = t0 + t;
 }
 
 }  // namespace fgrpo

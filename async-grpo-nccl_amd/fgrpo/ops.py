@@ -572,9 +572,15 @@ def _attn_operand(t: torch.Tensor, name: str) -> torch.Tensor:
     return t if ok else _aligned(t)
 
 
+def attention_bounds_numel(T: int) -> int:
+    """int32 elements of the attention kernels' segment scratch for ``T`` packed tokens: start and end of each
+    token's segment, then the launch order of the key tiles (128 tokens) and of the query tiles (128, 64, 32)."""
+    return 2 * T + 2 * ((T + 127) // 128) + (T + 63) // 64 + (T + 31) // 32
+
+
 def _attn_bounds(bounds: Optional[torch.Tensor], T: int, dev):
     """(buffer, already filled?) for the int32 segment scratch of the attention kernels."""
-    n = 2 * T + 2 * ((T + 127) // 128)
+    n = attention_bounds_numel(T)
     if bounds is None:
         return torch.empty(n, dtype=torch.int32, device=dev), False
     if bounds.dtype != torch.int32 or bounds.numel() != n or bounds.device != dev or not bounds.is_contiguous():

@@ -29,18 +29,21 @@ ATTENTION_NAME = "fgrpo_varlen"
 
 # (weak reference to the position_ids tensor, its version counter, result) of the last call
 _cu_cache = {"ref": None, "version": None, "value": None}
-# segment scratch of the attention kernels for the cu_seqlens tensor above: (weak reference, causal, buffer)
-_bounds_cache = {"ref": None, "causal": None, "value": None}
+# segment scratch of the attention kernels for a cu_seqlens tensor: (weak reference, its version counter, causal, buffer)
+_bounds_cache = {"ref": None, "version": None, "causal": None, "value": None}
 
 
-def _bounds_for(cu: torch.Tensor, total: int, causal: bool):
-    """The kernels' int32 segment scratch, or None when it has to be built: the layers of one forward pass share
-    the ``cu_seqlens`` tensor object, so the first layer's scratch serves the others."""
+def _bounds_for(cu: torch.Tensor, total: int, causal: bool) -> torch.Tensor:
+    """The kernels' int32 segment scratch (per-token segment bounds and tile launch order) for ``cu``: built on the
+    first call with a ``cu_seqlens`` tensor OBJECT and reused while that object is alive and unmodified - the
+    layers of one forward pass, and their backward passes, share the tensor."""
     ref = _bounds_cache["ref"]
-    if ref is not None and ref() is cu and _bounds_cache["causal"] == causal and \
-            _bounds_cache["value"].numel() == 2 * total + 2 * ((total + 127) // 128):
+    if ref is not None and ref() is cu and _bounds_cache["version"] == cu._version and \
+            _bounds_cache["causal"] == causal and _bounds_cache["value"].numel() == ops.attention_bounds_numel(total):
         return _bounds_cache["value"]
-    return None
+    bounds = ops.attention_bounds(cu, total, causal)
+    _bounds_cache.update(ref=weakref.ref(cu), version=cu._version, causal=causal, value=bounds)
+    return bounds
 
 
 def prepare_from_position_ids(position_ids: torch.Tensor) -> Tuple[torch.Tensor, int]:
@@ -80,7 +83,8 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q=Non
     if cu_seqlens_q is not cu_seqlens_k:
         if cu_seqlens_q.shape != cu_seqlens_k.shape or not torch.equal(cu_seqlens_q, cu_seqlens_k):
             raise RuntimeError("fgrpo varlen attention: queries and keys must share their segments (self-attention)")
-    return ops.varlen_attention(q, k, v, cu_seqlens_q, softmax_scale, bool(causal))
+    bounds = _bounds_for(cu_seqlens_q, q.shape[0], bool(causal)) if q.is_cuda else None
+    return ops.varlen_attention(q, k, v, cu_seqlens_q, softmax_scale, bool(causal), bounds)
 
 
 def varlen_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
@@ -116,10 +120,7 @@ def varlen_attention_forward(module, query: torch.Tensor, key: torch.Tensor, val
     if dt != torch.bfloat16:
         q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
     causal = bool(is_causal)
-    bounds = _bounds_for(cu, B * L, causal) if position_ids is not None else None
-    if bounds is None and position_ids is not None:
-        bounds = ops.attention_bounds(cu, B * L, causal)
-        _bounds_cache["ref"], _bounds_cache["causal"], _bounds_cache["value"] = weakref.ref(cu), causal, bounds
+    bounds = _bounds_for(cu, B * L, causal) if position_ids is not None and q.is_cuda else None
     out = ops.varlen_attention(q, k, v, cu, scaling, causal, bounds)
     return out.view(B, L, Hq, D).to(dt), None
 

