@@ -334,6 +334,23 @@ def test_random_shapes_and_segmentations(dev):
         check(dev, f"random {case}", T, cu, Hq, Hkv, causal, seed=100 + case, D=D)
 
 
+def test_every_heads_per_work_group_shape(dev):
+    """The forward and dQ kernels come in three shapes (1, 2 or 4 query heads of a K/V group per work-group over
+    128-, 64- or 32-token tiles).  Each is forced in turn over group sizes it divides and does not divide
+    (idle wavefronts past the last head), tile-edge token counts and both masks; the default choice is restored."""
+    from fgrpo import _lib
+    try:
+        for hb in (1, 2, 4):
+            _lib.set_tuning(attn_heads=hb)
+            for i, (T, Hq, Hkv, D, causal) in enumerate([(129, 3, 1, 128, True), (97, 10, 2, 128, True),
+                                                         (300, 6, 1, 64, False), (64, 7, 7, 128, True),
+                                                         (31, 8, 1, 64, True), (513, 5, 1, 128, False)]):
+                cu = [0, T // 3, T // 3 + 1, T]
+                check(dev, f"heads/wg={hb} #{i}", T, cu, Hq, Hkv, causal, seed=300 + 10 * hb + i, D=D)
+    finally:
+        _lib.set_tuning(attn_heads=0)
+
+
 def test_shared_segment_scratch_gives_identical_results(dev):
     """The segment scratch built once (ops.attention_bounds) and handed to forward and backward gives bit-identical
     results to calls that build their own; a scratch of another shape is refused."""
