@@ -75,7 +75,7 @@ struct Tuning {
   int fwd_nsplit = 0;   // 0 = heuristic
   int fwd_group_t = 8;
   int gemm_group_m = 4;
-  int panel_cols = 32768;  // default vocabulary panel width of the backward
+  int panel_cols = 0;      // vocabulary panel width of the backward when the caller gives no bound; 0 = a quarter of [T x V], 2^25 .. 2^30 elements
   int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
   int bwd_kmajor = 2;      // 0: transposed copies; 1: the dW GEMM reads dLogits and hidden in place; 2: the dH GEMM reads W in place too
   int attn_heads = 0;      // query heads per work-group of the attention forward / dQ kernels (1, 2, 4); 0 = heuristic
@@ -217,8 +217,10 @@ int choose_nsplit(int tiles_t, int tiles_v, int slots) {
   // Four splits x eight token tiles (the default raster group) put 32 work-groups = one XCD on an 8 x 4
   // patch of (token tile, vocabulary range): every W slice fetched into that XCD's L2 serves 8 work-groups and
   // every hidden slice 4.  With fewer splits the hidden tiles, which do not fit a 4 MiB L2, are re-fetched per
-  // work-group (measured: 0.94 -> 1.14 PFLOP/s at T=65536, H=3584).  Take it when it costs at most 3% in rounds.
-  if (cap >= 4 && cost_of(4) * 100 <= best_cost * 103) best = 4;
+  // work-group (measured: 0.94 -> 1.14 PFLOP/s at T=65536, H=3584; a 66-tile panel at one split instead of four:
+  // +6 % on the whole backward).  Take it when it costs at most 6% in rounds: rounding a share of 16 or more
+  // tiles up to a multiple of four never costs more.
+  if (cap >= 4 && cost_of(4) * 100 <= best_cost * 106) best = 4;
   return best;
 }
 
@@ -363,6 +365,40 @@ struct BwdPlan {
   size_t bytes;
 };
 
+// Panel budget when the caller gives none: a quarter of the [T x V] matrix, at least 2^25 and at most 2^30 elements
+// (2 GiB of bf16) - the whole matrix is only ever held when it is small.
+long long default_panel_elems(int T, int V) {
+  long long e = (long long)T * V / 4;
+  if (e < (1LL << 25)) e = 1LL << 25;
+  if (e > (1LL << 30)) e = 1LL << 30;
+  return e;
+}
+
+// Panels: at least `np_min` (the memory bound).  Of np_min .. np_min + 3, the count whose dW GEMMs (one tile per
+// 256 vocabulary rows x 256 hidden columns, contraction over all T tokens - the one GEMM of the backward whose
+// tile count depends on the panel width) waste the fewest rounds of the device, plus a fixed cost per panel
+// (three launches' tails and one pass over the fp32 dH accumulator, measured at about 0.15 of such a round).
+// Measured at T=32768, H=1536, V=151936: 8 panels (450 tiles, 1.76 rounds each) 39.1 ms, 7 panels (510 tiles) 38.2.
+int fit_panel_count(int np_min, int H, int V) {
+  const int cus = num_cus(), hT = H / 256, max_np = (V + 255) / 256;
+  if ((long long)((V + np_min - 1) / np_min + 255) / 256 * hT < cus / 2) return np_min;   // small problems: the small-tile path
+  int best = np_min;
+  long long best_cost = -1;
+  for (int np = np_min; np <= np_min + 3 && np <= max_np; ++np) {
+    const int panel = (int)round_up((V + np - 1) / np, 256);
+    long long cost = 0;
+    for (int v0 = 0; v0 < V; v0 += panel) {
+      const int rows = (V - v0) < panel ? (V - v0) : panel;
+      cost += 100LL * ((((long long)(rows + 255) / 256) * hT + cus - 1) / cus) + 15;
+    }
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = np;
+    }
+  }
+  return best;
+}
+
 void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long hint, bool has_bias, bool want_dh,
               bool want_dw) {
   pl.f32 = (dtype == FGRPO_F32);
@@ -373,11 +409,12 @@ void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long h
   pl.Tpad = (int)round_up(T, 256);
   pl.Vpad = (int)round_up(V, 256);
   pl.tiles_t = (T + pl.bn - 1) / pl.bn;
-  long long cols = g_tune.panel_cols;
+  long long cols = g_tune.panel_cols > 0 ? g_tune.panel_cols : default_panel_elems(T, V) / (T > 0 ? T : 1);
   if (hint > 0) cols = hint / (T > 0 ? T : 1);
   if (cols < 256) cols = 256;
   int np = (int)((V + cols - 1) / cols);
   if (np < 1) np = 1;
+  if (!pl.f32 && H % 256 == 0) np = fit_panel_count(np, H, V);
   pl.panel = (int)round_up((V + np - 1) / np, 256);
   pl.npanels = (V + pl.panel - 1) / pl.panel;
   pl.copy_ops = pl.f32 || (H % 64 != 0);

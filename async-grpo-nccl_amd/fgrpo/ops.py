@@ -446,6 +446,17 @@ def _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx):
     return lp, ent, lse_c, h_c, y_c
 
 
+def panel_elems_bound(T: int, V: int, loss_chunksize: Optional[int]) -> int:
+    """Upper bound on the elements of one dLogits panel of the backward, as ``panel_elems_hint``: 0 (the library's
+    own bound: a quarter of ``T * V``, between 2**25 and 2**30 elements) unless the caller's ``loss_chunksize``
+    rows of logits (what the reference holds per chunk, grpo_loss.py:286-313) are more than that."""
+    if loss_chunksize is None or loss_chunksize <= 0:
+        return 0
+    own = min(max(int(T) * int(V) // 4, 1 << 25), 1 << 30)
+    asked = int(loss_chunksize) * int(V)
+    return asked if asked > own else 0
+
+
 def _bwd_rows(h_used, weight, bias, y_used, lse, g_full, gout, temperature, need, panel_hint, idx, hidden_shape):
     g_used = g_full if idx is None else g_full.reshape(-1).index_select(0, idx)
     dH, dW, db = lmhead_bwd(h_used, weight, bias, y_used, lse, g_used, gout, temperature, need[0], need[1], need[2],

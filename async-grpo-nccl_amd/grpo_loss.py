@@ -240,9 +240,10 @@ def grpo_loss_and_entropy_ce_fn(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """6-tuple ``(loss, entropy, log_ratio, loss_clip1, loss_unclipped,
     loss_clipped)`` of the dual-clip token-mean objective (reference:
-    grpo_loss.py:256-348).  ``loss_chunksize`` only bounds the transient of the
-    backward (a dLogits panel of about ``loss_chunksize * V`` elements); the
-    result does not depend on it."""
+    grpo_loss.py:256-348).  ``loss_chunksize`` only widens the transient of the
+    backward (one dLogits panel, bf16) beyond the library's own bound of a
+    quarter of ``[T, V]``, at most 2 GiB, when ``loss_chunksize * V`` elements
+    are more than that; the result does not depend on it."""
     if advantages is None:
         raise ValueError("grpo_loss_and_entropy_ce_fn: advantages are required")
     ref_logprobs = unused_kwargs.get("ref_logprobs", None)
@@ -255,7 +256,7 @@ def grpo_loss_and_entropy_ce_fn(
     shifted = ops.shift_labels(labels).reshape(-1)
     w, b, hs = _prep(lm_head_weights, lm_head_bias, hidden_states)
     V = w.shape[0]
-    hint = int(loss_chunksize) * int(V) if (loss_chunksize is not None and loss_chunksize > 0) else 0
+    hint = ops.panel_elems_bound(hs.shape[0], V, loss_chunksize)
     denom = float(num_samples_total) if (num_samples_total and loss_agg_mode == "sample_mean") else 0.0
     if not _is_own_per_token_fn(per_token_fn):
         lp, ent = _materialised_log_probs_and_entropy(w, b, hidden_states, ops.shift_labels(labels), temperature,

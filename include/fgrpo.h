@@ -68,7 +68,9 @@ int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias,
  * in the workspace at a time.  g [T] fp32 = d loss / d lp; gout_dev = device
  * scalar with the upstream gradient of the loss (NULL = 1); lse [T] from the
  * forward.  dH_out [T x H], dW_out [V x H], dbias_out [V] in `dtype`; each may
- * be NULL.  panel_elems_hint: upper bound on T*panel_width (<=0 = default). */
+ * be NULL.  panel_elems_hint: upper bound on T*panel_width; <=0 = the library's
+ * own bound, a quarter of T*V clamped to 2^25 .. 2^30 elements.  Within the
+ * bound the panel count is fitted to whole rounds of the dW GEMM's tiles. */
 size_t fgrpo_lmhead_bwd_workspace(int T, int H, int V, int dtype, long long panel_elems_hint);
 int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
                      const int64_t* labels_shifted, const float* lse, const float* g,

@@ -62,4 +62,4 @@ def test_argument_errors_are_reported_without_a_gpu(lib_path):
     assert lib.fgrpo_logprob_fwd(None, None, None, None, 1.0, 8, 8, 8, 0, None, None, None, None, 0, None) == -1
     assert lib.fgrpo_logprob_fwd_workspace(32768, 1536, 151936, 0) > 0
     assert lib.fgrpo_lmhead_bwd_workspace(32768, 1536, 151936, 0, 0) > 0
-    assert lib.fgrpo_get_tuning(b"panel_cols") > 0
+    assert lib.fgrpo_get_tuning(b"panel_cols") >= 0
