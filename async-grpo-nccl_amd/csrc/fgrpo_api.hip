@@ -581,6 +581,13 @@ size_t fgrpo_lmhead_bwd_workspace(int T, int H, int V, int dtype, long long hint
   return pl.bytes;
 }
 
+int fgrpo_lmhead_bwd_panel_cols(int T, int H, int V, int dtype, long long hint) {
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_panel_cols: T=%d H=%d V=%d", T, H, V);
+  BwdPlan pl;
+  plan_bwd(pl, nullptr, T, H, V, dtype, hint, true, true, true);
+  return pl.panel;
+}
+
 int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, const int64_t* labels, const float* lse,
                      const float* g, const float* gout_dev, float inv_temp, int T, int H, int V, int dtype,
                      void* dH_out, void* dW_out, void* dbias_out, long long hint, void* ws, size_t ws_bytes,

@@ -72,6 +72,10 @@ int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias,
  * own bound, a quarter of T*V clamped to 2^25 .. 2^30 elements.  Within the
  * bound the panel count is fitted to whole rounds of the dW GEMM's tiles. */
 size_t fgrpo_lmhead_bwd_workspace(int T, int H, int V, int dtype, long long panel_elems_hint);
+/* Vocabulary columns of one dLogits panel that fgrpo_lmhead_bwd will use for these arguments (a multiple of 256;
+ * the backward makes ceil(V / columns) passes).  A query for callers that size or report memory; no counterpart
+ * in the reference, whose chunks are token rows (grpo_loss.py:280-316). */
+int fgrpo_lmhead_bwd_panel_cols(int T, int H, int V, int dtype, long long panel_elems_hint);
 int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
                      const int64_t* labels_shifted, const float* lse, const float* g,
                      const float* gout_dev, float inv_temperature,

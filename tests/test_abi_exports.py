@@ -63,3 +63,29 @@ def test_argument_errors_are_reported_without_a_gpu(lib_path):
     assert lib.fgrpo_logprob_fwd_workspace(32768, 1536, 151936, 0) > 0
     assert lib.fgrpo_lmhead_bwd_workspace(32768, 1536, 151936, 0, 0) > 0
     assert lib.fgrpo_get_tuning(b"panel_cols") >= 0
+
+
+def test_backward_panel_plan_respects_the_bound(lib_path):
+    """The dLogits panel of the backward: a multiple of 256 columns, never above the caller's bound (rounded up to
+    one 256-column block), at most three panels more than the bound alone would need, and by default at most a
+    quarter of [T x V] / 2**30 elements.  Host logic only: no GPU call."""
+    import random
+    from fgrpo import _lib
+    lib = _lib.load()
+    rnd = random.Random(0)
+    cases = [(32768, 1536, 151936), (65536, 3584, 152064), (16384, 8192, 128256), (131072, 5120, 152064),
+             (640, 64, 1000), (4096, 1000, 32000)]
+    for _ in range(40):
+        cases.append((rnd.randrange(1, 70000), rnd.choice([64, 256, 1536, 4096, 1000]), rnd.randrange(1, 200000)))
+    for T, H, V in cases:
+        for hint in (0, 256 * T, 4096 * V, rnd.randrange(1, 1 << 31)):
+            cols = lib.fgrpo_lmhead_bwd_panel_cols(T, H, V, 0, hint)
+            assert cols > 0 and cols % 256 == 0, (T, H, V, hint, cols)
+            bound = hint if hint > 0 else min(max(T * V // 4, 1 << 25), 1 << 30)
+            max_cols = max(bound // T, 256)
+            assert cols <= (max_cols + 255) // 256 * 256, (T, H, V, hint, cols, max_cols)
+            np_min = -(-V // max_cols)
+            assert -(-V // cols) <= np_min + 3, (T, H, V, hint, cols, np_min)
+            assert lib.fgrpo_lmhead_bwd_workspace(T, H, V, 0, hint) >= 2 * cols * T
+    assert lib.fgrpo_lmhead_bwd_panel_cols(32768, 1536, 151936, 0, 0) == 21760      # 7 panels: 510 dW tiles each
+    assert lib.fgrpo_lmhead_bwd_panel_cols(0, 1536, 151936, 0, 0) < 0
