@@ -64,33 +64,26 @@ def get_input_for_logprobs(batched_questions, output_indices, device):
     return dev[0:1], dev[1:2], dev[2:3]
 
 
+# scalar counters of a packed batch (fp32 device scalars), in the reference's key order
+_COUNTER_KEYS = ("num_output_tokens_non_masked", "num_output_tokens", "num_samples", "max_reward_in_group",
+                 "total_modified_reward", "total_non_modified_reward", "num_modified_samples", "delimiter_not_found",
+                 "total_reward_rank", "truncated_sample", "advantage_is_zero")
+
+
 def make_dummy_batch(batched_questions, device):
     """All-masked 4-token placeholder that keeps lock-step ranks busy without
-    touching the metrics (reference: sample_processing_utils.py:127-157)."""
-    ids = [11, 12, 13, 14]
-    z = lambda: torch.tensor(0.0, device=device, dtype=torch.float32)
-    n = len(ids)
-    return {
-        "batch_ids": torch.tensor([ids], dtype=torch.long, device=device),
-        "batch_position_ids": torch.arange(n, device=device).unsqueeze(0),
-        "output_indices": torch.empty((0,), dtype=torch.long, device=device),
-        "advantages": torch.zeros(n, device=device, dtype=torch.float32),
-        "reference_output_logprobs": torch.zeros(n, device=device, dtype=torch.float32),
-        "output_lens_broadcasted": torch.zeros(n, device=device, dtype=torch.float32),
-        "num_output_tokens_non_masked": z(),
-        "num_output_tokens": z(),
-        "num_samples": z(),
-        "max_reward_in_group": z(),
-        "total_modified_reward": z(),
-        "total_non_modified_reward": z(),
-        "num_modified_samples": z(),
-        "delimiter_not_found": z(),
-        "samples": batched_questions,
-        "labels": torch.full((1, n), -100, dtype=torch.long, device=device),
-        "total_reward_rank": z(),
-        "truncated_sample": z(),
-        "advantage_is_zero": z(),
-    }
+    touching the metrics (reference: sample_processing_utils.py:127-157): every
+    label is -100, there are no output positions, every counter is zero."""
+    n = 4
+    batch = {key: torch.zeros((), device=device, dtype=torch.float32) for key in _COUNTER_KEYS}
+    for key in ("advantages", "reference_output_logprobs", "output_lens_broadcasted"):
+        batch[key] = torch.zeros(n, device=device, dtype=torch.float32)
+    batch["batch_ids"] = torch.arange(11, 11 + n, dtype=torch.long, device=device).unsqueeze(0)
+    batch["batch_position_ids"] = torch.arange(n, device=device).unsqueeze(0)
+    batch["labels"] = torch.full((1, n), -100, dtype=torch.long, device=device)
+    batch["output_indices"] = torch.empty((0,), dtype=torch.long, device=device)
+    batch["samples"] = batched_questions
+    return batch
 
 
 def post_process_batch(batched_questions, device, constant_length_samples=None):

@@ -73,6 +73,27 @@ def test_post_process_batch_matches_oracle(dev):
     assert (const["output_lens_broadcasted"] == 7).all()
     dummy = spu.post_process_batch([{"dummy": True}], dev)
     assert dummy["labels"].eq(-100).all() and dummy["output_indices"].numel() == 0
+    # the dummy batch has the key set of a real one (reference: sample_processing_utils.py:137-157), zero counters,
+    # four tokens, and the same dtypes
+    assert set(dummy) == {"batch_ids", "batch_position_ids", "output_indices", "advantages", "reference_output_logprobs",
+                          "output_lens_broadcasted", "num_output_tokens_non_masked", "num_output_tokens", "num_samples",
+                          "max_reward_in_group", "total_modified_reward", "total_non_modified_reward",
+                          "num_modified_samples", "delimiter_not_found", "samples", "labels", "total_reward_rank",
+                          "truncated_sample", "advantage_is_zero"}
+    assert set(dummy) <= set(got), sorted(set(dummy) - set(got))
+    assert dummy["batch_ids"].tolist() == [[11, 12, 13, 14]] and dummy["batch_position_ids"].tolist() == [[0, 1, 2, 3]]
+    for k, v in dummy.items():
+        if k == "samples":
+            continue
+        assert v.dtype == got[k].dtype, k
+        if v.dim() == 0:
+            assert v.item() == 0.0, k
+    # the two helpers post_process_batch is built from (reference: sample_processing_utils.py:107-125)
+    idx, out_lens = spu.get_output_logits_indices(samples, dev)
+    assert torch.equal(idx.cpu(), want["output_indices"]) and list(out_lens) == [s["output_len"] for s in samples]
+    ids, pos, lab = spu.get_input_for_logprobs(samples, idx, dev)
+    for a, key in ((ids, "batch_ids"), (pos, "batch_position_ids"), (lab, "labels")):
+        assert a.dtype == torch.long and torch.equal(a.cpu(), want[key]), key
 
 
 def test_segment_kernels(dev):
