@@ -74,6 +74,10 @@ struct Tuning {
   int gemm_variant = 8;
   int fwd_nsplit = 0;   // 0 = heuristic
   int fwd_group_t = 8;
+  int ds_nsplit = 0;    // dLogits kernel: vocabulary splits of a panel; 0 = as the forward
+  int ds_group_t = 0;   // dLogits kernel: token tiles per raster group; 0 = as the forward
+  int dh_group_m = 0;   // dHidden GEMM raster group; 0 = gemm_group_m
+  int dw_group_m = 0;   // dW GEMM raster group; 0 = gemm_group_m
   int gemm_group_m = 4;
   int panel_cols = 0;      // vocabulary panel width of the backward when the caller gives no bound; 0 = a quarter of [T x V], 2^25 .. 2^30 elements
   int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
@@ -88,6 +92,10 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "gemm_variant")) return &g_tune.gemm_variant;
   if (!strcmp(key, "fwd_nsplit")) return &g_tune.fwd_nsplit;
   if (!strcmp(key, "fwd_group_t")) return &g_tune.fwd_group_t;
+  if (!strcmp(key, "ds_nsplit")) return &g_tune.ds_nsplit;
+  if (!strcmp(key, "ds_group_t")) return &g_tune.ds_group_t;
+  if (!strcmp(key, "dh_group_m")) return &g_tune.dh_group_m;
+  if (!strcmp(key, "dw_group_m")) return &g_tune.dw_group_m;
   if (!strcmp(key, "gemm_group_m")) return &g_tune.gemm_group_m;
   if (!strcmp(key, "panel_cols")) return &g_tune.panel_cols;
   if (!strcmp(key, "small_variant")) return &g_tune.small_variant;
@@ -196,8 +204,8 @@ struct FwdPlan {
   size_t bytes;
 };
 
-int choose_nsplit(int tiles_t, int tiles_v, int slots) {
-  if (g_tune.fwd_nsplit > 0) return g_tune.fwd_nsplit < tiles_v ? g_tune.fwd_nsplit : tiles_v;
+int choose_nsplit(int tiles_t, int tiles_v, int slots, int forced, int prefer = 4) {
+  if (forced > 0) return forced < tiles_v ? forced : tiles_v;
   int best = 1;
   long long best_cost = -1;
   const int cap = tiles_v < 64 ? tiles_v : 64;
@@ -220,6 +228,9 @@ int choose_nsplit(int tiles_t, int tiles_v, int slots) {
   // work-group (measured: 0.94 -> 1.14 PFLOP/s at T=65536, H=3584; a 66-tile panel at one split instead of four:
   // +6 % on the whole backward).  Take it when it costs at most 6% in rounds: rounding a share of 16 or more
   // tiles up to a multiple of four never costs more.
+  // The dLogits kernel, which also writes its tile, measures 1-2 % better on the whole backward with eight splits
+  // and two token tiles per group (`prefer` = 8); it falls back to four, then to the cheapest.
+  if (prefer != 4 && cap >= prefer && cost_of(prefer) * 100 <= best_cost * 106) return prefer;
   if (cap >= 4 && cost_of(4) * 100 <= best_cost * 106) best = 4;
   return best;
 }
@@ -229,7 +240,7 @@ void plan_fwd(FwdPlan& pl, void* ws, int T, int H, int V, int dtype, bool has_bi
   const CfgInfo& c = kCfg[pl.variant];
   pl.tiles_v = (V + c.bm - 1) / c.bm;
   pl.tiles_t = (T + c.bn - 1) / c.bn;
-  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu);
+  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu, g_tune.fwd_nsplit);
   pl.Hp = (int)round_up(H, 64);
   pl.copy_ops = (dtype == FGRPO_F32) || (H % 64 != 0);
   Carver cv(ws);
@@ -326,7 +337,10 @@ int run_store_gemm_kmajor(StoreParams p, bool akm, bool bkm, hipStream_t st) {
   if (bkm && (long long)p.tiles_n * Cfg8::BN > g.ldb) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): ldb < padded N");
   if (256LL * g.lda * 2 >= (1LL << 32) || 256LL * g.ldb * 2 >= (1LL << 32))
     return fail(FGRPO_ERR_UNSUPPORTED, "gemm(k-major): leading dimension too large");
-  p.group_m = g_tune.gemm_group_m > 0 ? g_tune.gemm_group_m : 1;
+  {
+    const int own = (akm && bkm) ? g_tune.dw_group_m : g_tune.dh_group_m;
+    p.group_m = own > 0 ? own : (g_tune.gemm_group_m > 0 ? g_tune.gemm_group_m : 1);
+  }
   const int nb = p.tiles_m * p.tiles_n;
   if (akm && bkm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, true, true>, p, nb, st);
   if (akm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, true, false>, p, nb, st);
@@ -634,7 +648,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
   d.gout = gout_dev;
   d.inv_temp = inv_temp;
   d.tiles_t = pl.tiles_t;
-  d.group_t = g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1;
+  d.group_t = g_tune.ds_group_t > 0 ? g_tune.ds_group_t : (g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1);
   d.tv_hi = pl.tv_hi;
   d.tv_lo = pl.tv_lo;
   d.vt_hi = pl.vt_hi;
@@ -651,7 +665,11 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
     const int rows = (V - v0) < pl.panel ? (V - v0) : pl.panel;
     d.v0 = v0;
     d.tiles_v = (rows + pl.bm - 1) / pl.bm;
-    d.nsplit = choose_nsplit(pl.tiles_t, d.tiles_v, num_cus() * kCfg[pl.variant].wgs_per_cu);
+    d.nsplit = choose_nsplit(pl.tiles_t, d.tiles_v, num_cus() * kCfg[pl.variant].wgs_per_cu,
+                             g_tune.ds_nsplit > 0 ? g_tune.ds_nsplit : g_tune.fwd_nsplit, 8);
+    d.group_t = g_tune.ds_group_t > 0 ? g_tune.ds_group_t
+                : d.nsplit == 8        ? 2       // 2 token tiles x 8 splits: half an XCD's work-groups per patch
+                : g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1;
     const int kv = d.tiles_v * pl.bm;        // written panel width
     const int kt = pl.tiles_t * pl.bn;       // written token extent
     if (f32) {
