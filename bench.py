@@ -245,6 +245,8 @@ def main():
         "ms_per_step_median": per_step[len(per_step) // 2], "ms_per_step_min": per_step[0],
         "path_mfma_frac": alg_flops_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "path_algorithmic_tflops": alg_flops_step / (ms * 1e-3) / 1e12,
+        # what the matrix pipeline executes: the backward recomputes the logits once (nothing [T x V] is kept)
+        "path_executed_tflops": (2.0 if fwd_only else 8.0) * T * H * V / (ms * 1e-3) / 1e12,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.config, p["chunk"], args.seed)
