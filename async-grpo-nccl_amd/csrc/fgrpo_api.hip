@@ -901,12 +901,12 @@ int fgrpo_logits_logprob_entropy(const void* logits, int dtype, long long ld, in
 
 int fgrpo_logits_logprob_bwd(const void* logits, int dtype, long long ld, int N, int V, const int64_t* labels,
                              long long ignore_index, int use_ignore, const float* g, const float* lse, void* dlogits,
-                             void* stream) {
-  if (!logits || !labels || !g || !lse || !dlogits || N <= 0 || V <= 0 || ld < V)
+                             long long ld_out, void* stream) {
+  if (!logits || !labels || !g || !lse || !dlogits || N <= 0 || V <= 0 || ld < V || ld_out < V)
     return fail(FGRPO_ERR_BAD_ARG, "logits_logprob_bwd: bad argument");
   if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "logits_logprob_bwd: dtype=%d", dtype);
   RowBwdParams p{{logits, dtype == FGRPO_F32, ld, N, V, (const long long*)labels, ignore_index, use_ignore, nullptr, nullptr, nullptr},
-                 g, lse, dlogits};
+                 g, lse, dlogits, ld_out};
   hipLaunchKernelGGL(logits_row_bwd_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, p);
   HIP_TRY(hipGetLastError());
   return 0;

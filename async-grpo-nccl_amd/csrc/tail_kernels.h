@@ -366,47 +366,69 @@ __device__ __forceinline__ float row_load(const RowParams& p, long long row, int
   return p.is_f32 ? ((const float*)p.logits)[o] : bf16_to_f32(((const bf16_t*)p.logits)[o]);
 }
 
+// eight consecutive elements of a row as floats: one 16-byte load for bf16, two for fp32 (the row must start on a
+// 16-byte boundary and c counts chunks of eight)
+template <bool F32>
+__device__ __forceinline__ void row_load8(const void* row_base, int c, float (&x)[8]) {
+  if constexpr (F32) {
+    const float4* b = (const float4*)row_base + 2 * (long long)c;
+    const float4 lo = b[0], hi = b[1];
+    x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w;
+    x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
+  } else {
+    const uint4 q = ((const uint4*)row_base)[c];
+    const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      x[2 * k] = __uint_as_float(u[k] << 16);
+      x[2 * k + 1] = __uint_as_float(u[k] & 0xffff0000u);
+    }
+  }
+}
+
+// running (max, sum exp, sum exp * x) of one thread over the chunks c = first, first + 256, ... of a row
+template <bool F32>
+__device__ __forceinline__ void row_stats_chunks(const void* row_base, int nv, float& m, float& s, float& sx) {
+  for (int c = threadIdx.x; c < nv; c += 256) {
+    float x[8];
+    row_load8<F32>(row_base, c, x);
+    float mt = x[0];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) mt = fmaxf(mt, x[k]);
+    const float mn = fmaxf(m, mt);
+    const float al = fast_exp2((m - mn) * kLog2e);
+    s *= al;
+    sx *= al;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float e = fast_exp2((x[k] - mn) * kLog2e);
+      s += e;
+      sx = __builtin_fmaf(e, x[k], sx);
+    }
+    m = mn;
+  }
+}
+
+__device__ __forceinline__ bool row_vectorisable(const RowParams& p) {
+  return (p.ld % 8 == 0) && ((((uintptr_t)p.logits) & 15) == 0);
+}
+
 __global__ __launch_bounds__(256) void logits_row_stats_kernel(const RowParams p) {
   __shared__ float sh[3][4];
   const long long row = blockIdx.x;
   float m = kNegBig, s = 0.f, sx = 0.f;
-  const bool vec = (p.ld % 8 == 0) && ((((uintptr_t)p.logits) & 15) == 0);
-  if (!p.is_f32 && vec) {
-    const uint4* base = (const uint4*)((const bf16_t*)p.logits + row * p.ld);
+  int done = 0;                      // elements covered by the 16-byte loop
+  if (row_vectorisable(p)) {
     const int nv = p.V / 8;
-    for (int c = threadIdx.x; c < nv; c += 256) {
-      const uint4 q = base[c];
-      const uint32_t u[4] = {q.x, q.y, q.z, q.w};
-      float x[8];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        x[2 * k] = __uint_as_float(u[k] << 16);
-        x[2 * k + 1] = __uint_as_float(u[k] & 0xffff0000u);
-      }
-      float mt = x[0];
-#pragma unroll
-      for (int k = 1; k < 8; ++k) mt = fmaxf(mt, x[k]);
-      const float mn = fmaxf(m, mt);
-      const float al = fast_exp2((m - mn) * kLog2e);
-      s *= al;
-      sx *= al;
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const float e = fast_exp2((x[k] - mn) * kLog2e);
-        s += e;
-        sx = __builtin_fmaf(e, x[k], sx);
-      }
-      m = mn;
-    }
-    for (int v = nv * 8 + threadIdx.x; v < p.V; v += 256) {
-      const float x = row_load(p, row, v);
-      lse_merge(m, s, sx, x, 1.f, x);
-    }
-  } else {
-    for (int v = threadIdx.x; v < p.V; v += 256) {
-      const float x = row_load(p, row, v);
-      lse_merge(m, s, sx, x, 1.f, x);
-    }
+    if (p.is_f32)
+      row_stats_chunks<true>((const float*)p.logits + row * p.ld, nv, m, s, sx);
+    else
+      row_stats_chunks<false>((const bf16_t*)p.logits + row * p.ld, nv, m, s, sx);
+    done = nv * 8;
+  }
+  for (int v = done + threadIdx.x; v < p.V; v += 256) {
+    const float x = row_load(p, row, v);
+    lse_merge(m, s, sx, x, 1.f, x);
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -445,7 +467,8 @@ struct RowBwdParams {
   RowParams f;
   const float* g;       // [N] upstream gradient of lp
   const float* lse;     // [N]
-  void* dlogits;        // same dtype/ld as logits
+  void* dlogits;        // [N x V] in the logits' dtype, rows ld_out elements apart
+  long long ld_out;
 };
 
 __global__ __launch_bounds__(256) void logits_row_bwd_kernel(const RowBwdParams p) {
@@ -454,11 +477,48 @@ __global__ __launch_bounds__(256) void logits_row_bwd_kernel(const RowBwdParams 
   const bool ign = p.f.use_ignore && lab == p.f.ignore;
   const float g = ign ? 0.f : p.g[row];
   const float l2 = p.lse[row] * kLog2e;
-  for (int v = threadIdx.x; v < p.f.V; v += 256) {
+  int done = 0;
+  if (row_vectorisable(p.f) && p.ld_out % 8 == 0 && ((((uintptr_t)p.dlogits) & 15) == 0)) {
+    // eight elements per thread and step: 16-byte loads and stores (two each for fp32)
+    const int nv = p.f.V / 8;
+    const int lab_chunk = (lab >= 0 && lab < p.f.V) ? (int)(lab >> 3) : -1, lab_k = (int)(lab & 7);
+    for (int c = threadIdx.x; c < nv; c += 256) {
+      float x[8], d[8];
+      if (ign) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) d[k] = 0.f;          // nothing to read: the row takes no gradient
+      } else {
+        if (p.f.is_f32)
+          row_load8<true>((const float*)p.f.logits + row * p.f.ld, c, x);
+        else
+          row_load8<false>((const bf16_t*)p.f.logits + row * p.f.ld, c, x);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) d[k] = -g * fast_exp2(__builtin_fmaf(x[k], kLog2e, -l2));
+        if (c == lab_chunk) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) d[k] += (k == lab_k) ? g : 0.f;
+        }
+      }
+      if (p.f.is_f32) {
+        float4* o = (float4*)((float*)p.dlogits + row * p.ld_out) + 2 * (long long)c;
+        o[0] = make_float4(d[0], d[1], d[2], d[3]);
+        o[1] = make_float4(d[4], d[5], d[6], d[7]);
+      } else {
+        uint4 q;
+        q.x = pack_bf16x2(d[0], d[1]);
+        q.y = pack_bf16x2(d[2], d[3]);
+        q.z = pack_bf16x2(d[4], d[5]);
+        q.w = pack_bf16x2(d[6], d[7]);
+        ((uint4*)((bf16_t*)p.dlogits + row * p.ld_out))[c] = q;
+      }
+    }
+    done = nv * 8;
+  }
+  for (int v = done + threadIdx.x; v < p.f.V; v += 256) {
     const float x = row_load(p.f, row, v);
     float d = -g * fast_exp2(__builtin_fmaf(x, kLog2e, -l2));
     if (v == lab) d += g;
-    const long long o = row * p.f.ld + v;
+    const long long o = row * p.ld_out + v;
     if (p.f.is_f32)
       ((float*)p.dlogits)[o] = d;
     else

@@ -38,7 +38,7 @@ SIGNATURES = {
     "fgrpo_output_indices": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
     "fgrpo_segment_starts": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "fgrpo_logits_logprob_entropy": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _vp]),
-    "fgrpo_logits_logprob_bwd": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _vp]),
+    "fgrpo_logits_logprob_bwd": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _ll, _vp]),
     "fgrpo_gemm_nt": (_i, [_vp, _vp, _i, _i, _i, _ll, _ll, _vp, _vp, _vp, _ll, _f, _i, _vp]),
     "fgrpo_gemm_kmajor": (_i, [_vp, _vp, _i, _i, _i, _ll, _ll, _i, _i, _ll, _i, _vp, _vp, _vp, _ll, _f, _vp]),
     "fgrpo_varlen_attn_bounds": (_i, [_vp, _i, _i, _i, _vp, _vp]),

@@ -369,7 +369,7 @@ def logits_logprob_bwd(logits, labels, ignore_index, g, lse) -> torch.Tensor:
         rc = lib.fgrpo_logits_logprob_bwd(_ptr(logits), _code(logits.dtype), logits.stride(0), N, V, _ptr(lab),
                                           int(ignore_index if ignore_index is not None else 0),
                                           int(ignore_index is not None), _ptr(_f32(g, N, "g")), _ptr(_f32(lse, N, "lse")),
-                                          _ptr(out), _stream())
+                                          _ptr(out), out.stride(0), _stream())
     _lib.check(rc, "logits_logprob_bwd")
     return out
 

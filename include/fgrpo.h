@@ -150,13 +150,14 @@ int fgrpo_segment_starts(const int64_t* position_ids, int T, int32_t* cu_out, in
  * (grpo_loss.py:203-208) for callers that already hold logits [N x V] (ld =
  * row stride in elements).  labels may be NULL when lp is NULL.  use_ignore = 0
  * disables the ignore_index test.  The backward writes
- * dlogits = g (onehot - softmax) in the logits' dtype. */
+ * dlogits = g (onehot - softmax) in the logits' dtype, rows ld_out elements apart
+ * (ld_out >= V; the rows of logits and dlogits need not share a stride). */
 int fgrpo_logits_logprob_entropy(const void* logits, int dtype, long long ld, int N, int V,
                                  const int64_t* labels, long long ignore_index, int use_ignore,
                                  float* lp, float* ent, float* lse, void* stream);
 int fgrpo_logits_logprob_bwd(const void* logits, int dtype, long long ld, int N, int V,
                              const int64_t* labels, long long ignore_index, int use_ignore,
-                             const float* g, const float* lse, void* dlogits, void* stream);
+                             const float* g, const float* lse, void* dlogits, long long ld_out, void* stream);
 
 /* ---- test hook: the GEMM core on its own -----------------------------------------
  * C[m,n] = alpha * sum_k A[m,k] B[n,k] (+ c_in); A [M x K], B [N x K] bf16,

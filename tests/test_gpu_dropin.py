@@ -169,6 +169,33 @@ def test_row_kernels_on_materialised_logits(dev, dtype):
     assert (lpn.float().cpu() - O.logprobs_from_logits(x.float(), y.clamp(min=0), None)).abs().max() <= tol
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V,ld", [(1003, 1008), (1024, 1024), (1003, 1003), (5, 8), (2400, 2400)])
+def test_row_kernels_vector_and_tail_paths(dev, dtype, V, ld):
+    """Rows that start on 16-byte boundaries are read and written 16 bytes at a time with a scalar tail (V % 8),
+    others element by element; labels are placed at chunk edges, inside the tail and on ignored rows."""
+    import grpo_loss as G
+    g = torch.Generator().manual_seed(V + ld)
+    N = 9
+    buf = (torch.randn(N, ld, generator=g) * 3).to(dtype)
+    x = buf[:, :V]
+    y = torch.tensor([0, min(7, V - 1), min(8, V - 1), V - 1, V - 2, V // 2, -100, (V - 1) // 8 * 8, 3 % V])
+    xg = buf.to(dev)[:, :V].requires_grad_(True)
+    assert xg.stride(0) == ld
+    lp = G.logprobs_from_logits_flash_attn(xg, y.to(dev))
+    want = O.logprobs_from_logits(x.float(), y)
+    assert (lp.cpu() - want).abs().max() <= 1e-5
+    ent = G.entropy_from_logits(xg.detach())
+    assert (ent.float().cpu() - O.entropy_from_logits(x.float())).abs().max() <= (1e-5 if dtype == torch.float32 else 0.04)
+    w = torch.randn(N, generator=g)
+    (lp * w.to(dev)).sum().backward()
+    xo = x.float().requires_grad_(True)
+    (O.logprobs_from_logits(xo, y) * w).sum().backward()
+    rel = (xg.grad.float().cpu() - xo.grad).norm() / xo.grad.norm()
+    assert rel <= (1e-5 if dtype == torch.float32 else 5e-3)
+    assert xg.grad[6].abs().max() == 0                       # the ignored row
+
+
 def _patched(dev, mode, dtype=torch.float32, chunk=None, temperature=1.0):
     import grpo_loss as G
     torch.manual_seed(0)
