@@ -818,7 +818,7 @@ int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, co
     // tokens outside every segment keep weight 0
     hipLaunchKernelGGL(fill_f32_kernel, dim3((T + 255) / 256), dim3(256), 0, st, tokw, 0.f, T);
     HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(segment_valid_weight_kernel, dim3((nseq + 3) / 4), dim3(256), 0, st, p.labels, cu, nseq, segc,
+    hipLaunchKernelGGL(segment_valid_weight_kernel, dim3((nseq + 3) / 4), dim3(256), 0, st, p.labels, cu, nseq, T, segc,
                        tokw);
     HIP_TRY(hipGetLastError());
     p.tokw = tokw;
@@ -843,37 +843,40 @@ int fgrpo_metrics(const int64_t* idx, int n, int T, const float* log_ratio, cons
   return 0;
 }
 
-int fgrpo_group_advantages(const void* rewards, int rewards_f64, const int32_t* goff, int ngroups, double eps,
-                           float* out_f32, double* out_f64, void* stream) {
-  if (!rewards || !goff || ngroups <= 0 || (!out_f32 && !out_f64)) return fail(FGRPO_ERR_BAD_ARG, "group_advantages: bad argument");
+int fgrpo_group_advantages(const void* rewards, int rewards_f64, const int32_t* goff, int ngroups, int n_rewards,
+                           double eps, float* out_f32, double* out_f64, void* stream) {
+  if (!rewards || !goff || ngroups <= 0 || n_rewards < 0 || (!out_f32 && !out_f64))
+    return fail(FGRPO_ERR_BAD_ARG, "group_advantages: bad argument");
   hipLaunchKernelGGL(group_advantage_kernel, dim3((ngroups + 3) / 4), dim3(256), 0, (hipStream_t)stream, rewards,
-                     rewards_f64, goff, ngroups, eps, out_f32, out_f64);
+                     rewards_f64, goff, ngroups, n_rewards, eps, out_f32, out_f64);
   HIP_TRY(hipGetLastError());
   return 0;
 }
 
-int fgrpo_segment_broadcast(const void* values, int values_f64, const int32_t* cu, int nseq, float* out, void* stream) {
-  if (!values || !cu || !out || nseq <= 0) return fail(FGRPO_ERR_BAD_ARG, "segment_broadcast: bad argument");
+int fgrpo_segment_broadcast(const void* values, int values_f64, const int32_t* cu, int nseq, int T, float* out,
+                            void* stream) {
+  if (!values || !cu || !out || nseq <= 0 || T < 0) return fail(FGRPO_ERR_BAD_ARG, "segment_broadcast: bad argument");
   hipLaunchKernelGGL(segment_broadcast_kernel, dim3((nseq + 3) / 4), dim3(256), 0, (hipStream_t)stream, values,
-                     values_f64, cu, nseq, out);
+                     values_f64, cu, nseq, T, out);
   HIP_TRY(hipGetLastError());
   return 0;
 }
 
-int fgrpo_segment_reduce(const float* x, const int64_t* labels, const int32_t* cu, int nseq, float* sum_out,
+int fgrpo_segment_reduce(const float* x, const int64_t* labels, const int32_t* cu, int nseq, int T, float* sum_out,
                          float* mean_out, int32_t* count_out, void* stream) {
-  if (!x || !cu || nseq <= 0) return fail(FGRPO_ERR_BAD_ARG, "segment_reduce: bad argument");
+  if (!x || !cu || nseq <= 0 || T < 0) return fail(FGRPO_ERR_BAD_ARG, "segment_reduce: bad argument");
   hipLaunchKernelGGL(segment_reduce_kernel, dim3((nseq + 3) / 4), dim3(256), 0, (hipStream_t)stream, x,
-                     (const long long*)labels, cu, nseq, sum_out, mean_out, count_out);
+                     (const long long*)labels, cu, nseq, T, sum_out, mean_out, count_out);
   HIP_TRY(hipGetLastError());
   return 0;
 }
 
 int fgrpo_output_indices(const int32_t* tok_off, const int32_t* in_len, const int32_t* out_off, int nsamples,
-                         int64_t* out, void* stream) {
-  if (!tok_off || !in_len || !out_off || !out || nsamples <= 0) return fail(FGRPO_ERR_BAD_ARG, "output_indices: bad argument");
+                         int n_out, int64_t* out, void* stream) {
+  if (!tok_off || !in_len || !out_off || !out || nsamples <= 0 || n_out < 0)
+    return fail(FGRPO_ERR_BAD_ARG, "output_indices: bad argument");
   hipLaunchKernelGGL(output_indices_kernel, dim3((nsamples + 3) / 4), dim3(256), 0, (hipStream_t)stream, tok_off, in_len,
-                     out_off, nsamples, (long long*)out);
+                     out_off, nsamples, n_out, (long long*)out);
   HIP_TRY(hipGetLastError());
   return 0;
 }

@@ -26,6 +26,14 @@ __device__ __forceinline__ int wave_sum_i(int v) {
   return v;
 }
 
+// Offsets read from device memory (cu_seqlens, group offsets) are clamped into [0, n] and made monotone before
+// they index anything: a malformed vector then yields wrong numbers for its own rows, never an access outside
+// the arrays.
+__device__ __forceinline__ void clamp_range(int& b, int& e, int n) {
+  b = b < 0 ? 0 : (b > n ? n : b);
+  e = e < b ? b : (e > n ? n : e);
+}
+
 __global__ void fill_f32_kernel(float* dst, float v, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = v;
@@ -36,11 +44,12 @@ __global__ void fill_f32_kernel(float* dst, float v, int n) {
 // ---------------------------------------------------------------------------
 // cnt[s] = number of valid (label != -100) tokens of segment s; tokw[t] = 1/cnt
 // of the token's segment (0 when the segment has no valid token).
-__global__ void segment_valid_weight_kernel(const long long* labels, const int* cu, int nseq, int* cnt, float* tokw) {
+__global__ void segment_valid_weight_kernel(const long long* labels, const int* cu, int nseq, int T, int* cnt, float* tokw) {
   const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (s >= nseq) return;
-  const int b = cu[s], e = cu[s + 1];
+  int b = cu[s], e = cu[s + 1];
+  clamp_range(b, e, T);
   int c = 0;
   for (int t = b + lane; t < e; t += 64) c += (labels[t] != -100);
   c = wave_sum_i(c);
@@ -50,23 +59,27 @@ __global__ void segment_valid_weight_kernel(const long long* labels, const int* 
 }
 
 // out[t] = values[s] for every token of segment s
-__global__ void segment_broadcast_kernel(const void* values, int values_f64, const int* cu, int nseq, float* out) {
+__global__ void segment_broadcast_kernel(const void* values, int values_f64, const int* cu, int nseq, int T, float* out) {
   const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (s >= nseq) return;
   const float v = values_f64 ? (float)((const double*)values)[s] : ((const float*)values)[s];
-  for (int t = cu[s] + lane; t < cu[s + 1]; t += 64) out[t] = v;
+  int b = cu[s], e = cu[s + 1];
+  clamp_range(b, e, T);
+  for (int t = b + lane; t < e; t += 64) out[t] = v;
 }
 
 // sum[s], and mean[s] = sum / count over the (optionally masked) tokens of segment s
-__global__ void segment_reduce_kernel(const float* x, const long long* labels, const int* cu, int nseq, float* sum,
+__global__ void segment_reduce_kernel(const float* x, const long long* labels, const int* cu, int nseq, int T, float* sum,
                                       float* mean, int* count) {
   const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (s >= nseq) return;
   float a = 0.f;
   int c = 0;
-  for (int t = cu[s] + lane; t < cu[s + 1]; t += 64) {
+  int b = cu[s], e = cu[s + 1];
+  clamp_range(b, e, T);
+  for (int t = b + lane; t < e; t += 64) {
     const bool ok = labels ? (labels[t] != -100) : true;
     a += ok ? x[t] : 0.f;
     c += ok;
@@ -85,13 +98,14 @@ __global__ void segment_reduce_kernel(const float* x, const long long* labels, c
 //   tok_off[i] + in_len[i] - 1 + j   for j in [0, out_len[i])
 // written at out_off[i] + j.  One wavefront per sample.
 __global__ void output_indices_kernel(const int* tok_off, const int* in_len, const int* out_off, int nsamples,
-                                      long long* out) {
+                                      int n_out, long long* out) {
   const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (s >= nsamples) return;
-  const int n = out_off[s + 1] - out_off[s];
+  int b = out_off[s], e = out_off[s + 1];
+  clamp_range(b, e, n_out);
   const long long first = (long long)tok_off[s] + in_len[s] - 1;
-  for (int j = lane; j < n; j += 64) out[out_off[s] + j] = first + j;
+  for (int j = lane; j < e - b; j += 64) out[b + j] = first + j;
 }
 
 // cu_seqlens from position ids: ordered list of the indices t with pos[t] == 0,
@@ -131,12 +145,13 @@ __global__ __launch_bounds__(1024) void segment_starts_kernel(const long long* p
 }
 
 // adv[i] = (r[i] - mean_g) / (std_pop_g + eps) per group, double arithmetic
-__global__ void group_advantage_kernel(const void* rewards, int rewards_f64, const int* goff, int ngroups, double eps,
-                                       float* out_f32, double* out_f64) {
+__global__ void group_advantage_kernel(const void* rewards, int rewards_f64, const int* goff, int ngroups, int n_rewards,
+                                       double eps, float* out_f32, double* out_f64) {
   const int g = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (g >= ngroups) return;
-  const int b = goff[g], e = goff[g + 1];
+  int b = goff[g], e = goff[g + 1];
+  clamp_range(b, e, n_rewards);
   auto rd = [&](int i) -> double {
     return rewards_f64 ? ((const double*)rewards)[i] : (double)((const float*)rewards)[i];
   };

@@ -32,10 +32,10 @@ SIGNATURES = {
     "fgrpo_loss_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _f, _f, _i, _d,
                             _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgrpo_metrics": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _vp]),
-    "fgrpo_group_advantages": (_i, [_vp, _i, _vp, _i, _d, _vp, _vp, _vp]),
-    "fgrpo_segment_broadcast": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
-    "fgrpo_segment_reduce": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp]),
-    "fgrpo_output_indices": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
+    "fgrpo_group_advantages": (_i, [_vp, _i, _vp, _i, _i, _d, _vp, _vp, _vp]),
+    "fgrpo_segment_broadcast": (_i, [_vp, _i, _vp, _i, _i, _vp, _vp]),
+    "fgrpo_segment_reduce": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
+    "fgrpo_output_indices": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp]),
     "fgrpo_segment_starts": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "fgrpo_logits_logprob_entropy": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _vp]),
     "fgrpo_logits_logprob_bwd": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _ll, _vp]),

@@ -249,7 +249,7 @@ def group_advantages(rewards: torch.Tensor, group_offsets: torch.Tensor, eps: fl
         raise RuntimeError("fgrpo: out_dtype must be float32 or float64")
     with torch.cuda.device(dev):
         rc = lib.fgrpo_group_advantages(_ptr(rewards), int(rewards.dtype == torch.float64), _ptr(goff),
-                                        goff.numel() - 1, float(eps), o32, o64, _stream())
+                                        goff.numel() - 1, rewards.numel(), float(eps), o32, o64, _stream())
     _lib.check(rc, "group_advantages")
     return out
 
@@ -267,7 +267,7 @@ def segment_broadcast(values: torch.Tensor, cu_seqlens: torch.Tensor, total: int
         return out
     with torch.cuda.device(dev):
         rc = lib.fgrpo_segment_broadcast(_ptr(values), int(values.dtype == torch.float64), _ptr(cu), cu.numel() - 1,
-                                         _ptr(out), _stream())
+                                         int(total), _ptr(out), _stream())
     _lib.check(rc, "segment_broadcast")
     return out
 
@@ -283,9 +283,11 @@ def segment_reduce(x: torch.Tensor, cu_seqlens: torch.Tensor, labels_shifted: Op
     m = torch.empty(n, dtype=torch.float32, device=dev)
     c = torch.empty(n, dtype=torch.int32, device=dev)
     lab = None if labels_shifted is None else labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    if lab is not None and lab.numel() != x.numel():
+        raise RuntimeError("fgrpo: labels must have one entry per token")
     if n > 0:
         with torch.cuda.device(dev):
-            rc = lib.fgrpo_segment_reduce(_ptr(x), _ptr(lab), _ptr(cu), n, _ptr(s), _ptr(m), _ptr(c), _stream())
+            rc = lib.fgrpo_segment_reduce(_ptr(x), _ptr(lab), _ptr(cu), n, x.numel(), _ptr(s), _ptr(m), _ptr(c), _stream())
         _lib.check(rc, "segment_reduce")
     return s, m, c
 
@@ -310,7 +312,7 @@ def output_indices(input_lens, output_lens, device) -> torch.Tensor:
     pack = torch.cat([tok_off.to(torch.int32), il.to(torch.int32), out_off.to(torch.int32)]).to(device)
     with torch.cuda.device(device):
         rc = lib.fgrpo_output_indices(pack.data_ptr(), pack.data_ptr() + 4 * n, pack.data_ptr() + 8 * n, n,
-                                      _ptr(out), _stream())
+                                      total, _ptr(out), _stream())
     _lib.check(rc, "output_indices")
     return out
 

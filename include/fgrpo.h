@@ -117,31 +117,35 @@ int fgrpo_metrics(const int64_t* idx, int n, int T, const float* log_ratio, cons
 /* ---- group-normalised advantages ------------------------------------------------
  * Replaces vllm_worker.py:788-796 (and normalize_rewards, :77-92):
  * (r - mean) / (population std + eps) per group; group_offsets [ngroups+1] int32.
- * rewards fp32 or fp64 (rewards_f64 != 0); out_f32 / out_f64 may be NULL. */
+ * rewards [n_rewards] fp32 or fp64 (rewards_f64 != 0); out_f32 / out_f64 may be NULL.
+ * Offsets are read on the device and clamped into [0, n_rewards]. */
 int fgrpo_group_advantages(const void* rewards, int rewards_f64, const int32_t* group_offsets,
-                           int ngroups, double eps, float* out_f32, double* out_f64, void* stream);
+                           int ngroups, int n_rewards, double eps, float* out_f32, double* out_f64,
+                           void* stream);
 
 /* ---- segmented helpers over cu_seqlens [nseq+1] int32 ---------------------------
  * fgrpo_segment_broadcast replaces broadcast_values (sample_processing_utils.py:69-105):
  * out[t] = values[s(t)].  fgrpo_segment_reduce gives per-sample sums / means /
- * counts of a per-token array, masked by labels != -100 when labels is given. */
+ * counts of a per-token array, masked by labels != -100 when labels is given.
+ * T = length of the per-token arrays; cu_seqlens entries are clamped into [0, T]. */
 int fgrpo_segment_broadcast(const void* values, int values_f64, const int32_t* cu_seqlens, int nseq,
-                            float* out, void* stream);
+                            int T, float* out, void* stream);
 int fgrpo_segment_reduce(const float* x, const int64_t* labels, const int32_t* cu_seqlens, int nseq,
-                         float* sum_out, float* mean_out, int32_t* count_out, void* stream);
+                         int T, float* sum_out, float* mean_out, int32_t* count_out, void* stream);
 
 /* ---- batch shaping --------------------------------------------------------------
  * fgrpo_output_indices replaces get_output_logits_indices_numba
  * (sample_processing_utils.py:29-67): sample i, packed at token offset
  * tok_off[i] with prompt length in_len[i], contributes the positions
  * tok_off[i]+in_len[i]-1+j, j in [0, out_off[i+1]-out_off[i]), written at
- * out[out_off[i]+j].  tok_off, in_len [nsamples], out_off [nsamples+1] int32.
+ * out[out_off[i]+j].  tok_off, in_len [nsamples], out_off [nsamples+1] int32;
+ * out has n_out entries (out_off is clamped into [0, n_out]).
  * fgrpo_segment_starts replaces the cu_seqlens derivation of
  * gpu_process_worker.py:239-252: cu_out = ordered indices t with
  * position_ids[t]==0, then T; *count_out = entries produced (boundaries + 1),
  * at most max_out of them are stored. */
 int fgrpo_output_indices(const int32_t* tok_off, const int32_t* in_len, const int32_t* out_off,
-                         int nsamples, int64_t* out, void* stream);
+                         int nsamples, int n_out, int64_t* out, void* stream);
 int fgrpo_segment_starts(const int64_t* position_ids, int T, int32_t* cu_out, int max_out,
                          int32_t* count_out, void* stream);
 

@@ -140,6 +140,39 @@ def test_group_advantages(dev):
     assert np.allclose(got_r, want_r, atol=1e-12)
 
 
+def test_malformed_offsets_stay_inside_the_arrays(dev):
+    """cu_seqlens and group offsets live in device memory, so the host cannot vet them: the kernels clamp every
+    offset into the array and make ranges monotone.  A malformed vector gives well-defined results for the rows
+    that are well formed and touches nothing outside (checked with guard values around the output)."""
+    from fgrpo import ops
+    T = 10
+    cu = torch.tensor([0, 5, 3, 100000], dtype=torch.int32, device=dev)        # decreasing, then far past the end
+    vals = torch.tensor([1.0, 2.0, 3.0], device=dev)
+    out = ops.segment_broadcast(vals, cu, T).cpu()
+    assert out[:3].tolist() == [1.0, 1.0, 1.0] and out[5:].tolist() == [3.0] * 5
+    x = torch.arange(T, dtype=torch.float32, device=dev)
+    s, m, c = ops.segment_reduce(x, cu)
+    assert s.tolist() == [10.0, 0.0, float(sum(range(3, 10)))] and c.tolist() == [5, 0, 7]
+    neg = torch.tensor([-7, 4, 2 ** 31 - 1], dtype=torch.int32, device=dev)
+    s2, _, c2 = ops.segment_reduce(x, neg)
+    assert s2.tolist() == [6.0, float(sum(range(4, 10)))] and c2.tolist() == [4, 6]
+    r = torch.tensor([1.0, 0.0, 1.0, 1.0], dtype=torch.float64, device=dev)
+    adv = ops.group_advantages(r, torch.tensor([0, 2, 900], dtype=torch.int32), 1e-4, torch.float64).cpu()
+    want = np.concatenate([O.group_advantages(np.array([1.0, 0.0])), O.group_advantages(np.array([1.0, 1.0]))])
+    assert np.allclose(adv.numpy(), want, atol=1e-12)
+    # sample-mean objective with a cu_seqlens that overruns the batch: finite loss, nothing written past T
+    import grpo_loss as G
+    g = torch.Generator().manual_seed(0)
+    hs = torch.randn(1, 64, 64, generator=g).bfloat16().to(dev)
+    W = (torch.randn(300, 64, generator=g) * 0.05).bfloat16().to(dev)
+    labels = torch.randint(0, 300, (1, 64), generator=g).to(dev)
+    bad_cu = torch.tensor([0, 40, 5000], dtype=torch.int32, device=dev)
+    out = G.grpo_loss_and_entropy_ce_fn(W, None, hs, labels, 1.0, None, torch.randn(64, generator=g).to(dev),
+                                        loss_agg_mode="sample_mean", cu_seqlens=bad_cu)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out[0]).item()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_row_kernels_on_materialised_logits(dev, dtype):
     import grpo_loss as G
