@@ -881,6 +881,20 @@ int fgrpo_output_indices(const int32_t* tok_off, const int32_t* in_len, const in
   return 0;
 }
 
+int fgrpo_build_labels(const int64_t* ids, const int32_t* tok_off, const int32_t* in_len, const int32_t* out_len,
+                       int nsamples, int T, int64_t* labels_out, void* stream) {
+  if (!ids || !tok_off || !in_len || !out_len || !labels_out || nsamples <= 0 || T <= 0)
+    return fail(FGRPO_ERR_BAD_ARG, "build_labels: bad argument");
+  hipStream_t st = (hipStream_t)stream;
+  // tokens outside every sample are masked
+  hipLaunchKernelGGL(fill_i64_kernel, dim3((T + 255) / 256), dim3(256), 0, st, (long long*)labels_out, -100LL, T);
+  HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(build_labels_kernel, dim3((nsamples + 3) / 4), dim3(256), 0, st, (const long long*)ids, tok_off,
+                     in_len, out_len, nsamples, T, (long long*)labels_out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 int fgrpo_segment_starts(const int64_t* position_ids, int T, int32_t* cu_out, int max_out, int32_t* count_out,
                          void* stream) {
   if (!position_ids || !cu_out || !count_out || T <= 0 || max_out <= 0) return fail(FGRPO_ERR_BAD_ARG, "segment_starts: bad argument");

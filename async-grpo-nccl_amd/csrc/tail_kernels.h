@@ -38,6 +38,10 @@ __global__ void fill_f32_kernel(float* dst, float v, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = v;
 }
+__global__ void fill_i64_kernel(long long* dst, long long v, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = v;
+}
 
 // ---------------------------------------------------------------------------
 // Segment (sample) statistics over cu_seqlens: one wavefront per segment.
@@ -106,6 +110,22 @@ __global__ void output_indices_kernel(const int* tok_off, const int* in_len, con
   clamp_range(b, e, n_out);
   const long long first = (long long)tok_off[s] + in_len[s] - 1;
   for (int j = lane; j < e - b; j += 64) out[b + j] = first + j;
+}
+
+// Training labels of a packed batch: inside sample i (tokens tok_off[i] .. tok_off[i+1]) the generated span
+// [in_len[i], in_len[i] + out_len[i]) keeps its token id, everything else is -100.  One wavefront per sample.
+__global__ void build_labels_kernel(const long long* ids, const int* tok_off, const int* in_len, const int* out_len,
+                                    int nsamples, int T, long long* labels) {
+  const int s = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (s >= nsamples) return;
+  int b = tok_off[s], e = tok_off[s + 1];
+  clamp_range(b, e, T);
+  const int lo = in_len[s], hi = lo + out_len[s];
+  for (int t = b + lane; t < e; t += 64) {
+    const int k = t - b;
+    labels[t] = (k >= lo && k < hi) ? ids[t] : -100;
+  }
 }
 
 // cu_seqlens from position ids: ordered list of the indices t with pos[t] == 0,

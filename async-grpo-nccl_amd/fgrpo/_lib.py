@@ -36,6 +36,7 @@ SIGNATURES = {
     "fgrpo_segment_broadcast": (_i, [_vp, _i, _vp, _i, _i, _vp, _vp]),
     "fgrpo_segment_reduce": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "fgrpo_output_indices": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "fgrpo_build_labels": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "fgrpo_segment_starts": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "fgrpo_logits_logprob_entropy": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _vp]),
     "fgrpo_logits_logprob_bwd": (_i, [_vp, _i, _ll, _i, _i, _vp, _ll, _i, _vp, _vp, _vp, _ll, _vp]),

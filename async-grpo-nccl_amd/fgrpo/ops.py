@@ -317,6 +317,36 @@ def output_indices(input_lens, output_lens, device) -> torch.Tensor:
     return out
 
 
+def build_labels(ids: torch.Tensor, input_lens, output_lens) -> torch.Tensor:
+    """Labels of a packed batch built on the device: ``ids`` [T] (or [1, T]) int64 on the GPU, sample i made of
+    ``input_lens[i]`` prompt tokens and ``output_lens[i]`` generated ones; returns int64 of ``ids``' shape with the
+    generated tokens kept and -100 elsewhere (what vllm_worker.py:768-774 builds per sample on the host)."""
+    dev = _require_cuda(ids)
+    lib = _lib.load()
+    flat = ids.reshape(-1).to(torch.int64).contiguous()
+    T = flat.numel()
+    il = torch.as_tensor(input_lens, dtype=torch.int64).reshape(-1)
+    ol = torch.as_tensor(output_lens, dtype=torch.int64).reshape(-1)
+    n = il.numel()
+    if ol.numel() != n:
+        raise RuntimeError("fgrpo: input_lens and output_lens must have one entry per sample")
+    if int((il + ol).sum()) != T:
+        raise RuntimeError(f"fgrpo: the samples hold {int((il + ol).sum())} tokens, ids has {T}")
+    out = torch.empty_like(flat)
+    if T == 0 or n == 0:
+        return out.view(ids.shape)
+    if T >= 2 ** 31:
+        raise RuntimeError("fgrpo: packed batch longer than 2^31 tokens")
+    tok_off = torch.zeros(n + 1, dtype=torch.int64)
+    tok_off[1:] = torch.cumsum(il + ol, 0)
+    pack = torch.cat([tok_off, il, ol]).to(torch.int32).to(dev)
+    base = pack.data_ptr()
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_build_labels(_ptr(flat), base, base + 4 * (n + 1), base + 4 * (2 * n + 1), n, T, _ptr(out), _stream())
+    _lib.check(rc, "build_labels")
+    return out.view(ids.shape)
+
+
 def cu_seqlens_from_position_ids(position_ids: torch.Tensor, max_segments: Optional[int] = None) -> torch.Tensor:
     """int32 [n+1]: indices where position_ids == 0, then T (one host sync for n)."""
     dev = _require_cuda(position_ids)

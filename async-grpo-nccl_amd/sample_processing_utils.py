@@ -50,18 +50,25 @@ def get_output_logits_indices(batched_questions, device):
 def get_input_for_logprobs(batched_questions, output_indices, device):
     """Concatenated ids / position ids / labels as [1, T] int64 device tensors
     (reference: sample_processing_utils.py:114-125).  One pinned staging buffer,
-    one copy."""
+    one copy.  Samples that carry no ``labels`` get them built on the device from
+    ``input_len`` / ``output_len`` (the rule of vllm_worker.py:768-774)."""
     n_tok = sum(len(s["sample_ids"]) for s in batched_questions)
-    host = torch.empty((3, n_tok), dtype=torch.long).pin_memory() if n_tok else torch.empty((3, 0), dtype=torch.long)
+    have_labels = all("labels" in s for s in batched_questions)
+    rows = 3 if have_labels else 2
+    host = torch.empty((rows, n_tok), dtype=torch.long).pin_memory() if n_tok else torch.empty((rows, 0), dtype=torch.long)
     off = 0
     for s in batched_questions:
         k = len(s["sample_ids"])
         host[0, off:off + k] = torch.as_tensor(s["sample_ids"], dtype=torch.long)
         host[1, off:off + k] = torch.as_tensor(s["sample_position_ids"], dtype=torch.long)
-        host[2, off:off + k] = torch.as_tensor(s["labels"], dtype=torch.long)
+        if have_labels:
+            host[2, off:off + k] = torch.as_tensor(s["labels"], dtype=torch.long)
         off += k
     dev = host.to(device, non_blocking=True)
-    return dev[0:1], dev[1:2], dev[2:3]
+    if have_labels:
+        return dev[0:1], dev[1:2], dev[2:3]
+    il, ol = _lens(batched_questions)
+    return dev[0:1], dev[1:2], ops.build_labels(dev[0:1], il, ol)
 
 
 # scalar counters of a packed batch (fp32 device scalars), in the reference's key order

@@ -148,6 +148,13 @@ int fgrpo_output_indices(const int32_t* tok_off, const int32_t* in_len, const in
                          int nsamples, int n_out, int64_t* out, void* stream);
 int fgrpo_segment_starts(const int64_t* position_ids, int T, int32_t* cu_out, int max_out,
                          int32_t* count_out, void* stream);
+/* fgrpo_build_labels replaces the per-sample label loop of the rollout worker
+ * (vllm_worker.py:768-774) for a packed batch that is already on the device:
+ * inside sample i (tokens tok_off[i] .. tok_off[i+1] of ids [T]) the generated
+ * span [in_len[i], in_len[i]+out_len[i]) keeps its token id, every other
+ * position is -100.  tok_off [nsamples+1], in_len, out_len [nsamples] int32. */
+int fgrpo_build_labels(const int64_t* ids, const int32_t* tok_off, const int32_t* in_len,
+                       const int32_t* out_len, int nsamples, int T, int64_t* labels_out, void* stream);
 
 /* ---- row soft-max on materialised logits ----------------------------------------
  * Replaces logprobs_from_logits (grpo_loss.py:146-173) and entropy_from_logits

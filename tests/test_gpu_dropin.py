@@ -88,6 +88,14 @@ def test_post_process_batch_matches_oracle(dev):
         assert v.dtype == got[k].dtype, k
         if v.dim() == 0:
             assert v.item() == 0.0, k
+    # labels built on the device when the samples carry none (the rule of vllm_worker.py:768-774)
+    bare = [{k: v for k, v in smp.items() if k != "labels"} for smp in samples]
+    got_bare = spu.post_process_batch(bare, dev)
+    assert torch.equal(got_bare["labels"].cpu(), want["labels"])
+    assert got_bare["num_output_tokens_non_masked"].item() == got["num_output_tokens_non_masked"].item()
+    from fgrpo import ops as _ops
+    with pytest.raises(RuntimeError):
+        _ops.build_labels(got["batch_ids"], [1, 2], [3, 4])                 # lens do not add up to the batch
     # the two helpers post_process_batch is built from (reference: sample_processing_utils.py:107-125)
     idx, out_lens = spu.get_output_logits_indices(samples, dev)
     assert torch.equal(idx.cpu(), want["output_indices"]) and list(out_lens) == [s["output_len"] for s in samples]
