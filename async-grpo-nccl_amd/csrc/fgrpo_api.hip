@@ -834,12 +834,21 @@ int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, co
 
 int fgrpo_metrics(const int64_t* idx, int n, int T, const float* log_ratio, const float* entropy,
                   const float* old_entropy, const float* adv, const float* unclipped, const float* clipped,
-                  float clip_low, float clip_high, double* stats_out, void* stream) {
+                  float clip_low, float clip_high, double* stats_out, double* partial_ws, void* stream) {
   if (!stats_out || n < 0 || T <= 0) return fail(FGRPO_ERR_BAD_ARG, "metrics: bad argument");
   if (n > 0 && (!idx || !log_ratio || !adv || !unclipped || !clipped)) return fail(FGRPO_ERR_BAD_ARG, "metrics: null argument");
-  MetricParams p{(const long long*)idx, n, T, log_ratio, entropy, old_entropy, adv, unclipped, clipped, clip_low, clip_high, stats_out};
-  hipLaunchKernelGGL(grpo_metrics_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, p);
+  // one work-group per 2048 positions, at most kMetricBlocks; without scratch (or for few positions) a single one
+  int nb = partial_ws ? (n + 2047) / 2048 : 1;
+  nb = nb < 1 ? 1 : (nb > kMetricBlocks ? kMetricBlocks : nb);
+  MetricParams p{(const long long*)idx, n, T, log_ratio, entropy, old_entropy, adv, unclipped, clipped, clip_low, clip_high,
+                 nb == 1 ? stats_out : partial_ws};
+  hipLaunchKernelGGL(grpo_metrics_kernel, dim3(nb), dim3(1024), 0, (hipStream_t)stream, p);
   HIP_TRY(hipGetLastError());
+  if (nb > 1) {
+    hipLaunchKernelGGL(grpo_metrics_reduce_kernel, dim3(1), dim3(64 * kNumStats), 0, (hipStream_t)stream, partial_ws, nb,
+                       stats_out);
+    HIP_TRY(hipGetLastError());
+  }
   return 0;
 }
 

@@ -332,15 +332,16 @@ struct MetricParams {
   const float* unclipped;    // [T]
   const float* clipped;      // [T]
   float clip_low, clip_high;
-  double* stats;             // [kNumStats]
+  double* stats;             // [kNumStats] (one work-group) or [gridDim.x][kNumStats] partial sums
 };
+constexpr int kMetricBlocks = 128;     // most work-groups of the first stage
 
 __global__ __launch_bounds__(1024) void grpo_metrics_kernel(const MetricParams p) {
   __shared__ double sh[kNumStats][16];
   double a[kNumStats];
 #pragma unroll
   for (int k = 0; k < kNumStats; ++k) a[k] = 0.0;
-  for (int i = threadIdx.x; i < p.n; i += 1024) {
+  for (long long i = (long long)blockIdx.x * 1024 + threadIdx.x; i < p.n; i += (long long)gridDim.x * 1024) {
     long long t = p.idx[i];
     if (t < 0) t += p.T;  // python-style negative index
     if (t < 0 || t >= p.T) {
@@ -375,8 +376,18 @@ __global__ __launch_bounds__(1024) void grpo_metrics_kernel(const MetricParams p
   if (threadIdx.x < kNumStats) {
     double v = 0.0;
     for (int w = 0; w < 16; ++w) v += sh[threadIdx.x][w];
-    p.stats[threadIdx.x] = v;
+    p.stats[(long long)blockIdx.x * kNumStats + threadIdx.x] = v;
   }
+}
+
+// second stage: one wavefront per statistic; lane l adds the partial sums of work-groups l, l + 64, ... and the 64
+// lanes are combined by the same butterfly every time (a fixed order: two runs agree bit for bit)
+__global__ __launch_bounds__(64 * kNumStats) void grpo_metrics_reduce_kernel(const double* partial, int nblocks, double* stats) {
+  const int k = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  double v = 0.0;
+  for (int b = lane; b < nblocks; b += 64) v += partial[(long long)b * kNumStats + k];
+  v = wave_sum_d(v);
+  if (lane == 0) stats[k] = v;
 }
 
 // ---------------------------------------------------------------------------

@@ -14,6 +14,7 @@ ERR = {-1: "bad argument", -2: "unsupported", -3: "workspace", -4: "HIP error", 
 BF16, F32 = 0, 1
 AGG_TOKEN_MEAN, AGG_SAMPLE_MEAN = 0, 1
 NUM_STATS = 16
+METRIC_BLOCKS = 128      # work-groups of the diagnostics' first stage (FGRPO_METRIC_BLOCKS)
 
 _vp, _i, _ll, _f, _d, _sz = C.c_void_p, C.c_int, C.c_longlong, C.c_float, C.c_double, C.c_size_t
 
@@ -31,7 +32,7 @@ SIGNATURES = {
     "fgrpo_loss_fwd_workspace": (_sz, [_i, _i]),
     "fgrpo_loss_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _f, _f, _i, _d,
                             _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "fgrpo_metrics": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _vp]),
+    "fgrpo_metrics": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _vp, _vp]),
     "fgrpo_group_advantages": (_i, [_vp, _i, _vp, _i, _i, _d, _vp, _vp, _vp]),
     "fgrpo_segment_broadcast": (_i, [_vp, _i, _vp, _i, _i, _vp, _vp]),
     "fgrpo_segment_reduce": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),

@@ -215,18 +215,20 @@ def grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens=None,
 
 def grpo_metrics(output_indices, log_ratio, entropy, old_entropy, adv, unclipped, clipped,
                  clip_low: float, clip_high: float) -> torch.Tensor:
-    """One launch, one [16] float64 device vector (layout in include/fgrpo.h)."""
+    """One [16] float64 device vector (layout in include/fgrpo.h): partial sums per work-group, added in a fixed
+    order by a second small launch when there are more than 2048 positions."""
     dev = _require_cuda(log_ratio, adv)
     lib = _lib.load()
     T = log_ratio.numel()
     idx = output_indices.to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
-    stats = torch.zeros(_lib.NUM_STATS, dtype=torch.float64, device=dev)
+    buf = torch.zeros(_lib.NUM_STATS * (1 + _lib.METRIC_BLOCKS), dtype=torch.float64, device=dev)
+    stats, partial = buf[:_lib.NUM_STATS], buf[_lib.NUM_STATS:]
     with torch.cuda.device(dev):
         rc = lib.fgrpo_metrics(_ptr(idx), idx.numel(), T, _ptr(_f32(log_ratio, T, "log_ratio")),
                                _ptr(_f32(entropy, T, "entropy")), _ptr(_f32(old_entropy, T, "old_entropy")),
                                _ptr(_f32(adv, T, "advantages")), _ptr(_f32(unclipped, T, "unclipped")),
                                _ptr(_f32(clipped, T, "clipped")), float(clip_low), float(clip_high),
-                               _ptr(stats), _stream())
+                               _ptr(stats), _ptr(partial), _stream())
     _lib.check(rc, "metrics")
     return stats
 

@@ -137,6 +137,84 @@ def attention_line(args):
     }), flush=True)
 
 
+def hbm_line(args):
+    """The bandwidth-bound kernels of the path at a size where bandwidth, not launch latency, decides: the
+    per-token objective (loss_fwd = token kernel + normaliser), the diagnostics, the segmented reductions and
+    broadcasts over cu_seqlens, and the row kernels on materialised logits.  Algorithmic bytes per kernel are the
+    arrays it must read and write once; times are HIP-event brackets on the launch stream."""
+    import torch
+    from fgrpo import ops
+    import grpo_loss as G
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    g = torch.Generator().manual_seed(args.seed)
+    PEAK = 8000.0
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    rows = []
+    for T in (32768, 1 << 20):
+        lens = []
+        while sum(lens) < T:
+            lens.append(int(torch.randint(128, 1025, (1,), generator=g)))
+        lens[-1] -= sum(lens) - T
+        cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+        lp = (-torch.rand(T, generator=g) * 3).to(dev)
+        old = lp + 0.01 * torch.randn(T, generator=g).to(dev)
+        ref = lp + 0.05 * torch.randn(T, generator=g).to(dev)
+        adv = torch.randn(T, generator=g).to(dev)
+        y = torch.randint(0, 1000, (T,), generator=g).to(dev)
+        idx = torch.nonzero(y >= 0).reshape(-1)
+        per_seg = torch.randn(len(lens), generator=g).to(dev)
+        # loss: reads lp, old, ref, adv (4 B each) and labels (8 B); writes g and four diagnostics; g is read and
+        # written once more by the normaliser
+        ms = timed(lambda: ops.grpo_loss_fwd(lp, old, ref, adv, y, None, 0.2, 0.2, 3.0, 0.01))
+        rows.append((f"objective (token + normaliser kernels), T={T}", T * (4 * 4 + 8 + 5 * 4 + 8), ms))
+        out = ops.grpo_loss_fwd(lp, old, ref, adv, y, None, 0.2, 0.2, 3.0, 0.01)
+        ms = timed(lambda: ops.grpo_metrics(idx, out[2], lp, None, adv, out[4], out[5], 0.2, 0.2))
+        rows.append((f"diagnostics (two-stage sum), T={T}", T * (8 + 5 * 4), ms))
+        ms = timed(lambda: ops.segment_reduce(lp, cu, y))
+        rows.append((f"segment_reduce over cu_seqlens, T={T}", T * (4 + 8), ms))
+        ms = timed(lambda: ops.segment_broadcast(per_seg, cu, T))
+        rows.append((f"segment_broadcast (incl. torch zero fill), T={T}", T * 8, ms))
+    for dt in (torch.bfloat16, torch.float32):
+        N, V = 4096, 151936
+        x = torch.randn(N, V, device=dev, dtype=dt)
+        yy = torch.randint(0, V, (N,), device=dev)
+        nb = x.numel() * x.element_size()
+        ms = timed(lambda: G.logprobs_from_logits_flash_attn(x, yy))
+        rows.append((f"row logprob forward, {str(dt).split('.')[1]} logits [{N} x {V}]", nb, ms))
+        ms = timed(lambda: G.entropy_from_logits(x))
+        rows.append((f"row entropy, {str(dt).split('.')[1]} logits [{N} x {V}]", nb, ms))
+        lse = ops.logits_logprob_entropy(x, yy, -100)[2]
+        gg = torch.randn(N, device=dev)
+        ms = timed(lambda: ops.logits_logprob_bwd(x, yy, -100, gg, lse))
+        rows.append((f"row logprob backward, {str(dt).split('.')[1]} logits [{N} x {V}]", 2 * nb, ms))
+        del x
+    kernels = [{"kernel": n, "algorithmic_bytes": b, "ms": ms, "achieved_GBps": b / (ms * 1e-3) / 1e9,
+                "frac": b / (ms * 1e-3) / 1e9 / PEAK} for n, b, ms in rows]
+    best = max(kernels, key=lambda r: r["achieved_GBps"])
+    print(json.dumps({
+        "metric": "achieved HBM GB/s of the reduction / elementwise / row kernels of the path",
+        "value": best["achieved_GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": best["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic", "config": {"workload": "bandwidth-bound kernels: " + best["kernel"]},
+        "roofline": {"bound": "hbm", "achieved": best["achieved_GBps"], "peak": PEAK, "unit": "GB/s",
+                     "frac": best["frac"], "traffic": None},
+        "kernels": kernels,
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -150,6 +228,8 @@ def main():
     ap.add_argument("--attention", action="store_true",
                     help="time the packed attention kernels instead (prints their own JSON line)")
     ap.add_argument("--attention-shape", choices=["cfg1", "long"], default="cfg1")
+    ap.add_argument("--hbm-kernels", action="store_true",
+                    help="time the bandwidth-bound kernels of the path instead (prints their own JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path shards by micro-batch, one per GPU); "
@@ -158,6 +238,8 @@ def main():
 
     if args.attention:
         return attention_line(args)
+    if args.hbm_kernels:
+        return hbm_line(args)
 
     import torch
     import grpo_loss as G

@@ -108,11 +108,14 @@ int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, co
  * [T] arrays.  stats_out: FGRPO_NUM_STATS doubles =
  * {n, sum|lr|, sum lr, sum lr^2, sum(r-1-lr), #(r>1+hi), #(r<1-lo), sum ent,
  *  sum old_ent, sum adv, sum adv^2, #(adv>0), #(adv==0), #(clipped>unclipped),
- *  0, #out-of-range idx}. */
+ *  0, #out-of-range idx}.  partial_ws: FGRPO_NUM_STATS * FGRPO_METRIC_BLOCKS doubles of
+ * scratch for the two-stage sum (fixed order: results are bit-reproducible), or NULL
+ * for a single work-group. */
+#define FGRPO_METRIC_BLOCKS 128
 int fgrpo_metrics(const int64_t* idx, int n, int T, const float* log_ratio, const float* entropy,
                   const float* old_entropy, const float* adv, const float* unclipped,
                   const float* clipped, float clip_low, float clip_high,
-                  double* stats_out, void* stream);
+                  double* stats_out, double* partial_ws, void* stream);
 
 /* ---- group-normalised advantages ------------------------------------------------
  * Replaces vllm_worker.py:788-796 (and normalize_rewards, :77-92):

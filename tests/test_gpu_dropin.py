@@ -299,6 +299,36 @@ def test_training_forward_metrics_and_backward(dev, entropy_coeff):
     assert torch.nn.functional.cosine_similarity(gp.flatten(), cpu_model.model.proj.weight.grad.flatten(), dim=0) > 0.9999
 
 
+@pytest.mark.parametrize("n_tok", [3000, 50000, 700000])
+def test_diagnostics_vector_against_direct_sums(dev, n_tok):
+    """The 16 sums behind the metric dictionary (reference: grpo_loss.py:408-498), from one work-group for few
+    positions and from a two-stage sum in fixed order for many: compared with float64 sums on the host, and two
+    runs agree bit for bit.  Negative and out-of-range positions are wrapped / counted, not dereferenced."""
+    from fgrpo import ops
+    g = torch.Generator().manual_seed(n_tok)
+    lr = torch.randn(n_tok, generator=g) * 0.2
+    ent = torch.rand(n_tok, generator=g) * 5
+    old_ent = torch.rand(n_tok, generator=g) * 5
+    adv = torch.randn(n_tok, generator=g).round(decimals=1)
+    l1 = torch.randn(n_tok, generator=g)
+    l2 = torch.randn(n_tok, generator=g)
+    idx = torch.nonzero(torch.rand(n_tok, generator=g) < 0.8).reshape(-1)
+    idx = torch.cat([idx, torch.tensor([-1, n_tok + 5, -n_tok - 9])])            # last token, two out of range
+    args = [t.to(dev) for t in (idx, lr, ent, old_ent, adv, l1, l2)]
+    got = ops.grpo_metrics(*args, 0.2, 0.28)
+    again = ops.grpo_metrics(*args, 0.2, 0.28)
+    assert torch.equal(got, again)
+    ok = torch.cat([idx[:-3], torch.tensor([n_tok - 1])])
+    x, a, r = lr[ok].double(), adv[ok].double(), torch.exp(lr[ok]).double()
+    want = [ok.numel(), x.abs().sum(), x.sum(), (x * x).sum(), (torch.exp(lr[ok]) - 1.0 - lr[ok]).double().sum(),
+            (torch.exp(lr[ok]) > 1.28).sum(), (torch.exp(lr[ok]) < 0.8).sum(), ent[ok].double().sum(),
+            old_ent[ok].double().sum(), a.sum(), (a * a).sum(), (a > 0).sum(), (a == 0).sum(), (l2[ok] > l1[ok]).sum(),
+            0, 2]
+    for k, (gv, wv) in enumerate(zip(got.cpu().tolist(), want)):
+        wv = float(wv)
+        assert abs(gv - wv) <= 2e-5 * max(1.0, abs(wv)) + (3 if k in (5, 6) else 0), (k, gv, wv)   # k 5, 6: thresholds met to 1 ulp of exp
+
+
 def test_trainer_harness_scaling_and_dummy(dev):
     from workers import TrainerHarness
     model, G = _patched(dev, "training", dtype=torch.bfloat16)
