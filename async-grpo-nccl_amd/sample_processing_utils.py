@@ -18,6 +18,24 @@ import torch
 from fgrpo import ops
 
 
+def _fill(dst: np.ndarray, batched_questions, key: str, lens, default=None) -> None:
+    """Writes the per-token values ``s[key]`` of every sample into consecutive pieces of ``dst`` (a numpy view of
+    the staging buffer).  Python lists go through ``np.fromiter`` (about half the cost of ``torch.as_tensor`` per
+    element, and this conversion is most of the time of packing a batch); arrays and tensors are copied."""
+    off = 0
+    for s, k in zip(batched_questions, lens):
+        x = s.get(key, None)
+        if x is None:
+            dst[off:off + k] = default
+        elif isinstance(x, (list, tuple)):
+            if len(x) != k:
+                raise ValueError(f"sample field {key!r} has {len(x)} entries for {k} tokens")
+            dst[off:off + k] = np.fromiter(x, dtype=dst.dtype, count=k)
+        else:
+            dst[off:off + k] = np.asarray(x.cpu() if torch.is_tensor(x) else x).reshape(-1)
+        off += k
+
+
 def _lens(batched_questions):
     il = np.fromiter((s["input_len"] for s in batched_questions), dtype=np.int64, count=len(batched_questions))
     ol = np.fromiter((s["output_len"] for s in batched_questions), dtype=np.int64, count=len(batched_questions))
@@ -52,18 +70,16 @@ def get_input_for_logprobs(batched_questions, output_indices, device):
     (reference: sample_processing_utils.py:114-125).  One pinned staging buffer,
     one copy.  Samples that carry no ``labels`` get them built on the device from
     ``input_len`` / ``output_len`` (the rule of vllm_worker.py:768-774)."""
-    n_tok = sum(len(s["sample_ids"]) for s in batched_questions)
+    lens = [len(s["sample_ids"]) for s in batched_questions]
+    n_tok = sum(lens)
     have_labels = all("labels" in s for s in batched_questions)
     rows = 3 if have_labels else 2
     host = torch.empty((rows, n_tok), dtype=torch.long).pin_memory() if n_tok else torch.empty((rows, 0), dtype=torch.long)
-    off = 0
-    for s in batched_questions:
-        k = len(s["sample_ids"])
-        host[0, off:off + k] = torch.as_tensor(s["sample_ids"], dtype=torch.long)
-        host[1, off:off + k] = torch.as_tensor(s["sample_position_ids"], dtype=torch.long)
-        if have_labels:
-            host[2, off:off + k] = torch.as_tensor(s["labels"], dtype=torch.long)
-        off += k
+    view = host.numpy()
+    _fill(view[0], batched_questions, "sample_ids", lens)
+    _fill(view[1], batched_questions, "sample_position_ids", lens)
+    if have_labels:
+        _fill(view[2], batched_questions, "labels", lens)
     dev = host.to(device, non_blocking=True)
     if have_labels:
         return dev[0:1], dev[1:2], dev[2:3]
@@ -113,19 +129,34 @@ def post_process_batch(batched_questions, device, constant_length_samples=None):
     else:
         output_lens_broadcasted = torch.full((total,), float(constant_length_samples), device=device, dtype=torch.float32)
 
-    lp_host = [torch.as_tensor(s["sample_logprobs"], dtype=torch.float32).reshape(-1) for s in batched_questions]
-    reference_output_logprobs = torch.cat(lp_host).to(device)
-    ent_host = []
-    for s, lp in zip(batched_questions, lp_host):
-        e = s.get("sample_entropies", None)
-        ent_host.append(torch.zeros(lp.numel()) if e is None else torch.as_tensor(e, dtype=torch.float32).reshape(-1))
-    reference_output_entropies = torch.cat(ent_host).to(device) if ent_host else torch.zeros_like(reference_output_logprobs)
+    # old-policy logprobs and entropies (zeros where a sample carries none): one pinned buffer, one copy
+    lp_lens = [len(s["sample_logprobs"]) for s in batched_questions]
+    n_lp = sum(lp_lens)
+    stage = torch.empty((2, n_lp), dtype=torch.float32).pin_memory() if n_lp else torch.empty((2, 0), dtype=torch.float32)
+    sv = stage.numpy()
+    _fill(sv[0], batched_questions, "sample_logprobs", lp_lens)
+    _fill(sv[1], batched_questions, "sample_entropies", lp_lens, default=0.0)
+    stage_dev = stage.to(device, non_blocking=True)
+    reference_output_logprobs, reference_output_entropies = stage_dev[0], stage_dev[1]
 
     batch_ids, batch_position_ids, labels = get_input_for_logprobs(batched_questions, output_indices, device)
 
     modified = [q for q in batched_questions if q['modified_reward'] is not None]
     plain = [q for q in batched_questions if q['modified_reward'] is None]
-    f32 = lambda x: torch.tensor(float(x), device=device, dtype=torch.float32)
+    # the scalar counters travel as one vector (one copy instead of eleven)
+    counters = {
+        "num_output_tokens": float(ol.sum()),
+        "num_samples": float(len(batched_questions)),
+        "max_reward_in_group": 0.0,
+        "total_modified_reward": float(sum(s['modified_reward'] for s in modified)) if modified else 0.0,
+        "total_non_modified_reward": float(sum(s['reward'] for s in plain)) if plain else 0.0,
+        "num_modified_samples": float(len(modified)),
+        "delimiter_not_found": float(sum(s['delimiter_not_found'] for s in modified)) if modified else 0.0,
+        "total_reward_rank": float(sum(s['reward'] for s in batched_questions)),
+        "truncated_sample": float(sum(s['truncated_sample'] for s in batched_questions)),
+        "advantage_is_zero": 0.0,
+    }
+    counter_vec = torch.tensor(list(counters.values()), dtype=torch.float32).to(device)
     out = {
         "batch_ids": batch_ids.contiguous(),
         "batch_position_ids": batch_position_ids.contiguous(),
@@ -135,21 +166,13 @@ def post_process_batch(batched_questions, device, constant_length_samples=None):
         "reference_output_entropies": reference_output_entropies.contiguous(),
         "output_lens_broadcasted": output_lens_broadcasted.contiguous(),
         "num_output_tokens_non_masked": (labels != -100).sum().to(torch.float32),
-        "num_output_tokens": f32(ol.sum()),
-        "num_samples": f32(len(batched_questions)),
-        "max_reward_in_group": f32(0.0),
-        "total_modified_reward": f32(sum(s['modified_reward'] for s in modified)) if modified else f32(0.0),
-        "total_non_modified_reward": f32(sum(s['reward'] for s in plain)) if plain else f32(0.0),
-        "num_modified_samples": f32(len(modified)),
-        "delimiter_not_found": f32(sum(s['delimiter_not_found'] for s in modified)) if modified else f32(0.0),
         "samples": batched_questions,
         "labels": labels.contiguous(),
-        "total_reward_rank": f32(sum(s['reward'] for s in batched_questions)),
-        "truncated_sample": f32(sum(s['truncated_sample'] for s in batched_questions)),
-        "advantage_is_zero": f32(0.0),
         # not in the reference: segment boundaries, so that the loss can aggregate per sample
         "cu_seqlens": cu,
     }
+    for k, key in enumerate(counters):
+        out[key] = counter_vec[k]
     try:
         out["uids"] = torch.tensor([int(s.get("__uid__", -1)) for s in batched_questions], device=device)
     except Exception:

@@ -11,10 +11,11 @@ from __future__ import annotations
 from types import SimpleNamespace
 from typing import List
 
+import numpy as np
 import torch
 
 from grpo_loss import compute_dual_clip_grpo_loss, make_grpo_forward
-from sample_processing_utils import post_process_batch
+from sample_processing_utils import _fill, post_process_batch
 
 
 def prepare_actor_module(model, config=None, mode: str = "training", use_varlen_attention: bool = True):
@@ -80,11 +81,12 @@ class LogProbHarness:
         lens = [len(s["sample_ids"]) for s in samples]
         total = sum(lens)
         host = torch.empty((3, total), dtype=torch.long)
+        view = host.numpy()
+        _fill(view[0], samples, "sample_ids", lens)
+        _fill(view[2], samples, "labels", lens, default=-100)
         off = 0
-        for s, k in zip(samples, lens):
-            host[0, off:off + k] = torch.as_tensor(s["sample_ids"], dtype=torch.long)
-            host[1, off:off + k] = torch.arange(k)
-            host[2, off:off + k] = torch.as_tensor(s.get("labels", [-100] * k), dtype=torch.long)
+        for k in lens:
+            view[1, off:off + k] = np.arange(k)
             off += k
         dev = host.to(self.device)
         out = self.actor_module_fsdp(input_ids=dev[0:1], attention_mask=None, position_ids=dev[1:2], labels=dev[2:3])
