@@ -102,3 +102,27 @@ def test_varlen_attention_argument_errors_and_route():
     assert VA.install_explicit_varlen_wrapper(model) is True
     with pytest.raises(RuntimeError, match="GPU"):
         model(input_ids=torch.zeros(1, 6, dtype=torch.long), position_ids=torch.tensor([[0, 1, 2, 0, 1, 2]]))
+
+
+def test_missing_library_raises_and_nothing_falls_back(monkeypatch, tmp_path):
+    """Without libfgrpo.so the product raises (naming the build command) instead of computing some other way."""
+    from fgrpo import _lib
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "no_such_libfgrpo.so"))
+    monkeypatch.setattr(_lib, "_lib", None)              # forget the handle loaded by earlier tests
+    with pytest.raises(RuntimeError, match="fgrpo.build"):
+        _lib.load()
+    import grpo_loss as G
+    import torch
+    with pytest.raises(RuntimeError):                    # the drop-in has no other way to compute
+        G.logprobs_from_logits(torch.zeros(2, 8), torch.zeros(2, dtype=torch.long))
+
+
+def test_product_modules_never_import_the_oracle():
+    """The oracle is test infrastructure: no module of the package imports, reads or names it."""
+    import os
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "async-grpo-nccl_amd")
+    for dirpath, _, files in os.walk(root):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip")):
+                text = open(os.path.join(dirpath, f), encoding="utf-8").read()
+                assert "oracle" not in text, os.path.join(dirpath, f)
