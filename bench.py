@@ -157,8 +157,12 @@ def hbm_line(args):
     PEAK = 8000.0
 
     def timed(fn):
-        for _ in range(args.warmup):
+        n_warm, t_w = 0, time.perf_counter()       # short kernels: warm up by time (0.1 s), not by count
+        while n_warm < args.warmup or time.perf_counter() - t_w < 0.1:
             fn()
+            n_warm += 1
+            if n_warm % 16 == 0:
+                torch.cuda.synchronize()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
