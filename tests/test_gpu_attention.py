@@ -334,6 +334,32 @@ def test_random_shapes_and_segmentations(dev):
         check(dev, f"random {case}", T, cu, Hq, Hkv, causal, seed=100 + case, D=D)
 
 
+@pytest.mark.parametrize("scale_in", [0.01, 4.0, 64.0])
+def test_input_scales_from_flat_to_saturated_softmax(dev, scale_in):
+    """Scores from nearly constant (softmax flat) to hundreds in magnitude (softmax one-hot, exponents far below
+    the fp32 range on the masked side): outputs and gradients stay finite and follow the fp32 oracle."""
+    from fgrpo import ops
+    T, Hq, Hkv, D = 300, 4, 2, 128
+    for causal in (True, False):
+        g = torch.Generator().manual_seed(int(scale_in * 100) + causal)
+        q = (torch.randn(T, Hq, D, generator=g) * scale_in).bfloat16()
+        k = (torch.randn(T, Hkv, D, generator=g) * scale_in).bfloat16()
+        v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+        do = torch.randn(T, Hq, D, generator=g).bfloat16()
+        cu = torch.tensor([0, 37, 38, 200, 300], dtype=torch.int32)
+        qo, ko, vo = (x.float().requires_grad_(True) for x in (q, k, v))
+        want = A.varlen_attention(qo, ko, vo, cu, causal=causal)
+        want.backward(do.float())
+        qg, kg, vg = (x.to(dev).requires_grad_(True) for x in (q, k, v))
+        got = ops.varlen_attention(qg, kg, vg, cu.to(dev), None, causal)
+        got.backward(do.to(dev))
+        torch.cuda.synchronize()
+        assert (got.float().cpu() - want.detach()).abs().max().item() <= OUT_ATOL
+        for a, b in ((qg.grad, qo.grad), (kg.grad, ko.grad), (vg.grad, vo.grad)):
+            assert torch.isfinite(a.float()).all()
+            assert ((a.float().cpu() - b).norm() / (b.norm() + 1e-30)).item() <= 3e-2
+
+
 def test_every_heads_per_work_group_shape(dev):
     """The forward and dQ kernels come in three shapes (1, 2 or 4 query heads of a K/V group per work-group over
     128-, 64- or 32-token tiles).  Each is forced in turn over group sizes it divides and does not divide
