@@ -5,6 +5,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <mutex>
 #include <string>
 
 #include "../../include/fgrpo.h"
@@ -12,6 +13,12 @@
 #include "attn_kernels.h"
 
 using namespace fgrpo;
+
+// Device memory that fgrpo_logprob_fwd_static uses in place of a caller workspace.  Every GPU the library runs
+// on holds its own copy until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress: kernels, fills and copies take the per-device address kept in g_static_scratch.
+static_assert(FGRPO_STATIC_SCRATCH_BYTES % 256 == 0, "scratch size");
+static __device__ __align__(256) unsigned char scratch[FGRPO_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -521,31 +528,8 @@ struct DqLauncher {
 }  // namespace
 
 
-extern "C" {
-
-int fgrpo_version(void) { return 100; }
-const char* fgrpo_last_error(void) { return g_err.c_str(); }
-
-int fgrpo_set_tuning(const char* key, int value) {
-  int* s = tuning_slot(key);
-  if (!s) return fail(FGRPO_ERR_BAD_ARG, "unknown tuning key '%s'", key ? key : "(null)");
-  *s = value;
-  return 0;
-}
-int fgrpo_get_tuning(const char* key) {
-  int* s = tuning_slot(key);
-  if (!s) return fail(FGRPO_ERR_BAD_ARG, "unknown tuning key '%s'", key ? key : "(null)");
-  return *s;
-}
-
-size_t fgrpo_logprob_fwd_workspace(int T, int H, int V, int dtype) {
-  if (T <= 0 || H <= 0 || V <= 0) return 0;
-  FwdPlan pl;
-  plan_fwd(pl, nullptr, T, H, V, dtype, true);
-  return pl.bytes;
-}
-
-int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
+namespace {
+int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
                       int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
                       size_t ws_bytes, void* stream) {
   hipStream_t st = (hipStream_t)stream;
@@ -586,6 +570,75 @@ int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias, 
   hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((T + 255) / 256), dim3(256), 0, st, c);
   HIP_TRY(hipGetLastError());
   return 0;
+}
+
+// Per-device address of `scratch`, resolved once per device with that device current.
+std::mutex g_static_mu;
+void* g_static_scratch[64] = {nullptr};
+
+int static_scratch_ptr(void** out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return fail(FGRPO_ERR_UNSUPPORTED, "static scratch: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_scratch[dev]) {
+    void* ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(FGRPO_ERR_HIP, "static scratch: hipGetSymbolAddress returned a null address");
+    g_static_scratch[dev] = ptr;
+  }
+  *out = g_static_scratch[dev];
+  return 0;
+}
+}  // namespace
+
+extern "C" {
+
+int fgrpo_version(void) { return 100; }
+const char* fgrpo_last_error(void) { return g_err.c_str(); }
+
+int fgrpo_set_tuning(const char* key, int value) {
+  int* s = tuning_slot(key);
+  if (!s) return fail(FGRPO_ERR_BAD_ARG, "unknown tuning key '%s'", key ? key : "(null)");
+  *s = value;
+  return 0;
+}
+int fgrpo_get_tuning(const char* key) {
+  int* s = tuning_slot(key);
+  if (!s) return fail(FGRPO_ERR_BAD_ARG, "unknown tuning key '%s'", key ? key : "(null)");
+  return *s;
+}
+
+size_t fgrpo_logprob_fwd_workspace(int T, int H, int V, int dtype) {
+  if (T <= 0 || H <= 0 || V <= 0) return 0;
+  FwdPlan pl;
+  plan_fwd(pl, nullptr, T, H, V, dtype, true);
+  return pl.bytes;
+}
+
+int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
+                      int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
+                      size_t ws_bytes, void* stream) {
+  return logprob_fwd_impl(hidden, weight, bias, labels, inv_temp, T, H, V, dtype, lp_out, ent_out, lse_out, ws, ws_bytes,
+                          stream);
+}
+
+int fgrpo_logprob_fwd_static(const void* hidden, const void* weight, const void* bias, const int64_t* labels,
+                             float inv_temp, int T, int H, int V, int dtype, float* lp_out, float* ent_out,
+                             float* lse_out, void* stream) {
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd_static: T=%d H=%d V=%d", T, H, V);
+  if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd_static: dtype=%d", dtype);
+  FwdPlan pl;
+  plan_fwd(pl, nullptr, T, H, V, dtype, bias != nullptr);
+  if (pl.bytes > FGRPO_STATIC_SCRATCH_BYTES)
+    return fail(FGRPO_ERR_WORKSPACE,
+                "logprob_fwd_static: this call needs %zu bytes of scratch, the built-in buffer holds %u "
+                "(use fgrpo_logprob_fwd with a caller workspace)", pl.bytes, (unsigned)FGRPO_STATIC_SCRATCH_BYTES);
+  void* ptr = nullptr;
+  int rc = static_scratch_ptr(&ptr);
+  if (rc) return rc;
+  return logprob_fwd_impl(hidden, weight, bias, labels, inv_temp, T, H, V, dtype, lp_out, ent_out, lse_out, ptr,
+                          FGRPO_STATIC_SCRATCH_BYTES, stream);
 }
 
 size_t fgrpo_lmhead_bwd_workspace(int T, int H, int V, int dtype, long long hint) {

@@ -14,6 +14,7 @@ ERR = {-1: "bad argument", -2: "unsupported", -3: "workspace", -4: "HIP error", 
 BF16, F32 = 0, 1
 AGG_TOKEN_MEAN, AGG_SAMPLE_MEAN = 0, 1
 NUM_STATS = 16
+STATIC_SCRATCH_BYTES = 8 << 20   # FGRPO_STATIC_SCRATCH_BYTES
 METRIC_BLOCKS = 128      # work-groups of the diagnostics' first stage (FGRPO_METRIC_BLOCKS)
 
 _vp, _i, _ll, _f, _d, _sz = C.c_void_p, C.c_int, C.c_longlong, C.c_float, C.c_double, C.c_size_t
@@ -26,6 +27,7 @@ SIGNATURES = {
     "fgrpo_get_tuning": (_i, [C.c_char_p]),
     "fgrpo_logprob_fwd_workspace": (_sz, [_i, _i, _i, _i]),
     "fgrpo_logprob_fwd": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgrpo_logprob_fwd_static": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "fgrpo_lmhead_bwd_workspace": (_sz, [_i, _i, _i, _i, _ll]),
     "fgrpo_lmhead_bwd_panel_cols": (_i, [_i, _i, _i, _i, _ll]),
     "fgrpo_lmhead_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _vp, _vp, _ll, _vp, _sz, _vp]),

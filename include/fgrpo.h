@@ -60,6 +60,21 @@ int fgrpo_logprob_fwd(const void* hidden, const void* weight, const void* bias,
                       float* lp_out, float* ent_out, float* lse_out,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* Same computation and results as fgrpo_logprob_fwd, for callers that cannot allocate (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): it takes no workspace and calls no allocating
+ * routine.  Its scratch (per-split soft-max partials and target logits, what fgrpo_logprob_fwd_workspace sizes)
+ * lives in a buffer of FGRPO_STATIC_SCRATCH_BYTES built into the library's device image, one copy per GPU, held
+ * until the process ends.  A call that would need more returns FGRPO_ERR_WORKSPACE (bf16 inputs with H a multiple
+ * of 64 need 16 * splits + 4 bytes per token: 2.2 MB at T = 32768, no bias; fp32 inputs and other H also stage
+ * operand copies there and fit only at small sizes).  All calls on one GPU share the buffer: calls that overlap on
+ * one GPU (different streams or threads) race; calls ordered on one stream do not.  Nothing in the buffer has to
+ * start at zero.  No counterpart in the reference. */
+#define FGRPO_STATIC_SCRATCH_BYTES (8u << 20)
+int fgrpo_logprob_fwd_static(const void* hidden, const void* weight, const void* bias,
+                             const int64_t* labels_shifted, float inv_temperature,
+                             int T, int H, int V, int dtype,
+                             float* lp_out, float* ent_out, float* lse_out, void* stream);
+
 /* ---- backward of the above (what autograd derives from grpo_loss.py:290-296
  * through torch.matmul / gather / logsumexp):
  *   dX_t = g_t * gout * inv_temperature * (onehot(y_t) - softmax(x_t))
