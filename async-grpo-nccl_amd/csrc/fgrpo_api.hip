@@ -8,9 +8,9 @@
 #include <mutex>
 #include <string>
 
-#include "../../include/fgrpo.h"
+#include "host_common.h"
+#include "prep_kernels.h"
 #include "tail_kernels.h"
-#include "attn_kernels.h"
 
 using namespace fgrpo;
 
@@ -20,9 +20,11 @@ using namespace fgrpo;
 static_assert(FGRPO_STATIC_SCRATCH_BYTES % 256 == 0, "scratch size");
 static __device__ __align__(256) unsigned char scratch[FGRPO_STATIC_SCRATCH_BYTES];
 
-namespace {
+namespace fgrpo {
 
+namespace {
 thread_local std::string g_err;
+}
 
 int fail(int code, const char* fmt, ...) {
   char buf[512];
@@ -34,63 +36,23 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-#define HIP_TRY(expr)                                                                  \
-  do {                                                                                 \
-    hipError_t e_ = (expr);                                                            \
-    if (e_ != hipSuccess) return fail(FGRPO_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
-  } while (0)
+Tuning g_tune;
 
-inline long long round_up(long long x, long long m) { return (x + m - 1) / m * m; }
-inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
-
-// ---- tile configurations ---------------------------------------------------------
-// id 0: 256x256x64, 4 wavefronts of 128x128, one work-group per CU
-// id 1: 256x128x64, 4 wavefronts of 128x64
-// id 2: 256x128x32, 4 wavefronts of 128x64, two work-groups per CU
-// id 3: 256x256x32, 8 wavefronts of 128x64 (two per SIMD)
-// id 4: 128x128x64, 4 wavefronts of 64x64, two work-groups per CU (small problems)
-typedef TileCfg<256, 256, 64, 2, 2, 1> Cfg0;
-typedef TileCfg<256, 128, 64, 2, 2, 1> Cfg1;
-typedef TileCfg<256, 128, 32, 2, 2, 2> Cfg2;
-typedef TileCfg<256, 256, 32, 2, 4, 2> Cfg3;
-typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg4;
-// id 5: 256x256x32, 4 wavefronts, direct-to-LDS loads, 5 LDS stages, look-ahead fragment prefetch
-// id 6: 256x256x64, 4 wavefronts, direct-to-LDS loads, 2 LDS stages
-// id 7: 256x128x32, 4 wavefronts of 128x64, direct-to-LDS, 4 stages, two work-groups per CU
-typedef TileCfg<256, 256, 32, 2, 2, 1, 5, true> Cfg5;
-typedef TileCfg<256, 256, 64, 2, 2, 1, 2, true> Cfg6;
-typedef TileCfg<256, 128, 32, 2, 2, 2, 3, true> Cfg7;
-// id 8/9: as 6/5 with 8 wavefronts of 128x64 (two per SIMD)
-typedef TileCfg<256, 256, 64, 2, 4, 2, 2, true> Cfg8;
-typedef TileCfg<256, 256, 32, 2, 4, 2, 5, true> Cfg9;
-constexpr int kNumCfg = 10;
-
-struct CfgInfo {
-  int bm, bn, bk, nt, lds, wgs_per_cu;
-};
-template <class C>
-constexpr CfgInfo info_of(int wgs) {
-  return CfgInfo{C::BM, C::BN, C::BK, C::NT, C::LDS_BYTES, wgs};
+int num_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
 }
-const CfgInfo kCfg[kNumCfg] = {info_of<Cfg0>(1), info_of<Cfg1>(1), info_of<Cfg2>(2), info_of<Cfg3>(1), info_of<Cfg4>(2),
-                                info_of<Cfg5>(1), info_of<Cfg6>(1), info_of<Cfg7>(2), info_of<Cfg8>(1), info_of<Cfg9>(1)};
 
-struct Tuning {
-  int fwd_variant = 8;
-  int ds_variant = 8;
-  int gemm_variant = 8;
-  int fwd_nsplit = 0;   // 0 = heuristic
-  int fwd_group_t = 8;
-  int ds_nsplit = 0;    // dLogits kernel: vocabulary splits of a panel; 0 = as the forward
-  int ds_group_t = 0;   // dLogits kernel: token tiles per raster group; 0 = as the forward
-  int dh_group_m = 0;   // dHidden GEMM raster group; 0 = gemm_group_m
-  int dw_group_m = 0;   // dW GEMM raster group; 0 = gemm_group_m
-  int gemm_group_m = 4;
-  int panel_cols = 0;      // vocabulary panel width of the backward when the caller gives no bound; 0 = a quarter of [T x V], 2^25 .. 2^30 elements
-  int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
-  int bwd_kmajor = 2;      // 0: transposed copies; 1: the dW GEMM reads dLogits and hidden in place; 2: the dH GEMM reads W in place too
-  int attn_heads = 0;      // query heads per work-group of the attention forward / dQ kernels (1, 2, 4); 0 = heuristic
-} g_tune;
+}  // namespace fgrpo
+
+namespace {
 
 int* tuning_slot(const char* key) {
   if (!key) return nullptr;
@@ -108,42 +70,8 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "small_variant")) return &g_tune.small_variant;
   if (!strcmp(key, "bwd_kmajor")) return &g_tune.bwd_kmajor;
   if (!strcmp(key, "attn_heads")) return &g_tune.attn_heads;
+  if (!strcmp(key, "wide_stores")) return &g_tune.wide_stores;
   return nullptr;
-}
-
-int num_cus() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      n = prop.multiProcessorCount;
-    if (n <= 0) n = 256;
-  }
-  return n;
-}
-
-// Kernels with more than 64 KiB of dynamic LDS need the limit raised once per
-// device and function.
-template <class C, class P>
-int raise_lds(void (*kern)(const P), int bytes) {
-  static bool done[64] = {false};
-  int dev = 0;
-  HIP_TRY(hipGetDevice(&dev));
-  if (dev >= 0 && dev < 64 && done[dev]) return 0;
-  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-  if (dev >= 0 && dev < 64) done[dev] = true;
-  return 0;
-}
-
-template <class C, class P>
-int launch_tile_kernel(void (*kern)(const P), const P& p, int nblocks, hipStream_t st) {
-  if (nblocks <= 0) return 0;
-  int rc = raise_lds<C, P>(kern, C::LDS_BYTES);
-  if (rc) return rc;
-  hipLaunchKernelGGL(kern, dim3(nblocks), dim3(C::NT), C::LDS_BYTES, st, p);
-  HIP_TRY(hipGetLastError());
-  return 0;
 }
 
 int check_operands(const GemmOperands& g, int bk) {
@@ -190,12 +118,12 @@ struct Carver {
   size_t total() const { return (size_t)round_up((long long)off, 256); }
 };
 
-int pick_variant(int requested, long long M, long long N) {
+int pick_variant(const Tuning& tn, int requested, long long M, long long N) {
   int v = requested;
   if (v < 0 || v >= kNumCfg) v = 0;
   // small problems: a big tile would leave most CUs idle
   const long long tiles = ((M + kCfg[v].bm - 1) / kCfg[v].bm) * ((N + kCfg[v].bn - 1) / kCfg[v].bn);
-  if (tiles < num_cus() / 2 && g_tune.small_variant >= 0 && g_tune.small_variant < kNumCfg) v = g_tune.small_variant;
+  if (tiles < num_cus() / 2 && tn.small_variant >= 0 && tn.small_variant < kNumCfg) v = tn.small_variant;
   return v;
 }
 
@@ -242,12 +170,12 @@ int choose_nsplit(int tiles_t, int tiles_v, int slots, int forced, int prefer = 
   return best;
 }
 
-void plan_fwd(FwdPlan& pl, void* ws, int T, int H, int V, int dtype, bool has_bias) {
-  pl.variant = pick_variant(g_tune.fwd_variant, V, T);
+void plan_fwd(const Tuning& tn, FwdPlan& pl, void* ws, int T, int H, int V, int dtype, bool has_bias) {
+  pl.variant = pick_variant(tn, tn.fwd_variant, V, T);
   const CfgInfo& c = kCfg[pl.variant];
   pl.tiles_v = (V + c.bm - 1) / c.bm;
   pl.tiles_t = (T + c.bn - 1) / c.bn;
-  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu, g_tune.fwd_nsplit);
+  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu, tn.fwd_nsplit);
   pl.Hp = (int)round_up(H, 64);
   pl.copy_ops = (dtype == FGRPO_F32) || (H % 64 != 0);
   Carver cv(ws);
@@ -295,40 +223,20 @@ int stage_logit_operands(GemmOperands& g, const void* hidden, const void* weight
   return 0;
 }
 
-template <class C>
-int launch_fwd(const FwdParams& p, hipStream_t st) {
-  return launch_tile_kernel<C>(lmhead_fwd_kernel<C>, p, p.tiles_t * p.nsplit, st);
+// 16-byte epilogue pieces need every row of the output (and of the addend) to start on a 16-byte boundary.
+bool can_store_wide(const Tuning& tn, const StoreParams& p) {
+  if (!tn.wide_stores) return false;
+  const long long per16 = p.c_out_bf16 ? 8 : 4;
+  if (p.ldc % per16) return false;
+  if (p.c_out_bf16 && !aligned16(p.c_out_bf16)) return false;
+  if (p.c_out_f32 && !aligned16(p.c_out_f32)) return false;
+  if (p.c_in && (!aligned16(p.c_in) || p.ldc % 4)) return false;
+  return true;
 }
-template <class C>
-int launch_ds(const DsParams& p, hipStream_t st) {
-  return launch_tile_kernel<C>(lmhead_ds_kernel<C, false>, p, p.tiles_t * p.nsplit, st);
-}
-// fp32 inputs: dS is written as bf16 hi + lo halves; only the small tile carries that epilogue
-int launch_ds_split(const DsParams& p, hipStream_t st) {
-  return launch_tile_kernel<Cfg4>(lmhead_ds_kernel<Cfg4, true>, p, p.tiles_t * p.nsplit, st);
-}
-template <class C>
-int launch_store(const StoreParams& p, hipStream_t st) {
-  return launch_tile_kernel<C>(gemm_store_kernel<C>, p, p.tiles_m * p.tiles_n, st);
-}
-
-#define DISPATCH_VARIANT(variant, fn, ...)                \
-  switch (variant) {                                      \
-    case 0: rc = fn<Cfg0>(__VA_ARGS__); break;            \
-    case 1: rc = fn<Cfg1>(__VA_ARGS__); break;            \
-    case 2: rc = fn<Cfg2>(__VA_ARGS__); break;            \
-    case 3: rc = fn<Cfg3>(__VA_ARGS__); break;            \
-    case 5: rc = fn<Cfg5>(__VA_ARGS__); break;            \
-    case 6: rc = fn<Cfg6>(__VA_ARGS__); break;            \
-    case 7: rc = fn<Cfg7>(__VA_ARGS__); break;            \
-    case 8: rc = fn<Cfg8>(__VA_ARGS__); break;            \
-    case 9: rc = fn<Cfg9>(__VA_ARGS__); break;            \
-    default: rc = fn<Cfg4>(__VA_ARGS__); break;           \
-  }
 
 // Gradient GEMMs whose contraction index is the row index of an operand as it lies in memory.
 // akm/bkm: that operand is [K][M] (resp. [K][N]) with leading dimension lda (ldb); the other is [M][K] ([N][K]).
-int run_store_gemm_kmajor(StoreParams p, bool akm, bool bkm, hipStream_t st) {
+int run_store_gemm_kmajor(const Tuning& tn, StoreParams p, bool akm, bool bkm, hipStream_t st) {
   const GemmOperands& g = p.g;
   if (g.nseg != 1 || !g.seg[0].A || !g.seg[0].B) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): one segment expected");
   if (g.M <= 0 || g.N <= 0 || g.seg[0].K <= 0 || g.seg[0].K % Cfg8::BK)
@@ -345,27 +253,26 @@ int run_store_gemm_kmajor(StoreParams p, bool akm, bool bkm, hipStream_t st) {
   if (256LL * g.lda * 2 >= (1LL << 32) || 256LL * g.ldb * 2 >= (1LL << 32))
     return fail(FGRPO_ERR_UNSUPPORTED, "gemm(k-major): leading dimension too large");
   {
-    const int own = (akm && bkm) ? g_tune.dw_group_m : g_tune.dh_group_m;
-    p.group_m = own > 0 ? own : (g_tune.gemm_group_m > 0 ? g_tune.gemm_group_m : 1);
+    const int own = (akm && bkm) ? tn.dw_group_m : tn.dh_group_m;
+    p.group_m = own > 0 ? own : (tn.gemm_group_m > 0 ? tn.gemm_group_m : 1);
   }
+  p.wide_stores = can_store_wide(tn, p);
   const int nb = p.tiles_m * p.tiles_n;
-  if (akm && bkm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, true, true>, p, nb, st);
-  if (akm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, true, false>, p, nb, st);
-  if (bkm) return launch_tile_kernel<Cfg8>(gemm_store_kernel<Cfg8, false, true>, p, nb, st);
-  return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): no k-major operand");
+  (void)nb;
+  return launch_store_kmajor(akm, bkm, p, st);
 }
 
-int run_store_gemm(StoreParams p, int variant, hipStream_t st) {
-  variant = pick_variant(variant, p.g.M, p.g.N);
+int run_store_gemm(const Tuning& tn, StoreParams p, int variant, hipStream_t st) {
+  variant = pick_variant(tn, variant, p.g.M, p.g.N);
   if (p.g.a_blk != 0 && variant != 6 && variant != 7 && variant != 8) variant = 8;  // loops that know the layout
   const CfgInfo& c = kCfg[variant];
   int rc = check_operands(p.g, c.bk);
   if (rc) return rc;
   p.tiles_m = (p.g.M + c.bm - 1) / c.bm;
   p.tiles_n = (p.g.N + c.bn - 1) / c.bn;
-  p.group_m = g_tune.gemm_group_m > 0 ? g_tune.gemm_group_m : 1;
-  DISPATCH_VARIANT(variant, launch_store, p, st);
-  return rc;
+  p.group_m = tn.gemm_group_m > 0 ? tn.gemm_group_m : 1;
+  p.wide_stores = can_store_wide(tn, p);
+  return launch_store_variant(variant, p, st);
 }
 
 // ---- backward plan ------------------------------------------------------------------
@@ -420,17 +327,17 @@ int fit_panel_count(int np_min, int H, int V) {
   return best;
 }
 
-void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long hint, bool has_bias, bool want_dh,
-              bool want_dw) {
+void plan_bwd(const Tuning& tn, BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long hint, bool has_bias,
+              bool want_dh, bool want_dw) {
   pl.f32 = (dtype == FGRPO_F32);
-  pl.variant = pl.f32 ? 4 : pick_variant(g_tune.ds_variant, V, T);
+  pl.variant = pl.f32 ? 4 : pick_variant(tn, tn.ds_variant, V, T);
   pl.bm = kCfg[pl.variant].bm;
   pl.bn = kCfg[pl.variant].bn;
   pl.Hp = (int)round_up(H, 64);
   pl.Tpad = (int)round_up(T, 256);
   pl.Vpad = (int)round_up(V, 256);
   pl.tiles_t = (T + pl.bn - 1) / pl.bn;
-  long long cols = g_tune.panel_cols > 0 ? g_tune.panel_cols : default_panel_elems(T, V) / (T > 0 ? T : 1);
+  long long cols = tn.panel_cols > 0 ? tn.panel_cols : default_panel_elems(T, V) / (T > 0 ? T : 1);
   if (hint > 0) cols = hint / (T > 0 ? T : 1);
   if (cols < 256) cols = 256;
   int np = (int)((V + cols - 1) / cols);
@@ -454,9 +361,9 @@ void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long h
   {
     const long long th = (long long)((T + 255) / 256) * (H / 256);
     const long long vh = (long long)(((V < pl.panel ? V : pl.panel) + 255) / 256) * (H / 256);
-    pl.kmajor = g_tune.bwd_kmajor && !pl.copy_ops && H % 256 == 0 && pl.bm == 256 && pl.bn % 64 == 0 &&
+    pl.kmajor = tn.bwd_kmajor && !pl.copy_ops && H % 256 == 0 && pl.bm == 256 && pl.bn % 64 == 0 &&
                 th >= num_cus() / 2 && vh >= num_cus() / 2;
-    pl.kmajor_dh = pl.kmajor && g_tune.bwd_kmajor >= 2;
+    pl.kmajor_dh = pl.kmajor && tn.bwd_kmajor >= 2;
   }
   pl.wT_hi = pl.wT_lo = pl.hT_hi = pl.hT_lo = nullptr;
   if (want_dh && !pl.kmajor_dh) {
@@ -482,52 +389,6 @@ void plan_bwd(BwdPlan& pl, void* ws, int T, int H, int V, int dtype, long long h
 
 }  // namespace
 
-// =====================================================================================
-namespace {
-// Query heads per work-group of the query-side kernels (tile = 128 / heads tokens).  Short segments gain from short
-// tiles (less masked work on the diagonal and at segment boundaries) as long as the heads of a group fill the
-// work-group; long ones do not care, and a lone head per K/V head has nothing to share.
-int attn_heads_per_group(int G, int T, int n_seq) {
-  if (g_tune.attn_heads == 1 || g_tune.attn_heads == 2 || g_tune.attn_heads == 4) return g_tune.attn_heads;
-  if (G <= 1 || (long long)T >= 8192LL * n_seq) return 1;      // measured: -10..-22 % up to 2048-token segments, +1 % at 8192
-  if (G % 4 == 0) return 4;
-  if (G % 2 == 0) return 2;
-  return G >= 3 ? 4 : 1;
-}
-
-template <template <int, int> class Launcher>
-int launch_query_side(int D, int hb, AttnParams& p, int T, int Hq, int Hkv, int32_t* bounds_ws, hipStream_t st) {
-  const int rb = 128 / hb, G = Hq / Hkv;
-  p.order_q = bounds_ws + attn_order_offset(T, hb == 1 ? 1 : hb == 2 ? 2 : 3);
-  const long long units = (long long)((T + rb - 1) / rb) * Hkv;            // (tile, K/V head)
-  const dim3 grid((unsigned)(((units + 7) / 8 * 8) * ((G + hb - 1) / hb)));
-  if (D == 128) {
-    if (hb == 1) Launcher<128, 1>::run(grid, st, p);
-    else if (hb == 2) Launcher<128, 2>::run(grid, st, p);
-    else Launcher<128, 4>::run(grid, st, p);
-  } else {
-    if (hb == 1) Launcher<64, 1>::run(grid, st, p);
-    else if (hb == 2) Launcher<64, 2>::run(grid, st, p);
-    else Launcher<64, 4>::run(grid, st, p);
-  }
-  HIP_TRY(hipGetLastError());
-  return 0;
-}
-template <int HD, int HB>
-struct FwdLauncher {
-  static void run(dim3 grid, hipStream_t st, const AttnParams& p) {
-    hipLaunchKernelGGL((varlen_attn_fwd_kernel<HD, HB>), grid, dim3(256), 0, st, p);
-  }
-};
-template <int HD, int HB>
-struct DqLauncher {
-  static void run(dim3 grid, hipStream_t st, const AttnParams& p) {
-    hipLaunchKernelGGL((varlen_attn_dq_kernel<HD, HB>), grid, dim3(256), 0, st, p);
-  }
-};
-}  // namespace
-
-
 namespace {
 int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
                       int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
@@ -539,8 +400,9 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: inv_temperature must be positive");
   if (!ws || !aligned16(ws)) return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd: workspace null or misaligned");
   if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "logprob_fwd: hidden/weight must be 16-byte aligned");
+  const Tuning tn = g_tune;   // one reading of the tuning state per call
   FwdPlan pl;
-  plan_fwd(pl, ws, T, H, V, dtype, bias != nullptr);
+  plan_fwd(tn, pl, ws, T, H, V, dtype, bias != nullptr);
   if (pl.bytes > ws_bytes) return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd: workspace %zu < %zu bytes", ws_bytes, pl.bytes);
 
   FwdParams p;
@@ -560,10 +422,10 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   p.tiles_v = pl.tiles_v;
   p.tiles_t = pl.tiles_t;
   p.nsplit = pl.nsplit;
-  p.group_t = g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1;
+  p.group_t = tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
   p.part = pl.part;
   p.xt = pl.xt;
-  DISPATCH_VARIANT(pl.variant, launch_fwd, p, st);
+  rc = launch_fwd_variant(pl.variant, p, st);
   if (rc) return rc;
 
   CombineParams c{pl.part, pl.xt, (const long long*)labels, T, V, pl.nsplit, lp_out, ent_out, lse_out};
@@ -612,7 +474,7 @@ int fgrpo_get_tuning(const char* key) {
 size_t fgrpo_logprob_fwd_workspace(int T, int H, int V, int dtype) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
   FwdPlan pl;
-  plan_fwd(pl, nullptr, T, H, V, dtype, true);
+  plan_fwd(g_tune, pl, nullptr, T, H, V, dtype, true);
   return pl.bytes;
 }
 
@@ -629,7 +491,7 @@ int fgrpo_logprob_fwd_static(const void* hidden, const void* weight, const void*
   if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd_static: T=%d H=%d V=%d", T, H, V);
   if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd_static: dtype=%d", dtype);
   FwdPlan pl;
-  plan_fwd(pl, nullptr, T, H, V, dtype, bias != nullptr);
+  plan_fwd(g_tune, pl, nullptr, T, H, V, dtype, bias != nullptr);
   if (pl.bytes > FGRPO_STATIC_SCRATCH_BYTES)
     return fail(FGRPO_ERR_WORKSPACE,
                 "logprob_fwd_static: this call needs %zu bytes of scratch, the built-in buffer holds %u "
@@ -644,14 +506,14 @@ int fgrpo_logprob_fwd_static(const void* hidden, const void* weight, const void*
 size_t fgrpo_lmhead_bwd_workspace(int T, int H, int V, int dtype, long long hint) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
   BwdPlan pl;
-  plan_bwd(pl, nullptr, T, H, V, dtype, hint, true, true, true);
+  plan_bwd(g_tune, pl, nullptr, T, H, V, dtype, hint, true, true, true);
   return pl.bytes;
 }
 
 int fgrpo_lmhead_bwd_panel_cols(int T, int H, int V, int dtype, long long hint) {
   if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_panel_cols: T=%d H=%d V=%d", T, H, V);
   BwdPlan pl;
-  plan_bwd(pl, nullptr, T, H, V, dtype, hint, true, true, true);
+  plan_bwd(g_tune, pl, nullptr, T, H, V, dtype, hint, true, true, true);
   return pl.panel;
 }
 
@@ -669,8 +531,9 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
   if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd: dbias requested without a bias");
   if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "lmhead_bwd: hidden/weight must be 16-byte aligned");
   const bool want_dh = dH_out != nullptr, want_dw = dW_out != nullptr;
+  const Tuning tn = g_tune;   // one reading of the tuning state per call
   BwdPlan pl;
-  plan_bwd(pl, ws, T, H, V, dtype, hint, bias != nullptr, want_dh, want_dw);
+  plan_bwd(tn, pl, ws, T, H, V, dtype, hint, bias != nullptr, want_dh, want_dw);
   if (pl.bytes > ws_bytes) return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd: workspace %zu < %zu bytes", ws_bytes, pl.bytes);
   const int f32 = pl.f32;
 
@@ -701,7 +564,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
   d.gout = gout_dev;
   d.inv_temp = inv_temp;
   d.tiles_t = pl.tiles_t;
-  d.group_t = g_tune.ds_group_t > 0 ? g_tune.ds_group_t : (g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1);
+  d.group_t = tn.ds_group_t > 0 ? tn.ds_group_t : (tn.fwd_group_t > 0 ? tn.fwd_group_t : 1);
   d.tv_hi = pl.tv_hi;
   d.tv_lo = pl.tv_lo;
   d.vt_hi = pl.vt_hi;
@@ -719,17 +582,13 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
     d.v0 = v0;
     d.tiles_v = (rows + pl.bm - 1) / pl.bm;
     d.nsplit = choose_nsplit(pl.tiles_t, d.tiles_v, num_cus() * kCfg[pl.variant].wgs_per_cu,
-                             g_tune.ds_nsplit > 0 ? g_tune.ds_nsplit : g_tune.fwd_nsplit, 8);
-    d.group_t = g_tune.ds_group_t > 0 ? g_tune.ds_group_t
+                             tn.ds_nsplit > 0 ? tn.ds_nsplit : tn.fwd_nsplit, 8);
+    d.group_t = tn.ds_group_t > 0 ? tn.ds_group_t
                 : d.nsplit == 8        ? 2       // 2 token tiles x 8 splits: half an XCD's work-groups per patch
-                : g_tune.fwd_group_t > 0 ? g_tune.fwd_group_t : 1;
+                : tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
     const int kv = d.tiles_v * pl.bm;        // written panel width
     const int kt = pl.tiles_t * pl.bn;       // written token extent
-    if (f32) {
-      rc = launch_ds_split(d, st);
-    } else {
-      DISPATCH_VARIANT(pl.variant, launch_ds, d, st);
-    }
+    rc = launch_ds_variant(pl.variant, f32 != 0, d, st);
     if (rc) return rc;
 
     if (want_dh) {  // dH[T x H] (+)= dS_tv[T x kv] * W^T[H x kv]^T
@@ -769,7 +628,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
         else
           s.c_out_f32 = pl.dh_acc;
       }
-      rc = pl.kmajor_dh ? run_store_gemm_kmajor(s, false, true, st) : run_store_gemm(s, g_tune.gemm_variant, st);
+      rc = pl.kmajor_dh ? run_store_gemm_kmajor(tn, s, false, true, st) : run_store_gemm(tn, s, tn.gemm_variant, st);
       if (rc) return rc;
     }
     if (want_dw) {  // dW[v0 : v0+rows, H] = dS_vt[rows x kt] * hidden^T[H x kt]^T
@@ -801,7 +660,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
         s.c_out_f32 = (float*)dW_out + (size_t)v0 * H;
       else
         s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
-      rc = pl.kmajor ? run_store_gemm_kmajor(s, true, true, st) : run_store_gemm(s, g_tune.gemm_variant, st);
+      rc = pl.kmajor ? run_store_gemm_kmajor(tn, s, true, true, st) : run_store_gemm(tn, s, tn.gemm_variant, st);
       if (rc) return rc;
     }
     if (dbias_out) {
@@ -1010,11 +869,9 @@ int fgrpo_gemm_nt(const void* A, const void* B, int M, int N, int K, long long l
   s.alpha = alpha;
   if (variant < 0 || variant >= kNumCfg) return fail(FGRPO_ERR_BAD_ARG, "gemm_nt: variant=%d", variant);
   // the hook runs exactly the requested variant
-  const int keep = g_tune.small_variant;
-  g_tune.small_variant = -1;
-  int rc = run_store_gemm(s, variant, (hipStream_t)stream);
-  g_tune.small_variant = keep;
-  return rc;
+  Tuning tn = g_tune;
+  tn.small_variant = -1;
+  return run_store_gemm(tn, s, variant, (hipStream_t)stream);
 }
 
 int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long long lda, long long ldb, int a_kmajor,
@@ -1041,110 +898,11 @@ int fgrpo_gemm_kmajor(const void* A, const void* B, int M, int N, int K, long lo
   s.ldc = ldc;
   s.alpha = alpha;
   if (!a_kmajor && !b_kmajor) {  // K-contiguous operands, A column-blocked
-    const int keep = g_tune.small_variant;
-    g_tune.small_variant = -1;
-    const int rc = run_store_gemm(s, 8, (hipStream_t)stream);
-    g_tune.small_variant = keep;
-    return rc;
+    Tuning tn = g_tune;
+    tn.small_variant = -1;
+    return run_store_gemm(tn, s, 8, (hipStream_t)stream);
   }
-  return run_store_gemm_kmajor(s, a_kmajor != 0, b_kmajor != 0, (hipStream_t)stream);
-}
-
-// ---- packed variable-length attention ------------------------------------------------------------------
-namespace {
-int check_attn(const char* who, const void* q, const void* k, const void* v, long long q_st, long long q_sh,
-               long long k_st, long long k_sh, long long v_st, long long v_sh, const int32_t* cu, int n_seq, int T,
-               int Hq, int Hkv, int D, float scale, const int32_t* bounds_ws) {
-  if (!q || !k || !v || !cu || !bounds_ws) return fail(FGRPO_ERR_BAD_ARG, "%s: null argument", who);
-  if (T <= 0 || n_seq <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0)
-    return fail(FGRPO_ERR_BAD_ARG, "%s: T=%d n_seq=%d Hq=%d Hkv=%d", who, T, n_seq, Hq, Hkv);
-  if (D != 128 && D != 64) return fail(FGRPO_ERR_BAD_ARG, "%s: head dimension %d not supported (128 or 64)", who, D);
-  if (!(scale > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "%s: softmax scale must be positive", who);
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v)) return fail(FGRPO_ERR_ALIGN, "%s: q/k/v must be 16-byte aligned", who);
-  const long long st[6] = {q_st, q_sh, k_st, k_sh, v_st, v_sh};
-  for (int i = 0; i < 6; ++i)
-    if (st[i] <= 0 || st[i] % 8 != 0) return fail(FGRPO_ERR_ALIGN, "%s: strides must be positive multiples of 8 elements", who);
-  return 0;
-}
-
-void fill_attn(AttnParams& p, const void* q, const void* k, const void* v, long long q_st, long long q_sh,
-               long long k_st, long long k_sh, long long v_st, long long v_sh, int T, int Hq, int Hkv, float scale,
-               int causal, int32_t* bounds_ws) {
-  memset(&p, 0, sizeof(p));
-  p.q = (const bf16_t*)q;
-  p.k = (const bf16_t*)k;
-  p.v = (const bf16_t*)v;
-  p.q_st = q_st, p.q_sh = q_sh, p.k_st = k_st, p.k_sh = k_sh, p.v_st = v_st, p.v_sh = v_sh;
-  p.seg_start = bounds_ws;
-  p.seg_end = bounds_ws + T;
-  p.order_k = bounds_ws + attn_order_offset(T, 0);
-  p.order_q = bounds_ws + attn_order_offset(T, 1);      // the query-side launches pick the list of their tile size
-  p.T = T, p.Hq = Hq, p.Hkv = Hkv;
-  p.scale = scale;
-  p.causal = causal != 0;
-}
-}  // namespace
-
-int fgrpo_varlen_attn_bounds(const int32_t* cu, int n_seq, int T, int causal, int32_t* bounds_ws, void* stream) {
-  hipStream_t st = (hipStream_t)stream;
-  if (!cu || !bounds_ws || T <= 0 || n_seq <= 0) return fail(FGRPO_ERR_BAD_ARG, "varlen_attn_bounds: bad argument");
-  hipLaunchKernelGGL(segment_bounds_kernel, dim3((T + 255) / 256), dim3(256), 0, st, cu, n_seq, T, bounds_ws, bounds_ws + T);
-  HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(attn_tile_order_kernel, dim3(4, kAttnOrderSlices), dim3(1024), 0, st, bounds_ws, bounds_ws + T, T, causal != 0, bounds_ws);
-  HIP_TRY(hipGetLastError());
-  return 0;
-}
-
-int fgrpo_varlen_attn_fwd(const void* q, const void* k, const void* v, long long q_st, long long q_sh, long long k_st,
-                          long long k_sh, long long v_st, long long v_sh, const int32_t* cu, int n_seq, int T, int Hq,
-                          int Hkv, int D, float scale, int causal, void* out, float* lse, int32_t* bounds_ws,
-                          int bounds_valid, void* stream) {
-  hipStream_t st = (hipStream_t)stream;
-  int rc = check_attn("varlen_attn_fwd", q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, cu, n_seq, T, Hq, Hkv, D, scale, bounds_ws);
-  if (rc) return rc;
-  if (!out || !lse) return fail(FGRPO_ERR_BAD_ARG, "varlen_attn_fwd: null output");
-  if (!aligned16(out)) return fail(FGRPO_ERR_ALIGN, "varlen_attn_fwd: out must be 16-byte aligned");
-  AttnParams p;
-  fill_attn(p, q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, T, Hq, Hkv, scale, causal, bounds_ws);
-  p.out = (bf16_t*)out;
-  p.lse = lse;
-  if (!bounds_valid) {   // else bounds_ws still holds what an earlier call with the same segments wrote
-    rc = fgrpo_varlen_attn_bounds(cu, n_seq, T, causal, bounds_ws, stream);
-    if (rc) return rc;
-  }
-  return launch_query_side<FwdLauncher>(D, attn_heads_per_group(Hq / Hkv, T, n_seq), p, T, Hq, Hkv, bounds_ws, st);
-}
-
-int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
-                          long long q_st, long long q_sh, long long k_st, long long k_sh, long long v_st, long long v_sh,
-                          const int32_t* cu, int n_seq, int T, int Hq, int Hkv, int D, float scale, int causal, void* dq,
-                          void* dk, void* dv, float* delta_ws, int32_t* bounds_ws, int bounds_valid, void* stream) {
-  hipStream_t st = (hipStream_t)stream;
-  int rc = check_attn("varlen_attn_bwd", q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, cu, n_seq, T, Hq, Hkv, D, scale, bounds_ws);
-  if (rc) return rc;
-  if (!dout || !out || !lse || !dq || !dk || !dv || !delta_ws) return fail(FGRPO_ERR_BAD_ARG, "varlen_attn_bwd: null argument");
-  if (!aligned16(dout) || !aligned16(out) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
-    return fail(FGRPO_ERR_ALIGN, "varlen_attn_bwd: dout/out/dq/dk/dv must be 16-byte aligned");
-  AttnParams p;
-  fill_attn(p, q, k, v, q_st, q_sh, k_st, k_sh, v_st, v_sh, T, Hq, Hkv, scale, causal, bounds_ws);
-  p.lse = const_cast<float*>(lse);
-  p.dout = (const bf16_t*)dout;
-  p.delta = delta_ws;
-  p.out_fwd = (const bf16_t*)out;
-  p.dq = (bf16_t*)dq;
-  p.dk = (bf16_t*)dk;
-  p.dv = (bf16_t*)dv;
-  if (!bounds_valid) {   // else bounds_ws still holds what an earlier call with the same segments wrote
-    rc = fgrpo_varlen_attn_bounds(cu, n_seq, T, causal, bounds_ws, stream);
-    if (rc) return rc;
-  }
-  rc = launch_query_side<DqLauncher>(D, attn_heads_per_group(Hq / Hkv, T, n_seq), p, T, Hq, Hkv, bounds_ws, st);
-  if (rc) return rc;
-  const dim3 grid_k(Hkv, (T + kAttnBQ - 1) / kAttnBQ);
-  if (D == 128) hipLaunchKernelGGL(varlen_attn_dkv_kernel<128>, grid_k, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL(varlen_attn_dkv_kernel<64>, grid_k, dim3(256), 0, st, p);
-  HIP_TRY(hipGetLastError());
-  return 0;
+  return run_store_gemm_kmajor(g_tune, s, a_kmajor != 0, b_kmajor != 0, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -193,40 +193,6 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
   }
 }
 
-// One thread per token: merge the vocabulary splits, emit logprob / entropy / lse.
-struct CombineParams {
-  const float4* part;
-  const float* xt;
-  const long long* labels;
-  int T, V, nsplit;
-  float* lp;    // [T]
-  float* ent;   // [T] or null
-  float* lse;   // [T] or null
-};
-
-__global__ void lmhead_fwd_combine_kernel(const CombineParams p) {
-  const int n = blockIdx.x * blockDim.x + threadIdx.x;
-  if (n >= p.T) return;
-  float4 a = p.part[n];
-  float m = a.x, s = a.y, sx = a.z;
-  for (int k = 1; k < p.nsplit; ++k) {
-    const float4 b = p.part[(long long)k * p.T + n];
-    lse_merge(m, s, sx, b.x, b.y, b.z);
-  }
-  const float lse = m + logf(s);
-  if (p.lse) p.lse[n] = lse;
-  const long long lab = p.labels[n];
-  const bool valid = (lab != -100);
-  float lp = 0.f, ent = 0.f;
-  if (valid) {
-    // a label outside [0, V) has no target logit: report NaN rather than a silent number
-    lp = (lab >= 0 && lab < p.V) ? (p.xt[n] - lse) : __uint_as_float(0x7fc00000u);
-    ent = lse - sx / s;
-  }
-  p.lp[n] = lp;
-  if (p.ent) p.ent[n] = ent;
-}
-
 // ---------------------------------------------------------------------------
 // Backward recompute: dLogits for one vocabulary panel, written as bf16
 //   * in-place mode (tv_blk != 0, vt_hi == null): once, as 256-column blocks [v/256][token][256], which both
@@ -458,6 +424,7 @@ struct StoreParams {
   float alpha;
   const float* alpha_dev;  // optional device scalar multiplied into alpha
   int tiles_m, tiles_n, group_m;
+  int wide_stores;         // ldc and the output / addend bases allow 16-byte pieces (set by the launcher)
 };
 
 // Output is either fp32 or bf16 (never both); rows/cols past M/N are skipped.
@@ -489,6 +456,79 @@ __device__ __forceinline__ void store_tile(const StoreParams& p, f32x16_t (&acc)
   }
 }
 
+// The same stores made wide.  A lane's accumulator holds single elements of 32 different output columns, so direct
+// stores are 2- or 4-byte scalars, 64-byte half lines per instruction.  Here every wavefront parks one 32-row slab of
+// its sub-tile (fp32, already scaled) in a private LDS patch, row-major, and reads it back as 16-byte pieces along
+// the output row: a store instruction then writes 8 consecutive bf16 (or 4 fp32) per lane and whole 128-byte lines per
+// row; the optional addend is loaded the same way.  LDS operations of one wavefront complete in program order, so
+// no barrier is needed between the slab's writes and reads, nor before the next slab overwrites the patch.
+// Needs ldc and the bases such that every piece is 16-byte aligned (checked by the caller); pieces that cross N
+// fall back to scalars.  `smem` must be free (the main loops end with a barrier).  Tiles whose accumulators fill the
+// register file (128x128 per wavefront) keep the scalar stores: the patch addressing would push them into scratch.
+template <class C>
+constexpr bool kStoreViaLds = C::NW * 32 * C::WTN * 4 <= C::LDS_BYTES && C::WTN % 8 == 0 && 64 % (C::WTN / 8) == 0 &&
+                              C::TM * C::TN <= 8;
+
+template <class C, bool HAS_IN, bool OUT_BF16>
+__device__ __forceinline__ void store_tile_lds(const StoreParams& p, f32x16_t (&acc)[C::TM][C::TN], float alpha, int row0,
+                                               int col0, int wm, int wn, int lane, int wave, char* smem) {
+  constexpr int WTN = C::WTN;
+  constexpr int PIECE = OUT_BF16 ? 8 : 4;                 // output elements per lane and store
+  constexpr int LPR = WTN / PIECE;                        // lanes per patch row
+  constexpr int RPP = 64 / LPR;                           // rows per store instruction
+  static_assert(32 % RPP == 0, "patch rows per pass");
+  float* patch = (float*)smem + wave * (32 * WTN);
+  const int prow = lane / LPR, pcol = (lane % LPR) * PIECE;
+  const int n0 = col0 + wn * WTN + pcol;                  // first output column of this lane's pieces
+  const bool n_full = n0 + PIECE <= p.g.N;
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * WTN + j * 32 + (lane & 31)] = acc[i][j][r] * alpha;
+#pragma unroll
+    for (int q = 0; q < 32 / RPP; ++q) {
+      const int rr = q * RPP + prow;
+      const int m = row0 + wm * C::WTM + i * 32 + rr;
+      float v[PIECE];
+#pragma unroll
+      for (int e = 0; e < PIECE; e += 4) {
+        const float4 t = *(const float4*)(patch + rr * WTN + pcol + e);
+        v[e] = t.x, v[e + 1] = t.y, v[e + 2] = t.z, v[e + 3] = t.w;
+      }
+      if (m >= p.g.M || n0 >= p.g.N) continue;
+      const long long o = (long long)m * p.ldc + n0;
+      if (n_full) {
+        if (HAS_IN) {
+#pragma unroll
+          for (int e = 0; e < PIECE; e += 4) {
+            const float4 t = *(const float4*)(p.c_in + o + e);
+            v[e] += t.x, v[e + 1] += t.y, v[e + 2] += t.z, v[e + 3] += t.w;
+          }
+        }
+        if (OUT_BF16) {
+          u32x4_t w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[PIECE - 4], v[PIECE - 3]),
+                       pack_bf16x2(v[PIECE - 2], v[PIECE - 1])};
+          *(u32x4_t*)(p.c_out_bf16 + o) = w;
+        } else {
+          *(float4*)(p.c_out_f32 + o) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      } else {
+        for (int e = 0; e < PIECE && n0 + e < p.g.N; ++e) {
+          float x = v[e];
+          if (HAS_IN) x += p.c_in[o + e];
+          if (OUT_BF16)
+            p.c_out_bf16[o + e] = f32_to_bf16_rn(x);
+          else
+            p.c_out_f32[o + e] = x;
+        }
+      }
+    }
+  }
+}
+
 template <class C, bool AKM = false, bool BKM = false>
 __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StoreParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -514,116 +554,22 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
 
   const float alpha = p.alpha * (p.alpha_dev ? *p.alpha_dev : 1.f);
   const int mode = (p.c_in ? 1 : 0) | (p.c_out_bf16 ? 2 : 0);
+  if constexpr (kStoreViaLds<C>) {
+    if (p.wide_stores) {
+      switch (mode) {
+        case 0: store_tile_lds<C, false, false>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+        case 1: store_tile_lds<C, true, false>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+        case 2: store_tile_lds<C, false, true>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+        default: store_tile_lds<C, true, true>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+      }
+      return;
+    }
+  }
   switch (mode) {
     case 0: store_tile<C, false, false>(p, acc, alpha, row0, col0, wm, wn, lane); break;
     case 1: store_tile<C, true, false>(p, acc, alpha, row0, col0, wm, wn, lane); break;
     case 2: store_tile<C, false, true>(p, acc, alpha, row0, col0, wm, wn, lane); break;
     default: store_tile<C, true, true>(p, acc, alpha, row0, col0, wm, wn, lane); break;
-  }
-}
-
-// ---------------------------------------------------------------------------
-// Operand preparation: copy / transpose a [R x Cn] matrix (fp32 or bf16) into a
-// zero-padded bf16 buffer, optionally also emitting the bf16 low half of an fp32
-// source (x ~= hi + lo).  Destination is [Rpad x ld] (or [Cpad x ld] transposed).
-// ---------------------------------------------------------------------------
-struct ConvertParams {
-  const void* src;
-  int src_is_f32;
-  long long ld_src;
-  int R, Cn;          // logical source shape
-  int Rpad, Cpad;     // padded extents written
-  bf16_t* hi;
-  bf16_t* lo;         // or null
-  long long ld_dst;
-  int transpose;
-};
-
-__global__ __launch_bounds__(256) void convert_pad_kernel(const ConvertParams p) {
-  __shared__ float th[64][65];
-  __shared__ float tl[64][65];
-  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
-  for (int rr = ty; rr < 64; rr += 4) {
-    const int r = r0 + rr, c = c0 + tx;
-    float v = 0.f;
-    if (r < p.R && c < p.Cn) {
-      const long long o = (long long)r * p.ld_src + c;
-      v = p.src_is_f32 ? ((const float*)p.src)[o] : bf16_to_f32(((const bf16_t*)p.src)[o]);
-    }
-    const float h = bf16_to_f32(f32_to_bf16_rn(v));
-    th[rr][tx] = h;
-    tl[rr][tx] = v - h;
-  }
-  __syncthreads();
-  if (!p.transpose) {
-    for (int rr = ty; rr < 64; rr += 4) {
-      const int r = r0 + rr, c = c0 + tx;
-      if (r < p.Rpad && c < p.Cpad) {
-        const long long o = (long long)r * p.ld_dst + c;
-        p.hi[o] = f32_to_bf16_rn(th[rr][tx]);
-        if (p.lo) p.lo[o] = f32_to_bf16_rn(tl[rr][tx]);
-      }
-    }
-  } else {
-    for (int cc = ty; cc < 64; cc += 4) {
-      const int c = c0 + cc, r = r0 + tx;
-      if (c < p.Cpad && r < p.Rpad) {
-        const long long o = (long long)c * p.ld_dst + r;
-        p.hi[o] = f32_to_bf16_rn(th[tx][cc]);
-        if (p.lo) p.lo[o] = f32_to_bf16_rn(tl[tx][cc]);
-      }
-    }
-  }
-}
-
-__global__ void to_f32_kernel(const void* src, int src_is_f32, float* dst, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) dst[i] = src_is_f32 ? ((const float*)src)[i] : bf16_to_f32(((const bf16_t*)src)[i]);
-}
-
-// dbias from the [token][vocab] panel alone: out[v] = sum_t tv[t][v].  One block owns 64 columns; its four
-// row groups are combined in a fixed order, so the result does not depend on scheduling.
-__global__ void panel_col_sum_kernel(const bf16_t* tv_hi, const bf16_t* tv_lo, long long ld, long long blk, int rows_t,
-                                     int cols, float* out_f32, bf16_t* out_bf16) {
-  __shared__ float red[4][64];
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  const int c = blockIdx.x * 64 + tx;
-  float s = 0.f;
-  if (c < cols) {
-    // blk != 0: 256-column blocks of row length 256 (block b at + b * blk)
-    const long long base = blk ? (long long)(c >> 8) * blk + (c & 255) : (long long)c;
-    const long long step = blk ? 256 : ld;
-    for (int t = ty; t < rows_t; t += 4) {
-      s += bf16_to_f32(tv_hi[base + (long long)t * step]);
-      if (tv_lo) s += bf16_to_f32(tv_lo[base + (long long)t * step]);
-    }
-  }
-  red[ty][tx] = s;
-  __syncthreads();
-  if (ty == 0 && c < cols) {
-    const float r = (red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]);
-    if (out_f32) out_f32[c] = r;
-    if (out_bf16) out_bf16[c] = f32_to_bf16_rn(r);
-  }
-}
-
-// bias gradient: db[v] = sum_t dS[v][t] over one [vocab][token] panel
-__global__ void panel_row_sum_kernel(const bf16_t* vt_hi, const bf16_t* vt_lo, long long ld, int rows, int cols,
-                                     float* out_f32, bf16_t* out_bf16) {
-  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (row >= rows) return;
-  float s = 0.f;
-  for (int c = lane; c < cols; c += 64) {
-    s += bf16_to_f32(vt_hi[(long long)row * ld + c]);
-    if (vt_lo) s += bf16_to_f32(vt_lo[(long long)row * ld + c]);
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
-  if (lane == 0) {
-    if (out_f32) out_f32[row] = s;
-    if (out_bf16) out_bf16[row] = f32_to_bf16_rn(s);
   }
 }
 

@@ -132,17 +132,36 @@ def test_ragged_shapes(dev, T, H, V, dtype):
     check(want, got, o, g, f32=(dtype == "fp32"))
 
 
+LMHEAD_VARIANTS = (2, 3, 4, 7, 8, 9)     # tile ids the LM-head kernels are built for (the plain GEMM has all ten)
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
 def test_every_tile_variant(dev, variant):
     from fgrpo import _lib
     from fgrpo.synthetic import make_workload
     w = make_workload("cfg1", seed=4, overrides=dict(H=192, V=9000, tokens=1400, len_lo=8, len_hi=200, h_scale=1.0))
-    _lib.set_tuning(fwd_variant=variant, ds_variant=variant, gemm_variant=variant, small_variant=-1)
+    lm = variant if variant in LMHEAD_VARIANTS else 8
+    _lib.set_tuning(fwd_variant=lm, ds_variant=lm, gemm_variant=variant, small_variant=-1, bwd_kmajor=0)
     try:
         want, got, o, g, _, _ = run_case(w, dev, "north_star")
     finally:
-        _lib.set_tuning(fwd_variant=8, ds_variant=8, gemm_variant=8, small_variant=4)
+        _lib.set_tuning(fwd_variant=8, ds_variant=8, gemm_variant=8, small_variant=4, bwd_kmajor=2)
     check(want, got, o, g, f32=False)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 5, 6])
+def test_unbuilt_lmhead_variants_are_refused(dev, variant):
+    """Tile ids whose LM-head kernels would spill to scratch are not built: asking for one fails loudly."""
+    from fgrpo import _lib, ops
+    h = torch.randn(512, 128, device=dev).bfloat16()
+    W = torch.randn(2048, 128, device=dev).bfloat16()
+    y = torch.randint(0, 2048, (512,), device=dev)
+    _lib.set_tuning(fwd_variant=variant, small_variant=-1)
+    try:
+        with pytest.raises(RuntimeError, match="not built"):
+            ops.lmhead_logprob_fwd(h, W, None, y, 1.0)
+    finally:
+        _lib.set_tuning(fwd_variant=8, small_variant=4)
 
 
 def test_bias_and_temperature(dev):
