@@ -71,6 +71,7 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "bwd_kmajor")) return &g_tune.bwd_kmajor;
   if (!strcmp(key, "attn_heads")) return &g_tune.attn_heads;
   if (!strcmp(key, "wide_stores")) return &g_tune.wide_stores;
+  if (!strcmp(key, "keep_panels")) return &g_tune.keep_panels;
   return nullptr;
 }
 
@@ -390,9 +391,19 @@ void plan_bwd(const Tuning& tn, BwdPlan& pl, void* ws, int T, int H, int V, int 
 }  // namespace
 
 namespace {
+// Conditions of the kept-logits pair: the forward on the 256x256x64 two-buffer tile with operands used in place,
+// both gradient GEMMs on operands read where they lie.
+bool keep_supported(const Tuning& tn, int T, int H, int V, int dtype) {
+  if (dtype != FGRPO_BF16 || T <= 0 || V <= 0 || H <= 0 || H % 256 != 0) return false;
+  if (pick_variant(tn, 8, V, T) != 8) return false;
+  const long long th = (long long)((T + 255) / 256) * (H / 256), vh = (long long)((V + 255) / 256) * (H / 256);
+  return th >= num_cus() / 2 && vh >= num_cus() / 2;
+}
+size_t keep_bytes(int T, int V) { return (size_t)round_up(V, 256) * (size_t)round_up(T, 256) * sizeof(bf16_t); }
+
 int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
                       int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
-                      size_t ws_bytes, void* stream) {
+                      size_t ws_bytes, void* stream, void* keep = nullptr) {
   hipStream_t st = (hipStream_t)stream;
   if (!hidden || !weight || !labels || !lp_out) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: null argument");
   if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: T=%d H=%d V=%d", T, H, V);
@@ -400,9 +411,11 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: inv_temperature must be positive");
   if (!ws || !aligned16(ws)) return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd: workspace null or misaligned");
   if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "logprob_fwd: hidden/weight must be 16-byte aligned");
-  const Tuning tn = g_tune;   // one reading of the tuning state per call
+  Tuning tn = g_tune;   // one reading of the tuning state per call
+  if (keep) tn.fwd_variant = 8;
   FwdPlan pl;
   plan_fwd(tn, pl, ws, T, H, V, dtype, bias != nullptr);
+  if (keep && (pl.variant != 8 || pl.copy_ops)) return fail(FGRPO_ERR_UNSUPPORTED, "logprob_fwd_keep: shape not supported");
   if (pl.bytes > ws_bytes) return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd: workspace %zu < %zu bytes", ws_bytes, pl.bytes);
 
   FwdParams p;
@@ -425,7 +438,13 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   p.group_t = tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
   p.part = pl.part;
   p.xt = pl.xt;
-  rc = launch_fwd_variant(pl.variant, p, st);
+  if (keep) {
+    p.keep = (bf16_t*)keep;
+    p.keep_blk = (long long)pl.tiles_t * kCfg[8].bn * 256;
+    rc = launch_fwd_keep(p, st);
+  } else {
+    rc = launch_fwd_variant(pl.variant, p, st);
+  }
   if (rc) return rc;
 
   CombineParams c{pl.part, pl.xt, (const long long*)labels, T, V, pl.nsplit, lp_out, ent_out, lse_out};
@@ -674,6 +693,133 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
                            (long long)pl.Tpad, rows, T, o32, o16);
       HIP_TRY(hipGetLastError());
     }
+  }
+  return 0;
+}
+
+int fgrpo_keep_supported(int T, int H, int V, int dtype) { return keep_supported(g_tune, T, H, V, dtype) ? 1 : 0; }
+
+size_t fgrpo_logits_keep_bytes(int T, int V) { return (T > 0 && V > 0) ? keep_bytes(T, V) : 0; }
+
+int fgrpo_logprob_fwd_keep(const void* hidden, const void* weight, const void* bias, const int64_t* labels,
+                           float inv_temp, int T, int H, int V, int dtype, float* lp_out, float* ent_out,
+                           float* lse_out, void* logits_keep, size_t logits_keep_bytes, void* ws, size_t ws_bytes,
+                           void* stream) {
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd_keep: T=%d H=%d V=%d", T, H, V);
+  if (!keep_supported(g_tune, T, H, V, dtype))
+    return fail(FGRPO_ERR_UNSUPPORTED, "logprob_fwd_keep: needs bf16, H %% 256 == 0 and a device-filling problem (T=%d H=%d V=%d)", T, H, V);
+  if (!logits_keep || !aligned16(logits_keep) || logits_keep_bytes < keep_bytes(T, V))
+    return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd_keep: logits buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
+  return logprob_fwd_impl(hidden, weight, bias, labels, inv_temp, T, H, V, dtype, lp_out, ent_out, lse_out, ws, ws_bytes,
+                          stream, logits_keep);
+}
+
+namespace {
+// Vocabulary panels of the kept-logits backward.  One by default: each gradient GEMM is a single launch over the
+// whole vocabulary, dH is written once and nothing is accumulated (measured at T=32768, H=1536, V=151936:
+// 1 or 2 panels 26.8 ms, 7 panels 27.2, 10 panels 30.7).  The tuning key keep_panels splits them.
+void kept_panels(const Tuning& tn, int T, int H, int V, int& panel, int& npanels) {
+  (void)T;
+  (void)H;
+  int np = tn.keep_panels > 0 ? tn.keep_panels : 1;
+  const int max_np = (V + 255) / 256;
+  np = np < 1 ? 1 : (np > max_np ? max_np : np);
+  panel = (int)round_up((V + np - 1) / np, 256);
+  npanels = (V + panel - 1) / panel;
+}
+}  // namespace
+
+size_t fgrpo_lmhead_bwd_kept_workspace(int T, int H, int V, int dtype) {
+  if (T <= 0 || H <= 0 || V <= 0 || dtype != FGRPO_BF16) return 0;
+  int panel = 0, np = 0;
+  kept_panels(g_tune, T, H, V, panel, np);
+  // sized for any panel count: a concurrent set_tuning must not turn a sufficient workspace into a short one
+  (void)np;
+  return (size_t)round_up((long long)T * H * (long long)sizeof(float), 256);
+}
+
+int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bias, const int64_t* labels,
+                          const float* lse, const float* g, const float* gout_dev, float inv_temp, int T, int H, int V,
+                          int dtype, void* logits_keep, size_t logits_keep_bytes, void* dH_out, void* dW_out,
+                          void* dbias_out, void* ws, size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!hidden || !weight || !labels || !lse || !g) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: null argument");
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: T=%d H=%d V=%d", T, H, V);
+  if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: inv_temperature must be positive");
+  const Tuning tn = g_tune;
+  if (!keep_supported(tn, T, H, V, dtype))
+    return fail(FGRPO_ERR_UNSUPPORTED, "lmhead_bwd_kept: needs bf16, H %% 256 == 0 and a device-filling problem (T=%d H=%d V=%d)", T, H, V);
+  if (!logits_keep || !aligned16(logits_keep) || logits_keep_bytes < keep_bytes(T, V))
+    return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: logits buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
+  if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: dbias requested without a bias");
+  if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "lmhead_bwd_kept: hidden/weight must be 16-byte aligned");
+  if (!dH_out && !dW_out && !dbias_out) return 0;
+  const int Tpad = (int)round_up(T, 256), Vpad = (int)round_up(V, 256);
+  const long long blk = (long long)Tpad * 256;
+  bf16_t* ds = (bf16_t*)logits_keep;
+  int panel = 0, npanels = 0;
+  kept_panels(tn, T, H, V, panel, npanels);
+  float* dh_acc = nullptr;
+  if (dH_out && npanels > 1) {
+    if (!ws || !aligned16(ws) || ws_bytes < (size_t)T * H * sizeof(float))
+      return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: workspace null, misaligned or smaller than %zu bytes", (size_t)T * H * sizeof(float));
+    dh_acc = (float*)ws;
+  }
+
+  KeptParams k{ds, blk, Tpad, T, V, (const long long*)labels, lse, g, gout_dev, inv_temp};
+  hipLaunchKernelGGL(kept_logits_to_dlogits_kernel, dim3((unsigned)((Vpad / 256) * (Tpad / kKeptRows))), dim3(256), 0, st, k);
+  HIP_TRY(hipGetLastError());
+
+  int rc = 0;
+  for (int pi = 0; pi < npanels; ++pi) {
+    const int v0 = pi * panel;
+    const int rows = (V - v0) < panel ? (V - v0) : panel;      // vocabulary rows of W / dW in this panel
+    const int kv = (int)round_up(rows, 256);                   // dLogits columns of the panel (zero past V)
+    bf16_t* ds_p = ds + (long long)(v0 / 256) * blk;
+    if (dH_out) {   // dH[T x H] (+)= dS[T x kv] W[v0 : v0+rows, H]: A column-blocked K-contiguous, B = W read in place
+      StoreParams s;
+      memset(&s, 0, sizeof(s));
+      s.g.M = T;
+      s.g.N = H;
+      s.g.lda = 256;
+      s.g.a_blk = blk;
+      s.g.ldb = H;
+      s.g.nseg = 1;
+      s.g.seg[0] = GemmSeg{ds_p, (const bf16_t*)weight + (size_t)v0 * H, kv};
+      s.g.kb_valid = rows;
+      s.ldc = H;
+      s.alpha = 1.f;
+      const bool first = (pi == 0), last = (pi == npanels - 1);
+      s.c_in = first ? nullptr : dh_acc;
+      if (last)
+        s.c_out_bf16 = (bf16_t*)dH_out;
+      else
+        s.c_out_f32 = dh_acc;
+      rc = run_store_gemm_kmajor(tn, s, false, true, st);
+      if (rc) return rc;
+    }
+    if (dW_out) {   // dW[v0 : v0+rows, H] = dS^T[rows x Tpad] hidden[Tpad x H]: the token is the contraction row of both
+      StoreParams s;
+      memset(&s, 0, sizeof(s));
+      s.g.M = rows;
+      s.g.N = H;
+      s.g.lda = 256;
+      s.g.a_blk = blk;
+      s.g.ldb = H;
+      s.g.nseg = 1;
+      s.g.seg[0] = GemmSeg{ds_p, (const bf16_t*)hidden, Tpad};
+      s.g.kb_valid = T;
+      s.ldc = H;
+      s.alpha = 1.f;
+      s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
+      rc = run_store_gemm_kmajor(tn, s, true, true, st);
+      if (rc) return rc;
+    }
+  }
+  if (dbias_out) {
+    hipLaunchKernelGGL(panel_col_sum_kernel, dim3((V + 63) / 64), dim3(256), 0, st, ds, (const bf16_t*)nullptr,
+                       (long long)Vpad, blk, T, V, (float*)nullptr, (bf16_t*)dbias_out);
+    HIP_TRY(hipGetLastError());
   }
   return 0;
 }

@@ -88,6 +88,7 @@ struct Tuning {
   int bwd_kmajor = 2;      // 0: transposed copies; 1: the dW GEMM reads dLogits and hidden in place; 2: the dH GEMM reads W in place too
   int attn_heads = 0;      // query heads per work-group of the attention forward / dQ kernels (1, 2, 4); 0 = heuristic
   int wide_stores = 1;     // GEMM epilogues write 16-byte pieces through an LDS patch where alignment allows
+  int keep_panels = 0;     // kept-logits backward: vocabulary panels of the gradient GEMMs; 0 = one
 };
 extern Tuning g_tune;
 
@@ -121,6 +122,8 @@ int launch_tile_kernel(const P& p, int nblocks, hipStream_t st) {
 // lmhead_variant_built() accepts; the others are refused with FGRPO_ERR_UNSUPPORTED.
 bool lmhead_variant_built(int variant);
 int launch_fwd_variant(int variant, const FwdParams& p, hipStream_t st);
+// the forward that also keeps the bf16 logits (tile id 8 only)
+int launch_fwd_keep(const FwdParams& p, hipStream_t st);
 // split: fp32 inputs, dS written as bf16 hi + lo halves (small tile only)
 int launch_ds_variant(int variant, bool split, const DsParams& p, hipStream_t st);
 int launch_store_variant(int variant, const StoreParams& p, hipStream_t st);

@@ -36,6 +36,10 @@ int launch_fwd_variant(int variant, const FwdParams& p, hipStream_t st) {
   DISPATCH_LMHEAD(variant, launch_fwd, p, st);
 }
 
+int launch_fwd_keep(const FwdParams& p, hipStream_t st) {
+  return launch_tile_kernel<lmhead_fwd_kernel<Cfg8, true>, Cfg8>(p, p.tiles_t * p.nsplit, st);
+}
+
 int launch_ds_variant(int variant, bool split, const DsParams& p, hipStream_t st) {
   // fp32 inputs: dS is written as bf16 hi + lo halves; only the small tile carries that epilogue
   if (split) return launch_tile_kernel<lmhead_ds_kernel<Cfg4, true>, Cfg4>(p, p.tiles_t * p.nsplit, st);

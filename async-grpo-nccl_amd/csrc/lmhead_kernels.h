@@ -46,9 +46,57 @@ struct FwdParams {
   int tiles_v, tiles_t, nsplit, group_t;
   float4* part;              // [nsplit][T] : (m, s, sx, unused)
   float* xt;                 // [T] target logit (written only where a valid label exists)
+  // KEEP kernels only: the raw products x = W h + b (before the temperature), rounded to bf16, for the backward
+  // that does not recompute them.  Column-blocked [V/256][keep_rows][256]: element (t, v) at
+  // (v / 256) * keep_blk + t * 256 + v % 256, keep_blk = keep_rows * 256, keep_rows = token tiles * BN.
+  bf16_t* keep;
+  long long keep_blk;
 };
 
-template <class C>
+// One 32-token x WTM-entry slab of bf16 values (the sub-tile column block j of a wavefront in the LM-head
+// orientation: lane = token, 16 vocabulary rows per 32x32 block) written to a column-blocked buffer through the
+// wavefront's private LDS patch: a lane's 8 bytes (4 vocabulary entries of one token) would be a 64-line scatter per
+// store instruction; parked in the patch and read back as 16-byte pieces, PPT lanes per token row, every store
+// instruction fills whole 128-byte lines.  Patch rows are unpadded; the 8-byte slots of row n are XOR-swizzled with
+// n so that the 32 lanes of a write hit 32 different slots.  LDS traffic is inline assembly (the compiler would
+// otherwise wait for the direct-to-LDS loads of the next tile that are in flight); LDS operations of one wavefront
+// complete in order, so one wait before the stores is enough.  `out` points at (first token of the slab, first
+// vocabulary entry of the wavefront's rows) in the block; pk(i, q) returns the packed entries
+// i*32 + 8*q + 4*(lane/32) + 0..3 of this lane's token.
+template <class C, class PK>
+__device__ __forceinline__ void store_slab_via_patch(char* patch, bf16_t* out, int lane_v, PK&& pk) {
+  constexpr int ROWP = C::WTM * 2;                       // patch row: one token's WTM entries
+  constexpr int NSLOT = ROWP / 8;                        // 8-byte slots per row
+  constexpr int PPT = ROWP / 16, TPP = 64 / PPT;         // 16-byte pieces per token, tokens per store instruction
+  static_assert(64 % PPT == 0 && 32 % TPP == 0 && (NSLOT & (NSLOT - 1)) == 0, "epilogue patch");
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint2 v = pk(i, q);
+      const int slot = ((i * 32 + 8 * q) >> 2) + (lane_v >> 5);
+      lds_write_b64_asm(lds_addr(patch) + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3), v.x, v.y);
+    }
+  u32x4_t pv[32 / TPP];
+#pragma unroll
+  for (int r = 0; r < 32 / TPP; ++r) {
+    const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
+    const int m = tok & (NSLOT - 1);
+    pv[r] = __builtin_bit_cast(u32x4_t, lds_read_b128_asm<0>(lds_addr(patch) + tok * ROWP + ((piece ^ (m >> 1)) << 4)));
+  }
+  wait_lgkm<0>();
+  __builtin_amdgcn_sched_barrier(0);     // nothing that consumes pv may move above the wait
+#pragma unroll
+  for (int r = 0; r < 32 / TPP; ++r) {
+    const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
+    const int m = tok & (NSLOT - 1);
+    u32x4_t v = pv[r];
+    if (m & 1) v = u32x4_t{v[2], v[3], v[0], v[1]};       // odd rows hold the two slots of a piece swapped
+    *(u32x4_t*)(out + (long long)tok * 256 + piece * 8) = v;
+  }
+}
+
+template <class C, bool KEEP = false>
 __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -79,6 +127,12 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
     long long lab = (n < T) ? p.labels[n] : -1;
     y[j] = (lab >= 0 && lab < V) ? (int)lab : -1;
   }
+
+  // KEEP: the wavefront's patch lives behind LDS buffer 0, which the prefetch of the next tile may already be filling
+  constexpr int KEEP_PATCH = C::NW * 32 * C::WTM * 2;
+  static_assert(!KEEP || (kSplitPrologue<C> && C::BM == 256 && C::STAGE + KEEP_PATCH <= C::LDS_BYTES),
+                "kept logits: 256-row tiles on the two-buffer direct-to-LDS loop");
+  char* patch = smem + C::STAGE + wave * (32 * C::WTM * 2);
 
   // With the two-buffer direct-to-LDS loop the first K slice of the NEXT vocabulary tile is requested before this
   // tile's statistics are folded in, so its latency hides under that arithmetic.
@@ -154,6 +208,18 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
             hit = hit || h;
           }
         if (hit) p.xt[col0 + acc_col<C>(wn, j, lane)] = xv * p.inv_temp;
+      }
+      if constexpr (KEEP) {
+        // the addresses are recomputed per tile on purpose (hoisted they would sit in registers across the main loop)
+        int lane_v = lane;
+        asm volatile("" : "+v"(lane_v));
+        bf16_t* out = p.keep + (long long)vt * p.keep_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
+        store_slab_via_patch<C>(patch, out, lane_v, [&](int i, int q) {
+          uint2 pk;
+          pk.x = pack_bf16x2(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
+          pk.y = pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+          return pk;
+        });
       }
     }
   }

@@ -145,4 +145,84 @@ __global__ void panel_row_sum_kernel(const bf16_t* vt_hi, const bf16_t* vt_lo, l
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Backward without recomputation: the forward kept x = W h + b (bf16, column-blocked [V/256][rows][256]); this
+// kernel turns the buffer into dLogits in place,
+//   dS[t, v] = c_t * (1[v == y_t] - exp(x_tv / temperature - lse_t)),  c_t = g_t * gout / temperature,
+// which the two gradient GEMMs then read where it lies.  Rows with c_t == 0 (ignored labels, zero gradient, padding
+// rows t >= T) are written as zeros without being read.  HBM-bound: 2 bytes read and 2 written per logit.
+// One work-group = 64 token rows of one 256-column block (32 KiB, contiguous); a row is 32 lanes x 16 bytes.
+// ---------------------------------------------------------------------------
+struct KeptParams {
+  bf16_t* x;                 // in: kept logits, out: dLogits
+  long long blk;             // elements between column blocks (= rows * 256)
+  int rows;                  // token rows per block (multiple of 64, >= T)
+  int T, V;
+  const long long* labels;   // shifted labels [T]
+  const float* lse;          // [T]
+  const float* gtok;         // [T]
+  const float* gout;         // device scalar or null
+  float inv_temp;
+};
+
+constexpr int kKeptRows = 64;
+
+__global__ __launch_bounds__(256) void kept_logits_to_dlogits_kernel(const KeptParams p) {
+  __shared__ float s_c[kKeptRows], s_l2[kKeptRows];
+  __shared__ int s_y[kKeptRows];
+  const int chunks = p.rows / kKeptRows;
+  const int vb = blockIdx.x / chunks, t0 = (blockIdx.x - vb * chunks) * kKeptRows;
+  const int tid = threadIdx.x;
+  if (tid < kKeptRows) {
+    const int t = t0 + tid;
+    float c = 0.f, l2 = 0.f;
+    int y = -1;
+    if (t < p.T) {
+      const long long lab = p.labels[t];
+      if (lab != -100) {
+        c = p.gtok[t] * (p.gout ? *p.gout : 1.f) * p.inv_temp;
+        l2 = p.lse[t] * kLog2e;
+        y = (lab >= 0 && lab < p.V) ? (int)lab - vb * 256 : -1;    // column inside this block, or out of range
+      }
+    }
+    s_c[tid] = c;
+    s_l2[tid] = l2;
+    s_y[tid] = y;
+  }
+  __syncthreads();
+  const float xs = p.inv_temp * kLog2e;
+  const int r0 = tid >> 5, cpos = (tid & 31) * 8;          // row inside a pass of 8 rows, first column of the lane
+  u32x4_t* base = (u32x4_t*)(p.x + (long long)vb * p.blk + (long long)t0 * 256) + tid;   // + pass * 256 pieces
+  u32x4_t v[kKeptRows / 8];
+#pragma unroll
+  for (int ps = 0; ps < kKeptRows / 8; ++ps)
+    if (s_c[ps * 8 + r0] != 0.f) v[ps] = __builtin_nontemporal_load(base + ps * 256);
+#pragma unroll
+  for (int ps = 0; ps < kKeptRows / 8; ++ps) {
+    const int r = ps * 8 + r0;
+    const float c = s_c[r];
+    u32x4_t o = {0u, 0u, 0u, 0u};
+    if (c != 0.f) {
+      const float nc = -c, l2 = s_l2[r];
+      const int yrel = s_y[r] - cpos;                       // 0..7 when the target sits in this lane's piece
+      float d[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t w = v[ps][e];
+        const float x0 = __uint_as_float(w << 16), x1 = __uint_as_float(w & 0xffff0000u);
+        d[2 * e] = nc * fast_exp2(__builtin_fmaf(x0, xs, -l2));
+        d[2 * e + 1] = nc * fast_exp2(__builtin_fmaf(x1, xs, -l2));
+      }
+      if (yrel >= 0 && yrel < 8) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d[e] += (e == yrel) ? c : 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(d[2 * e], d[2 * e + 1]);
+    }
+    __builtin_nontemporal_store(o, base + ps * 256);
+  }
+}
+
 }  // namespace fgrpo

@@ -31,6 +31,12 @@ SIGNATURES = {
     "fgrpo_lmhead_bwd_workspace": (_sz, [_i, _i, _i, _i, _ll]),
     "fgrpo_lmhead_bwd_panel_cols": (_i, [_i, _i, _i, _i, _ll]),
     "fgrpo_lmhead_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _vp, _vp, _ll, _vp, _sz, _vp]),
+    "fgrpo_keep_supported": (_i, [_i, _i, _i, _i]),
+    "fgrpo_logits_keep_bytes": (_sz, [_i, _i]),
+    "fgrpo_logprob_fwd_keep": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp]),
+    "fgrpo_lmhead_bwd_kept_workspace": (_sz, [_i, _i, _i, _i]),
+    "fgrpo_lmhead_bwd_kept": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp,
+                                   _vp, _sz, _vp]),
     "fgrpo_loss_fwd_workspace": (_sz, [_i, _i]),
     "fgrpo_loss_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _f, _f, _i, _d,
                             _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

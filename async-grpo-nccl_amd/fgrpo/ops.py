@@ -83,11 +83,23 @@ def set_fwd_event_sink(sink) -> None:
     _fwd_event_sink = sink
 
 
+def keep_supported(T: int, H: int, V: int, dtype: torch.dtype) -> bool:
+    """Whether the kept-logits forward/backward pair handles this problem (bf16, H % 256 == 0, device-filling)."""
+    if dtype != torch.bfloat16 or T <= 0:
+        return False
+    return bool(_lib.load().fgrpo_keep_supported(int(T), int(H), int(V), _lib.BF16))
+
+
+def logits_keep_bytes(T: int, V: int) -> int:
+    return int(_lib.load().fgrpo_logits_keep_bytes(int(T), int(V)))
+
+
 def lmhead_logprob_fwd(hidden: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
                        labels_shifted: torch.Tensor, temperature: float = 1.0,
-                       want_entropy: bool = True, want_lse: bool = True):
+                       want_entropy: bool = True, want_lse: bool = True, keep: bool = False):
     """hidden [T,H], weight [V,H] (same dtype, bf16 or fp32), labels_shifted [T] int64
-    -> (lp [T] fp32, entropy [T] fp32 | None, lse [T] fp32 | None)."""
+    -> (lp [T] fp32, entropy [T] fp32 | None, lse [T] fp32 | None); with ``keep`` a fourth result, the uint8 buffer
+    holding the bf16 logits in the library's blocked layout, for ``lmhead_bwd_kept``."""
     dev = _require_cuda(hidden, weight, bias, labels_shifted)
     lib = _lib.load()
     if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
@@ -109,23 +121,32 @@ def lmhead_logprob_fwd(hidden: torch.Tensor, weight: torch.Tensor, bias: Optiona
     lp = torch.empty(T, dtype=torch.float32, device=dev)
     ent = torch.empty(T, dtype=torch.float32, device=dev) if want_entropy else None
     lse = torch.empty(T, dtype=torch.float32, device=dev) if want_lse else None
+    if keep and not keep_supported(T, H, V, weight.dtype):
+        raise RuntimeError(f"fgrpo: the kept-logits forward does not handle T={T} H={H} V={V} {weight.dtype}")
     if T == 0:
         return lp, ent, lse
     nbytes = lib.fgrpo_logprob_fwd_workspace(T, H, V, code)
     ws = _ws(nbytes, dev)
+    kept = torch.empty(lib.fgrpo_logits_keep_bytes(T, V), dtype=torch.uint8, device=dev) if keep else None
     with torch.cuda.device(dev):
         sink = _fwd_event_sink
         if sink is not None:
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-        rc = lib.fgrpo_logprob_fwd(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted),
-                                   1.0 / float(temperature), T, H, V, code,
-                                   _ptr(lp), _ptr(ent), _ptr(lse), _ptr(ws), ws.numel(), _stream())
+        if keep:
+            rc = lib.fgrpo_logprob_fwd_keep(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted),
+                                            1.0 / float(temperature), T, H, V, code,
+                                            _ptr(lp), _ptr(ent), _ptr(lse), _ptr(kept), kept.numel(),
+                                            _ptr(ws), ws.numel(), _stream())
+        else:
+            rc = lib.fgrpo_logprob_fwd(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted),
+                                       1.0 / float(temperature), T, H, V, code,
+                                       _ptr(lp), _ptr(ent), _ptr(lse), _ptr(ws), ws.numel(), _stream())
         if sink is not None:
             e1.record()
             sink.append((e0, e1))
-    _lib.check(rc, "logprob_fwd")
-    return lp, ent, lse
+    _lib.check(rc, "logprob_fwd_keep" if keep else "logprob_fwd")
+    return (lp, ent, lse, kept) if keep else (lp, ent, lse)
 
 
 def lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torch.Tensor],
@@ -164,6 +185,39 @@ def lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torc
                                   _ptr(dH), _ptr(dW), _ptr(db), int(panel_elems_hint),
                                   _ptr(ws), ws.numel(), _stream())
     _lib.check(rc, "lmhead_bwd")
+    return dH, dW, db
+
+
+def lmhead_bwd_kept(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torch.Tensor], temperature: float,
+                    kept: torch.Tensor, need_dh: bool, need_dw: bool, need_db: bool):
+    """The backward on the logits the forward kept (``lmhead_logprob_fwd(..., keep=True)``): ``kept`` is turned into
+    dLogits in place (its contents are spent afterwards), then dH / dW / dbias come from one GEMM each."""
+    dev = _require_cuda(hidden, weight, labels_shifted, lse, g, kept)
+    lib = _lib.load()
+    T, H = hidden.shape
+    V = weight.shape[0]
+    code = _code(weight.dtype)
+    hidden = _aligned(hidden)
+    weight = _aligned(weight)
+    if bias is not None:
+        bias = bias.detach().to(weight.dtype).contiguous()
+    labels_shifted = labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    lse = _f32(lse, T, "lse")
+    g = _f32(g, T, "g")
+    if gout is not None:
+        gout = gout.detach().reshape(-1)[:1].to(device=dev, dtype=torch.float32).contiguous()
+    dH = torch.empty_like(hidden) if need_dh else None
+    dW = torch.empty_like(weight) if need_dw else None
+    db = torch.empty(V, dtype=weight.dtype, device=dev) if (need_db and bias is not None) else None
+    if not (need_dh or need_dw or db is not None):
+        return dH, dW, db
+    ws = _ws(lib.fgrpo_lmhead_bwd_kept_workspace(T, H, V, code) if need_dh else 0, dev)
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_lmhead_bwd_kept(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted), _ptr(lse), _ptr(g),
+                                       _ptr(gout), 1.0 / float(temperature), T, H, V, code,
+                                       _ptr(kept), kept.numel(), _ptr(dH), _ptr(dW), _ptr(db),
+                                       _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "lmhead_bwd_kept")
     return dH, dW, db
 
 
@@ -466,18 +520,47 @@ def _valid_rows(labels_shifted: torch.Tensor, compact: bool):
     return mask.nonzero(as_tuple=False).squeeze(1)
 
 
-def _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx):
-    """Forward on the rows ``idx`` (or on all rows when idx is None); outputs scattered back into [T] vectors."""
-    if idx is None:
-        lp, ent, lse = lmhead_logprob_fwd(hidden, weight, bias, labels_shifted, temperature)
-        return lp, ent, lse, hidden, labels_shifted
-    T = hidden.shape[0]
-    h_c = hidden.index_select(0, idx)
-    y_c = labels_shifted.reshape(-1).index_select(0, idx)
-    lp_c, ent_c, lse_c = lmhead_logprob_fwd(h_c, weight, bias, y_c, temperature)
-    lp = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, lp_c)
-    ent = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, ent_c)
-    return lp, ent, lse_c, h_c, y_c
+# Keeping the logits for the backward (as the reference's autograd does) instead of recomputing them: "auto" keeps
+# them when the kernels support the shape and the buffer takes at most this share of the memory still obtainable
+# (free on the device + cached by torch's allocator); True insists (raises when unsupported); False recomputes.
+KEEP_LOGITS = "auto"
+KEEP_MAX_MEMORY_FRACTION = 0.5
+
+
+def _want_keep(T: int, H: int, V: int, dtype, dev, needs_grad: bool, keep_logits=None) -> bool:
+    mode = KEEP_LOGITS if keep_logits is None else keep_logits
+    if not needs_grad or mode is False or T == 0:
+        return False
+    ok = keep_supported(T, H, V, dtype)
+    if mode is True:
+        if not ok:
+            raise RuntimeError(f"fgrpo: keep_logits=True but T={T} H={H} V={V} {dtype} is not supported")
+        return True
+    if not ok:
+        return False
+    free, _total = torch.cuda.mem_get_info(dev)
+    obtainable = free + torch.cuda.memory_reserved(dev) - torch.cuda.memory_allocated(dev)
+    return logits_keep_bytes(T, V) <= KEEP_MAX_MEMORY_FRACTION * obtainable
+
+
+def _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx, needs_grad=False, keep_logits=None):
+    """Forward on the rows ``idx`` (or on all rows when idx is None); outputs scattered back into [T] vectors.
+    Returns (lp, ent, lse, hidden used, labels used, kept logits | None)."""
+    if idx is not None:
+        hidden = hidden.index_select(0, idx)
+        y = labels_shifted.reshape(-1).index_select(0, idx)
+    else:
+        y = labels_shifted
+    keep = _want_keep(hidden.shape[0], hidden.shape[1], weight.shape[0], weight.dtype, hidden.device, needs_grad,
+                      keep_logits)
+    res = lmhead_logprob_fwd(hidden, weight, bias, y, temperature, keep=keep)
+    lp, ent, lse = res[:3]
+    kept = res[3] if keep else None
+    if idx is not None:
+        T = labels_shifted.numel()
+        lp = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, lp)
+        ent = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, ent)
+    return lp, ent, lse, hidden, y, kept
 
 
 def panel_elems_bound(T: int, V: int, loss_chunksize: Optional[int]) -> int:
@@ -491,10 +574,15 @@ def panel_elems_bound(T: int, V: int, loss_chunksize: Optional[int]) -> int:
     return asked if asked > own else 0
 
 
-def _bwd_rows(h_used, weight, bias, y_used, lse, g_full, gout, temperature, need, panel_hint, idx, hidden_shape):
+def _bwd_rows(h_used, weight, bias, y_used, lse, g_full, gout, temperature, need, panel_hint, idx, hidden_shape,
+              kept=None):
     g_used = g_full if idx is None else g_full.reshape(-1).index_select(0, idx)
-    dH, dW, db = lmhead_bwd(h_used, weight, bias, y_used, lse, g_used, gout, temperature, need[0], need[1], need[2],
-                            panel_hint)
+    if kept is not None:
+        dH, dW, db = lmhead_bwd_kept(h_used, weight, bias, y_used, lse, g_used, gout, temperature, kept, need[0],
+                                     need[1], need[2])
+    else:
+        dH, dW, db = lmhead_bwd(h_used, weight, bias, y_used, lse, g_used, gout, temperature, need[0], need[1],
+                                need[2], panel_hint)
     if idx is not None and dH is not None:
         dH = torch.zeros(hidden_shape, dtype=dH.dtype, device=dH.device).index_copy_(0, idx, dH)
     return dH, dW, db
@@ -504,11 +592,14 @@ class _LMHeadLogprob(torch.autograd.Function):
     """(hidden, weight, bias, labels_shifted) -> (lp, entropy); entropy carries no gradient."""
 
     @staticmethod
-    def forward(ctx, hidden, weight, bias, labels_shifted, temperature, panel_hint, compact):
+    def forward(ctx, hidden, weight, bias, labels_shifted, temperature, panel_hint, compact, keep_logits=None):
         idx = _valid_rows(labels_shifted, compact)
-        lp, ent, lse, h_used, y_used = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx)
+        needs_grad = any(ctx.needs_input_grad[:3])
+        lp, ent, lse, h_used, y_used, kept = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx,
+                                                               needs_grad, keep_logits)
         ctx.save_for_backward(h_used, weight, bias if bias is not None else hidden.new_empty(0), y_used, lse,
                               idx if idx is not None else hidden.new_empty(0))
+        ctx.kept = kept       # consumed by the one backward (a second backward through this node recomputes)
         ctx.has_bias = bias is not None
         ctx.compacted = idx is not None
         ctx.hidden_shape = tuple(hidden.shape)
@@ -522,9 +613,10 @@ class _LMHeadLogprob(torch.autograd.Function):
         h_used, weight, bias, y_used, lse, idx = ctx.saved_tensors
         bias = bias if ctx.has_bias else None
         need = (ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.has_bias and ctx.needs_input_grad[2])
+        kept, ctx.kept = ctx.kept, None
         dH, dW, db = _bwd_rows(h_used, weight, bias, y_used, lse, g_lp, None, ctx.temperature, need, ctx.panel_hint,
-                               idx if ctx.compacted else None, ctx.hidden_shape)
-        return dH, dW, db, None, None, None, None
+                               idx if ctx.compacted else None, ctx.hidden_shape, kept)
+        return dH, dW, db, None, None, None, None, None
 
 
 class _FusedGRPOLoss(torch.autograd.Function):
@@ -533,9 +625,13 @@ class _FusedGRPOLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens, temperature,
-                clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode, denom_override, panel_hint, compact):
+                clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode, denom_override, panel_hint, compact,
+                keep_logits=None):
         idx = _valid_rows(labels_shifted, compact)
-        lp, ent, lse, h_used, y_used = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx)
+        needs_grad = any(ctx.needs_input_grad[:3])
+        lp, ent, lse, h_used, y_used, kept = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx,
+                                                               needs_grad, keep_logits)
+        ctx.kept = kept       # consumed by the one backward (a second backward through this node recomputes)
         loss, g, lr, c1, l1, l2, scal = grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
                                                       clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
                                                       denom_override)
@@ -554,9 +650,10 @@ class _FusedGRPOLoss(torch.autograd.Function):
         h_used, weight, bias, y_used, lse, g, idx = ctx.saved_tensors
         bias = bias if ctx.has_bias else None
         need = (ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.has_bias and ctx.needs_input_grad[2])
+        kept, ctx.kept = ctx.kept, None
         dH, dW, db = _bwd_rows(h_used, weight, bias, y_used, lse, g, g_loss, ctx.temperature, need, ctx.panel_hint,
-                               idx if ctx.compacted else None, ctx.hidden_shape)
-        return (dH, dW, db) + (None,) * 14
+                               idx if ctx.compacted else None, ctx.hidden_shape, kept)
+        return (dH, dW, db) + (None,) * 15
 
 
 class _GRPOLossFromLogprobs(torch.autograd.Function):
@@ -590,17 +687,20 @@ def grpo_loss_from_logprobs(lp, labels_shifted, old_lp, adv, ref_lp=None, cu_seq
 
 
 def lmhead_logprob(hidden, weight, bias, labels_shifted, temperature=1.0, panel_hint=0,
-                   compact=False) -> Tuple[torch.Tensor, torch.Tensor]:
-    return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint), bool(compact))
+                   compact=False, keep_logits=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint), bool(compact),
+                                keep_logits)
 
 
 def fused_grpo_loss(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp=None, cu_seqlens=None,
                     temperature=1.0, clip_low=0.2, clip_high=0.4, clip_ratio_c=1e32, kl_beta=0.0,
-                    loss_agg_mode="token_mean", denom_override=0.0, panel_hint=0, compact=False):
-    """(loss, entropy, log_ratio, clip1, unclipped, clipped, lp); only loss carries a gradient."""
+                    loss_agg_mode="token_mean", denom_override=0.0, panel_hint=0, compact=False, keep_logits=None):
+    """(loss, entropy, log_ratio, clip1, unclipped, clipped, lp); only loss carries a gradient.
+    ``keep_logits``: None = the module default (``KEEP_LOGITS``), True / False / "auto"."""
     return _FusedGRPOLoss.apply(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens,
                                 float(temperature), float(clip_low), float(clip_high), float(clip_ratio_c),
-                                float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint), bool(compact))
+                                float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint), bool(compact),
+                                keep_logits)
 
 
 # --------------------------------------------------------------------------- packed variable-length attention

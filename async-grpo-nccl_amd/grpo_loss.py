@@ -210,7 +210,8 @@ def fused_log_probs_and_entropy_fn(
                                                    per_token_fn, None)
     shifted = ops.shift_labels(labels).reshape(-1)
     lp, ent = ops.lmhead_logprob(hs, w, b, shifted, temperature,
-                                 compact=bool(unused_kwargs.get("compact_masked_tokens", False)))
+                                 compact=bool(unused_kwargs.get("compact_masked_tokens", False)),
+                                 keep_logits=unused_kwargs.get("keep_logits", None))
     return lp, ent
 
 
@@ -243,7 +244,11 @@ def grpo_loss_and_entropy_ce_fn(
     grpo_loss.py:256-348).  ``loss_chunksize`` only widens the transient of the
     backward (one dLogits panel, bf16) beyond the library's own bound of a
     quarter of ``[T, V]``, at most 2 GiB, when ``loss_chunksize * V`` elements
-    are more than that; the result does not depend on it."""
+    are more than that; the result does not depend on it.  Where the kernels
+    support the shape and memory allows, the bf16 logits are kept for the
+    backward as the reference's autograd keeps them (``keep_logits=False``
+    among the keyword arguments forces the recomputing backward, ``True``
+    insists on keeping)."""
     if advantages is None:
         raise ValueError("grpo_loss_and_entropy_ce_fn: advantages are required")
     ref_logprobs = unused_kwargs.get("ref_logprobs", None)
@@ -272,7 +277,7 @@ def grpo_loss_and_entropy_ce_fn(
         advantages.reshape(-1),
         None if ref_logprobs is None else ref_logprobs.reshape(-1),
         cu_seqlens, temperature, clip_low, clip_high, clip_ratio_c, kl_beta,
-        loss_agg_mode, denom, hint, compact)
+        loss_agg_mode, denom, hint, compact, unused_kwargs.get("keep_logits", None))
     return loss, ent, lr, c1, l1, l2
 
 
@@ -320,7 +325,7 @@ def make_grpo_forward(model, temperature: float = 1.0, mode: str = 'training', u
         return_dict = return_dict if return_dict is not None else cfg.use_return_dict
         # objective extensions travel in kwargs but are not for the transformer body
         extra = {k: kwargs.pop(k) for k in ("ref_logprobs", "kl_beta", "loss_agg_mode", "cu_seqlens", "num_samples_total",
-                                            "compact_masked_tokens")
+                                            "compact_masked_tokens", "keep_logits")
                  if k in kwargs}
         body_out = model.model(
             input_ids=input_ids,
@@ -371,7 +376,7 @@ def make_grpo_forward(model, temperature: float = 1.0, mode: str = 'training', u
                 hidden_states=hidden_states,
                 labels=labels,
                 temperature=temperature,
-                **{k: v for k, v in extra.items() if k == "compact_masked_tokens"},
+                **{k: v for k, v in extra.items() if k in ("compact_masked_tokens", "keep_logits")},
             )
             return LogProbsOutput(loss=out[0], entropy=out[1])
         else:

@@ -99,6 +99,39 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
                      long long panel_elems_hint,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- the same forward / backward pair WITHOUT recomputation: the logits are kept --------------------------
+ * The reference keeps every chunk's logits alive for autograd (grpo_loss.py:286-313: 9.96 GB of bf16 at T = 32768,
+ * V = 151936) and its backward reads them back; fgrpo_lmhead_bwd instead recomputes them (a fourth [T x V x H]
+ * product).  Where memory allows - 288 GB of HBM per MI355X - this pair does what the reference does:
+ * fgrpo_logprob_fwd_keep is fgrpo_logprob_fwd that also writes x = W h + b (before the temperature, rounded to
+ * bf16 exactly as the reference's bf16 logits are) into `logits_keep`, and fgrpo_lmhead_bwd_kept turns that buffer
+ * IN PLACE into dLogits (one HBM-bound pass) and runs each gradient product as one launch over the whole
+ * vocabulary: 6 instead of 8 T*H*V products per step, dH written once.  The workspace (T*H*4 bytes) is only
+ * touched when the tuning key keep_panels splits the products into vocabulary panels (fp32 dH accumulator);
+ * NULL is accepted otherwise.  lp / entropy / lse are computed from the fp32 accumulators and are bit-identical
+ * to fgrpo_logprob_fwd's.
+ * logits_keep: fgrpo_logits_keep_bytes(T, V) bytes, 16-byte aligned, laid out in 256-column blocks
+ * [ceil(V/256)][round_up(T,256)][256] bf16; its contents after fgrpo_lmhead_bwd_kept are dLogits (not an output).
+ * Supported (fgrpo_keep_supported() != 0): bf16, H a multiple of 256, enough tiles to fill the device; anything
+ * else returns FGRPO_ERR_UNSUPPORTED - use the recomputing pair.  dH_out / dW_out / dbias_out as in
+ * fgrpo_lmhead_bwd. */
+int fgrpo_keep_supported(int T, int H, int V, int dtype);
+size_t fgrpo_logits_keep_bytes(int T, int V);
+int fgrpo_logprob_fwd_keep(const void* hidden, const void* weight, const void* bias,
+                           const int64_t* labels_shifted, float inv_temperature,
+                           int T, int H, int V, int dtype,
+                           float* lp_out, float* ent_out, float* lse_out,
+                           void* logits_keep, size_t logits_keep_bytes,
+                           void* workspace, size_t workspace_bytes, void* stream);
+size_t fgrpo_lmhead_bwd_kept_workspace(int T, int H, int V, int dtype);
+int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bias,
+                          const int64_t* labels_shifted, const float* lse, const float* g,
+                          const float* gout_dev, float inv_temperature,
+                          int T, int H, int V, int dtype,
+                          void* logits_keep, size_t logits_keep_bytes,
+                          void* dH_out, void* dW_out, void* dbias_out,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- per-token GRPO objective -------------------------------------------------
  * Replaces the tail of grpo_loss_and_entropy_ce_fn (grpo_loss.py:318-348):
  * ratio, dual clip, masked mean.  old_lp NULL => ratio 1 (grpo_loss.py:318-319).

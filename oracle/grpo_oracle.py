@@ -122,6 +122,40 @@ def grpo_token_terms(lp, old, adv, clip_low, clip_high, clip_ratio_c):
     return log_ratio, ratio, unclipped, clipped, clip1, tok
 
 
+def grpo_objective_from_logprobs(lp, shifted_labels, old_logprobs, advantages, clip_low, clip_high, clip_ratio_c,
+                                 ref_logprobs=None, kl_beta=0.0, loss_agg_mode="token_mean", cu_seqlens=None,
+                                 num_samples_total=None):
+    """The tail of the objective on per-token vectors [T] (reference: grpo_loss.py:318-348): ratio, dual clip,
+    masked mean; plus the two extensions described in ``grpo_loss_and_entropy``.  ``lp`` may require grad.
+    Returns (loss, log_ratio, clip1, unclipped, clipped) - the last four attached to ``lp``'s graph."""
+    if old_logprobs is None:
+        old_logprobs = lp.detach()
+    old = old_logprobs.reshape(-1).to(lp.dtype)
+    adv = advantages.reshape(-1).to(lp.dtype)
+    log_ratio, ratio, unclipped, clipped, clip1, tok = grpo_token_terms(
+        lp, old, adv, clip_low, clip_high, clip_ratio_c)
+    if ref_logprobs is not None and kl_beta != 0.0:
+        d = ref_logprobs.reshape(-1).to(lp.dtype) - lp
+        tok = tok + kl_beta * (torch.exp(d) - d - 1.0)
+    mask = shifted_labels.reshape(-1) != IGNORE_INDEX
+    vec = torch.where(mask, tok, torch.zeros_like(tok))
+    if loss_agg_mode == "token_mean":
+        denom = mask.sum().clamp(min=1).to(vec.dtype)
+        loss = vec.sum() / denom
+    elif loss_agg_mode == "sample_mean":
+        assert cu_seqlens is not None
+        seg = segment_ids_from_cu_seqlens(cu_seqlens, vec.numel())
+        n = int(seg.max()) + 1 if seg.numel() else 0
+        cnt = torch.zeros(n, dtype=vec.dtype).index_add_(0, seg, mask.to(vec.dtype))
+        sums = torch.zeros(n, dtype=vec.dtype).index_add_(0, seg, vec)
+        per = sums / cnt.clamp(min=1)
+        N = num_samples_total if num_samples_total is not None else int((cnt > 0).sum())
+        loss = per.sum() / max(N, 1)
+    else:
+        raise ValueError(loss_agg_mode)
+    return loss, log_ratio, clip1, unclipped, clipped
+
+
 def grpo_loss_and_entropy(lm_head_weights, lm_head_bias, hidden_states, labels,
                           temperature: float = 1.0,
                           old_logprobs: Optional[torch.Tensor] = None,
@@ -163,31 +197,9 @@ def grpo_loss_and_entropy(lm_head_weights, lm_head_bias, hidden_states, labels,
     else:
         lp, entropy = fused_log_probs_and_entropy(lm_head_weights, lm_head_bias, hidden_states,
                                                   labels, temperature)
-    if old_logprobs is None:
-        old_logprobs = lp.detach()
-    old = old_logprobs.reshape(-1).to(lp.dtype)
-    adv = advantages.reshape(-1).to(lp.dtype)
-    log_ratio, ratio, unclipped, clipped, clip1, tok = grpo_token_terms(
-        lp, old, adv, clip_low, clip_high, clip_ratio_c)
-    if ref_logprobs is not None and kl_beta != 0.0:
-        d = ref_logprobs.reshape(-1).to(lp.dtype) - lp
-        tok = tok + kl_beta * (torch.exp(d) - d - 1.0)
-    mask = shift_labels(labels).reshape(-1) != IGNORE_INDEX
-    vec = torch.where(mask, tok, torch.zeros_like(tok))
-    if loss_agg_mode == "token_mean":
-        denom = mask.sum().clamp(min=1).to(vec.dtype)
-        loss = vec.sum() / denom
-    elif loss_agg_mode == "sample_mean":
-        assert cu_seqlens is not None
-        seg = segment_ids_from_cu_seqlens(cu_seqlens, vec.numel())
-        n = int(seg.max()) + 1 if seg.numel() else 0
-        cnt = torch.zeros(n, dtype=vec.dtype).index_add_(0, seg, mask.to(vec.dtype))
-        sums = torch.zeros(n, dtype=vec.dtype).index_add_(0, seg, vec)
-        per = sums / cnt.clamp(min=1)
-        N = num_samples_total if num_samples_total is not None else int((cnt > 0).sum())
-        loss = per.sum() / max(N, 1)
-    else:
-        raise ValueError(loss_agg_mode)
+    loss, log_ratio, clip1, unclipped, clipped = grpo_objective_from_logprobs(
+        lp, shift_labels(labels).reshape(-1), old_logprobs, advantages, clip_low, clip_high, clip_ratio_c,
+        ref_logprobs, kl_beta, loss_agg_mode, cu_seqlens, num_samples_total)
     return loss, entropy, log_ratio.detach(), clip1.detach(), unclipped.detach(), clipped.detach()
 
 

@@ -1,0 +1,210 @@
+"""The forward/backward pair that keeps the bf16 logits (as the reference's autograd does, grpo_loss.py:286-313)
+instead of recomputing them, and the whole path at the full benchmark sizes through the drop-in's own entry point.
+
+Small device-filling shapes are compared with the CPU oracle outright.  At the full sizes the oracle cannot form
+[T x V] in seconds: the per-token logprobs (pinned against sampled oracle rows in test_gpu_parity) feed the oracle's
+objective on [T] vectors, whose autograd gives the per-token gradient that sampled rows of dH and dW must show."""
+import math
+
+import pytest
+import torch
+
+from oracle import grpo_oracle as O
+from test_gpu_parity import COS_MIN, LOSS_REL, LP_TOL_BF16, check, cos, group_adv, run_case
+
+pytestmark = pytest.mark.gpu
+
+
+def filling_workload(seed, **over):
+    """A shape the kept-logits kernels accept (H % 256 == 0, at least half the device's tiles in both gradient
+    products) that the oracle still finishes in seconds."""
+    from fgrpo.synthetic import make_workload
+    cfg = dict(H=1024, V=8492, tokens=8155, len_lo=40, len_hi=700, h_scale=1.0, w_std=0.05, prompts=4, group=8)
+    cfg.update(over)
+    return make_workload("cfg1", seed=seed, overrides=cfg)
+
+
+@pytest.mark.parametrize("mode", ["reference", "north_star"])
+def test_kept_logits_against_oracle(dev, mode):
+    from fgrpo import ops
+    w = filling_workload(11)
+    assert ops.keep_supported(w.T, w.H, w.V, torch.bfloat16)
+    want, got, o, g, _, _ = run_case(w, dev, mode, keep_logits=True)
+    check(want, got, o, g, f32=False)
+
+
+def test_kept_logits_with_bias_and_temperature(dev):
+    w = filling_workload(12)
+    bias = (torch.randn(w.V, generator=torch.Generator().manual_seed(9)) * 0.3).to(w.dtype)
+    want, got, o, g, _, _ = run_case(w, dev, "north_star", temperature=0.7, bias=bias, keep_logits=True)
+    check(want, got, o, g, f32=False)
+
+
+def test_kept_forward_is_bit_identical_and_backward_close_to_recompute(dev):
+    """Keeping the logits changes nothing in the forward (statistics come from the fp32 accumulators either way);
+    the backward differs from the recomputing one only by the bf16 rounding of the kept logits."""
+    from fgrpo import ops
+    w = filling_workload(13, tokens=8192 + 64)           # token count past a multiple of 256
+    hs, W = w.hidden.reshape(w.T, w.H).to(dev), w.weight.to(dev)
+    y = ops.shift_labels(w.labels.to(dev)).reshape(-1)
+    a = ops.lmhead_logprob_fwd(hs, W, None, y, 0.9)
+    b = ops.lmhead_logprob_fwd(hs, W, None, y, 0.9, keep=True)
+    for x, z in zip(a, b[:3]):
+        assert torch.equal(x, z)
+    g = torch.randn(w.T, generator=torch.Generator().manual_seed(2)).to(dev) / w.T
+    g[::5] = 0
+    gout = torch.tensor([2.5], device=dev)
+    dH0, dW0, _ = ops.lmhead_bwd(hs, W, None, y, a[2], g, gout, 0.9, True, True, False, 0)
+    dH1, dW1, _ = ops.lmhead_bwd_kept(hs, W, None, y, a[2], g, gout, 0.9, b[3], True, True, False)
+    assert cos(dH0, dH1) >= 0.99999 and cos(dW0, dW1) >= 0.99999
+    dead = (g == 0) | (y == -100)
+    assert (dH1[dead] == 0).all()                                      # rows without gradient are exact zeros
+    # two runs on the same kept logits are bit-identical (no atomics anywhere)
+    b2 = ops.lmhead_logprob_fwd(hs, W, None, y, 0.9, keep=True)
+    dH2, dW2, _ = ops.lmhead_bwd_kept(hs, W, None, y, a[2], g, gout, 0.9, b2[3], True, True, False)
+    assert torch.equal(dH1, dH2) and torch.equal(dW1, dW2)
+
+
+def test_kept_logits_panel_split_matches_single_launch(dev):
+    """The tuning key keep_panels splits the gradient products into vocabulary panels with an fp32 dH accumulator:
+    dW is bit-identical (each row block is still written once), dH agrees to bf16 rounding."""
+    from fgrpo import _lib, ops
+    w = filling_workload(14)
+    hs, W = w.hidden.reshape(w.T, w.H).to(dev), w.weight.to(dev)
+    y = ops.shift_labels(w.labels.to(dev)).reshape(-1)
+    g = torch.randn(w.T, generator=torch.Generator().manual_seed(3)).to(dev) / w.T
+    lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
+    dH1, dW1, _ = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
+    kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)[3]
+    _lib.set_tuning(keep_panels=3)
+    try:
+        dH3, dW3, _ = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
+    finally:
+        _lib.set_tuning(keep_panels=0)
+    assert torch.equal(dW1, dW3)
+    assert cos(dH1, dH3) >= 0.99999
+
+
+def test_keep_refuses_what_it_cannot_do(dev):
+    from fgrpo import ops
+    hs = torch.randn(512, 192, device=dev).bfloat16()
+    W = torch.randn(4096, 192, device=dev).bfloat16()
+    y = torch.randint(0, 4096, (512,), device=dev)
+    assert not ops.keep_supported(512, 192, 4096, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="kept-logits"):
+        ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
+    with pytest.raises(RuntimeError, match="keep_logits=True"):
+        ops.fused_grpo_loss(hs.requires_grad_(True), W, None, y, None, torch.randn(512, device=dev), keep_logits=True)
+    # "auto" quietly recomputes for such a shape
+    out = ops.fused_grpo_loss(hs, W, None, y, None, torch.randn(512, device=dev), keep_logits="auto")
+    out[0].backward()
+    assert hs.grad is not None and torch.isfinite(hs.grad.float()).all()
+
+
+# ------------------------------------------------------------------ full benchmark sizes through the drop-in
+@pytest.mark.parametrize("name,keep", [("cfg1", True), ("cfg1", False), ("cfg2", True), ("cfg2", False),
+                                       ("cfg4", True), ("cfg4", False)])
+def test_full_size_through_the_drop_in(dev, name, keep):
+    """grpo_loss_and_entropy_ce_fn exactly as bench.py calls it (KL to the reference policy, mean over samples of
+    per-sample token means, cu_seqlens, the configuration's chunk hint), then backward with a non-unit upstream
+    scale.  Checked: loss and the four per-token diagnostics against the oracle's objective evaluated on the
+    kernel's per-token logprobs; sampled rows of dH and of dW against the closed form with the oracle's per-token
+    gradient; columns of dW summing to zero."""
+    import grpo_loss as G
+    from fgrpo import ops
+    from fgrpo.synthetic import make_workload
+    w = make_workload(name, seed=0, device=dev)
+    p = w.params
+    T, H, V = w.T, w.H, w.V
+    assert ops.keep_supported(T, H, V, torch.bfloat16)
+    shifted = ops.shift_labels(w.labels).reshape(-1)
+    hs2 = w.hidden.reshape(T, H)
+    adv = group_adv(w, p["adv_eps"]).to(dev)
+    lp0, _, lse = ops.lmhead_logprob_fwd(hs2, w.weight, None, shifted)
+    old, ref = lp0 + w.noise_old, lp0 + w.noise_ref
+
+    hidden = w.hidden.clone().requires_grad_(True)
+    weight = w.weight.clone().requires_grad_(True)
+    out = G.grpo_loss_and_entropy_ce_fn(weight, None, hidden, w.labels, 1.0, old, adv, p["clip_low"], p["clip_high"],
+                                        p["clip_ratio_c"], loss_chunksize=p["chunk"], ref_logprobs=ref,
+                                        kl_beta=p["kl_beta"], loss_agg_mode="sample_mean", cu_seqlens=w.cu_seqlens,
+                                        keep_logits=keep)
+    scale = 3.7
+    (out[0] * scale).backward()
+    torch.cuda.synchronize()
+
+    # the oracle's objective on the kernel's logprobs, on the CPU in fp64
+    lp_c = lp0.double().cpu().requires_grad_(True)
+    want = O.grpo_objective_from_logprobs(lp_c, shifted.cpu(), old.double().cpu(), adv.double().cpu(), p["clip_low"],
+                                          p["clip_high"], p["clip_ratio_c"], ref.double().cpu(), p["kl_beta"],
+                                          "sample_mean", w.cu_seqlens.cpu())
+    (want[0] * scale).backward()
+    assert abs(out[0].item() - want[0].item()) <= LOSS_REL * abs(want[0].item()) + 1e-7
+    for k_got, k_want in ((2, 1), (3, 2), (4, 3), (5, 4)):          # log_ratio, clip1, unclipped, clipped
+        assert (out[k_got].double().cpu() - want[k_want].detach()).abs().max().item() <= 10 * LP_TOL_BF16
+    g = lp_c.grad.float().to(dev)                                    # d (scale * loss) / d lp_t
+
+    gsel = torch.Generator().manual_seed(5)
+    rows = torch.randperm(T, generator=gsel)[:128].to(dev)
+    x = hs2[rows].float() @ w.weight.float().t()
+    prob = torch.softmax(x, -1)
+    safe = shifted[rows].clamp(min=0)
+    want_dH = g[rows, None] * (w.weight.float()[safe] - prob @ w.weight.float())
+    assert cos(hidden.grad.reshape(T, H)[rows], want_dH) >= COS_MIN
+    vs = torch.randperm(V, generator=gsel)[:16].to(dev)
+    xv = hs2.float() @ w.weight[vs].float().t()
+    coef = g[:, None] * ((shifted[:, None] == vs[None, :]).float() - torch.exp(xv - lse[:, None]))
+    want_dW = coef.t() @ hs2.float()
+    assert cos(weight.grad[vs], want_dW) >= COS_MIN
+    col = weight.grad.float().sum(0)
+    assert col.abs().max().item() <= 1e-2 * weight.grad.float().abs().sum(0).max().item()
+
+
+def test_cfg3_through_the_logprob_harness(dev):
+    """The forward-only configuration (T = 131072, H = 5120) through LogProbHarness on a model whose body is an
+    embedding: per-sample lists equal the kernel's flat vectors, sampled rows equal the oracle."""
+    from types import SimpleNamespace
+    import grpo_loss as G
+    import workers
+    from fgrpo import ops
+    from fgrpo.synthetic import make_workload
+    w = make_workload("cfg3", seed=0, device=dev)
+    T, H, V = w.T, w.H, w.V
+
+    class Body(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.table = w.hidden.reshape(T, H)
+
+        def forward(self, input_ids=None, position_ids=None, **kw):
+            # hidden state of packed position t is row t of the workload's hidden matrix
+            n = input_ids.shape[1]
+            return (self.table[:n].reshape(1, n, H),)
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.model = Body()
+            self.lm_head = torch.nn.Linear(H, V, bias=False, device="meta")
+            self.lm_head.weight = torch.nn.Parameter(w.weight, requires_grad=False)
+            self.config = SimpleNamespace(output_attentions=False, output_hidden_states=False, use_return_dict=True)
+
+        def forward(self, *a, **kw):
+            raise AssertionError("the patched forward must be used")
+
+    model = G.make_grpo_forward(Model(), temperature=1.0, mode="eval")
+    harness = workers.LogProbHarness(model, dev)
+    ids, labels = w.input_ids.reshape(-1).cpu(), w.labels.reshape(-1).cpu()
+    cu = w.cu_seqlens.cpu().tolist()
+    samples = [dict(sample_ids=ids[a:b].tolist(), labels=labels[a:b].tolist()) for a, b in zip(cu[:-1], cu[1:])]
+    got = harness.compute_log_probs_from_samples(samples)
+    shifted = ops.shift_labels(w.labels).reshape(-1)
+    lp, ent, _ = ops.lmhead_logprob_fwd(w.hidden.reshape(T, H), w.weight, None, shifted)
+    flat_lp = torch.tensor([v for s in got for v in s["logprobs"]])
+    flat_ent = torch.tensor([v for s in got for v in s["entropies"]])
+    assert torch.equal(flat_lp, lp.cpu()) and torch.equal(flat_ent, ent.cpu())
+    rows = torch.randperm(T, generator=torch.Generator().manual_seed(6))[:96].to(dev)
+    x_c = (w.hidden.reshape(T, H)[rows].float() @ w.weight.float().t()).cpu()
+    want_lp = O.logprobs_from_logits(x_c, shifted[rows].cpu())
+    assert (lp[rows].cpu() - want_lp).abs().max() <= LP_TOL_BF16
+    assert (lp <= 1e-6).all() and (ent <= math.log(V) + 1e-3).all()

@@ -35,8 +35,9 @@ def group_adv(w, eps):
     return torch.from_numpy(O.broadcast_values(adv, w.sample_lens)).float()
 
 
-def run_case(w, dev, mode, temperature=1.0, bias=None, chunk=None):
-    """mode 'reference': token-mean, no KL; 'north_star': sample-mean + KL penalty."""
+def run_case(w, dev, mode, temperature=1.0, bias=None, chunk=None, **extra):
+    """mode 'reference': token-mean, no KL; 'north_star': sample-mean + KL penalty.  ``extra`` goes to the drop-in
+    only (keyword arguments the oracle has no use for, such as keep_logits)."""
     import grpo_loss as G
     p = w.params
     hs_c, W_c = oracle_inputs(w)
@@ -61,7 +62,8 @@ def run_case(w, dev, mode, temperature=1.0, bias=None, chunk=None):
     b_g = None if bias is None else bias.to(dev).clone().requires_grad_(True)
     gkw = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in kw.items()}
     got = G.grpo_loss_and_entropy_ce_fn(W_g, b_g, hs_g, w.labels.to(dev), temperature, old.to(dev), adv.to(dev),
-                                        p["clip_low"], p["clip_high"], p["clip_ratio_c"], loss_chunksize=chunk, **gkw)
+                                        p["clip_low"], p["clip_high"], p["clip_ratio_c"], loss_chunksize=chunk, **gkw,
+                                        **extra)
     got[0].backward()
     torch.cuda.synchronize()
     return want, got, (hs_o, W_o, b_o), (hs_g, W_g, b_g), lp0, old
@@ -433,7 +435,7 @@ def test_full_size_properties_and_sampled_rows(dev, name):
         return
     g = torch.randn(T, generator=torch.Generator().manual_seed(2)).to(dev) / T
     g = g * mask
-    hint = (w.params["chunk"] or 0) * V            # what the drop-in passes for loss_chunksize
+    hint = ops.panel_elems_bound(T, V, w.params["chunk"])       # what the drop-in passes for loss_chunksize
     dH, dW, _ = ops.lmhead_bwd(hs, w.weight, None, shifted, lse, g, None, 1.0, True, True, False, hint)
     dH2, dW2, _ = ops.lmhead_bwd(hs, w.weight, None, shifted, lse, g, None, 1.0, True, True, False, hint)
     assert torch.equal(dH, dH2) and torch.equal(dW, dW2)
