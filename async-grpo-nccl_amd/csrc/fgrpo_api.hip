@@ -54,6 +54,40 @@ int num_cus() {
 
 namespace {
 
+// Optional per-phase event brackets of the backward (fgrpo_phase_timing_begin / _end).  One timer per process:
+// the backward usually runs on another thread (autograd's) than the one that asked for the timing.
+struct PhaseTimer {
+  bool on = false, created = false;
+  int n = 0, dropped = 0;
+  hipEvent_t ev[2 * FGRPO_MAX_TIMED_PHASES];
+  int kind[FGRPO_MAX_TIMED_PHASES];
+};
+PhaseTimer g_phase;
+std::mutex g_phase_mu;
+
+struct PhaseScope {
+  hipStream_t st;
+  int slot = -1;
+  PhaseScope(int kind, hipStream_t s) : st(s) {
+    PhaseTimer& t = g_phase;
+    if (!t.on) return;                            // unlocked peek: timing is off in every production call
+    std::lock_guard<std::mutex> lock(g_phase_mu);
+    if (!t.on) return;
+    if (t.n >= FGRPO_MAX_TIMED_PHASES) {
+      ++t.dropped;
+      return;
+    }
+    slot = t.n++;
+    t.kind[slot] = kind;
+    (void)hipEventRecord(t.ev[2 * slot], st);
+  }
+  ~PhaseScope() {
+    if (slot >= 0) (void)hipEventRecord(g_phase.ev[2 * slot + 1], st);
+  }
+};
+enum { kPhaseDlogits = 0, kPhaseDh = 1, kPhaseDw = 2, kPhaseOther = 3 };
+
+
 int* tuning_slot(const char* key) {
   if (!key) return nullptr;
   if (!strcmp(key, "fwd_variant")) return &g_tune.fwd_variant;
@@ -607,7 +641,10 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
                 : tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
     const int kv = d.tiles_v * pl.bm;        // written panel width
     const int kt = pl.tiles_t * pl.bn;       // written token extent
-    rc = launch_ds_variant(pl.variant, f32 != 0, d, st);
+    {
+      PhaseScope ph(kPhaseDlogits, st);
+      rc = launch_ds_variant(pl.variant, f32 != 0, d, st);
+    }
     if (rc) return rc;
 
     if (want_dh) {  // dH[T x H] (+)= dS_tv[T x kv] * W^T[H x kv]^T
@@ -647,7 +684,10 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
         else
           s.c_out_f32 = pl.dh_acc;
       }
-      rc = pl.kmajor_dh ? run_store_gemm_kmajor(tn, s, false, true, st) : run_store_gemm(tn, s, tn.gemm_variant, st);
+      {
+        PhaseScope ph(kPhaseDh, st);
+        rc = pl.kmajor_dh ? run_store_gemm_kmajor(tn, s, false, true, st) : run_store_gemm(tn, s, tn.gemm_variant, st);
+      }
       if (rc) return rc;
     }
     if (want_dw) {  // dW[v0 : v0+rows, H] = dS_vt[rows x kt] * hidden^T[H x kt]^T
@@ -679,7 +719,10 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias, c
         s.c_out_f32 = (float*)dW_out + (size_t)v0 * H;
       else
         s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
-      rc = pl.kmajor ? run_store_gemm_kmajor(tn, s, true, true, st) : run_store_gemm(tn, s, tn.gemm_variant, st);
+      {
+        PhaseScope ph(kPhaseDw, st);
+        rc = pl.kmajor ? run_store_gemm_kmajor(tn, s, true, true, st) : run_store_gemm(tn, s, tn.gemm_variant, st);
+      }
       if (rc) return rc;
     }
     if (dbias_out) {
@@ -767,7 +810,10 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
   }
 
   KeptParams k{ds, blk, Tpad, T, V, (const long long*)labels, lse, g, gout_dev, inv_temp};
-  hipLaunchKernelGGL(kept_logits_to_dlogits_kernel, dim3((unsigned)((Vpad / 256) * (Tpad / kKeptRows))), dim3(256), 0, st, k);
+  {
+    PhaseScope ph(kPhaseDlogits, st);
+    hipLaunchKernelGGL(kept_logits_to_dlogits_kernel, dim3((unsigned)((Vpad / 256) * (Tpad / kKeptRows))), dim3(256), 0, st, k);
+  }
   HIP_TRY(hipGetLastError());
 
   int rc = 0;
@@ -795,7 +841,10 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
         s.c_out_bf16 = (bf16_t*)dH_out;
       else
         s.c_out_f32 = dh_acc;
-      rc = run_store_gemm_kmajor(tn, s, false, true, st);
+      {
+        PhaseScope ph(kPhaseDh, st);
+        rc = run_store_gemm_kmajor(tn, s, false, true, st);
+      }
       if (rc) return rc;
     }
     if (dW_out) {   // dW[v0 : v0+rows, H] = dS^T[rows x Tpad] hidden[Tpad x H]: the token is the contraction row of both
@@ -812,7 +861,10 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       s.ldc = H;
       s.alpha = 1.f;
       s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
-      rc = run_store_gemm_kmajor(tn, s, true, true, st);
+      {
+        PhaseScope ph(kPhaseDw, st);
+        rc = run_store_gemm_kmajor(tn, s, true, true, st);
+      }
       if (rc) return rc;
     }
   }
@@ -822,6 +874,36 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
     HIP_TRY(hipGetLastError());
   }
   return 0;
+}
+
+int fgrpo_phase_timing_begin(void) {
+  std::lock_guard<std::mutex> lock(g_phase_mu);
+  PhaseTimer& t = g_phase;
+  if (!t.created) {
+    for (int i = 0; i < 2 * FGRPO_MAX_TIMED_PHASES; ++i) HIP_TRY(hipEventCreate(&t.ev[i]));
+    t.created = true;
+  }
+  t.n = t.dropped = 0;
+  t.on = true;
+  return 0;
+}
+
+int fgrpo_phase_timing_end(float* ms_by_phase, int* brackets_by_phase) {
+  std::lock_guard<std::mutex> lock(g_phase_mu);
+  PhaseTimer& t = g_phase;
+  if (!t.on) return fail(FGRPO_ERR_BAD_ARG, "phase_timing_end without phase_timing_begin");
+  t.on = false;
+  if (!ms_by_phase || !brackets_by_phase) return fail(FGRPO_ERR_BAD_ARG, "phase_timing_end: null argument");
+  for (int k = 0; k < FGRPO_NUM_PHASES; ++k) ms_by_phase[k] = 0.f, brackets_by_phase[k] = 0;
+  if (t.n > 0) HIP_TRY(hipEventSynchronize(t.ev[2 * (t.n - 1) + 1]));
+  for (int i = 0; i < t.n; ++i) {
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, t.ev[2 * i], t.ev[2 * i + 1]));
+    const int k = (t.kind[i] >= 0 && t.kind[i] < FGRPO_NUM_PHASES) ? t.kind[i] : FGRPO_NUM_PHASES - 1;
+    ms_by_phase[k] += ms;
+    ++brackets_by_phase[k];
+  }
+  return t.dropped;
 }
 
 size_t fgrpo_loss_fwd_workspace(int T, int nseq) {

@@ -149,6 +149,23 @@ def lmhead_logprob_fwd(hidden: torch.Tensor, weight: torch.Tensor, bias: Optiona
     return (lp, ent, lse, kept) if keep else (lp, ent, lse)
 
 
+def phase_timing_begin() -> None:
+    """Start bracketing the launches of this thread's backward calls with HIP events (diagnostics)."""
+    _lib.check(_lib.load().fgrpo_phase_timing_begin(), "phase_timing_begin")
+
+
+def phase_timing_end():
+    """Stop and read: ({phase: summed ms}, {phase: brackets}, dropped) for the phases dlogits / dh / dw / other."""
+    import ctypes
+    ms = (ctypes.c_float * _lib.NUM_PHASES)()
+    cnt = (ctypes.c_int * _lib.NUM_PHASES)()
+    rc = _lib.load().fgrpo_phase_timing_end(ctypes.cast(ms, ctypes.c_void_p), ctypes.cast(cnt, ctypes.c_void_p))
+    if rc < 0:
+        _lib.check(rc, "phase_timing_end")
+    names = ("dlogits", "dh", "dw", "other")
+    return {n: float(ms[i]) for i, n in enumerate(names)}, {n: int(cnt[i]) for i, n in enumerate(names)}, int(rc)
+
+
 def lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torch.Tensor],
                temperature: float, need_dh: bool, need_dw: bool, need_db: bool,
                panel_elems_hint: int = 0):

@@ -18,20 +18,22 @@ for p in (os.path.join(ROOT, "async-grpo-nccl_amd"), ROOT):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published (256 CUs x 4 SIMDs x 1024 flop/cycle at 2.4 GHz)
+PEAK_CLOCK_MHZ = 2400.0
 
-# Bytes per launch of the forward kernel that leave the L2s, from two rocprofv3 --pmc runs of this file
-# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 1 GiB
-# device copy of --copy-probe: FETCH_SIZE reads 524317.4 KiB for 2^20 KiB (factor 2.0000), WRITE_SIZE reads
-# 1048576 KiB (factor 1.0).  cfg1, launches of the timed steps: 10995346 KiB x 2.0 + 3046 KiB x 1.0.
-# None for workloads not measured.
-MEASURED_TRAFFIC_BYTES = {"cfg1": 10995346 * 1024 * (1048576 / 524317.4) + 3046 * 1024}
+# HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 1 GiB device copy of
+# --copy-probe.  Not measured in the run that prints it: the figure belongs to the binary and workload named in the
+# profile summary it cites, and is None for workloads that were not profiled.
+PROFILED_TRAFFIC = {
+    # workload: (bytes per launch, summary under profiles/)
+}
 
 
 def cpu_baseline(name: str, cfg_chunk, seed: int):
     """The oracle (a port of the reference's eager path) on the host cores, on a
     bounded slice: one chunk of tokens at the full H and V, forward + backward,
-    bf16-rounded inputs with fp32 math.  Work is linear in tokens."""
+    bf16-rounded inputs with fp32 math, one warm-up then the median of three runs.  Work is linear in tokens."""
     import torch
     from oracle import grpo_oracle as O
     from fgrpo.synthetic import CONFIGS
@@ -58,15 +60,105 @@ def cpu_baseline(name: str, cfg_chunk, seed: int):
         return time.perf_counter() - t0
 
     probe = 128
-    t_probe = run(probe)
-    # aim at ~15 s of CPU work, at most the configuration's own chunk size
-    n = int(max(probe, min(cfg_chunk or 4096, probe * 15.0 / max(t_probe, 1e-3))))
+    t_probe = run(probe)            # also the warm-up
+    # aim at ~5 s per run (three timed runs), at most the configuration's own chunk size
+    n = int(max(probe, min(cfg_chunk or 4096, probe * 5.0 / max(t_probe, 1e-3))))
     n = max(probe, (n // 128) * 128)
-    times = [run(n) for _ in range(2)]
-    t = min(times)
+    times = sorted(run(n) for _ in range(3))
+    t = times[1]
     return {"value": n / t, "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"{n} tokens (one chunk) at full H={H}, V={V}, fwd{'' if cfg['forward_only'] else '+bwd'}, "
-                      f"fp32 math on bf16-rounded inputs, best of 2; tokens/s is linear in tokens"}
+                      f"fp32 math on bf16-rounded inputs, one warm-up, median of 3 ({times[0]:.2f}/{times[1]:.2f}/"
+                      f"{times[2]:.2f} s); tokens/s is linear in tokens"}
+
+
+class ClockSampler:
+    """Samples the GPU's shader clock from sysfs (the level pp_dpm_sclk marks with '*') while the timed steps run."""
+
+    def __init__(self, period=0.02):
+        import glob
+        import threading
+        self.paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.samples, self.period = [], period
+        self._stop = threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _read(self):
+        for path in self.paths:
+            try:
+                for line in open(path):
+                    if "*" in line:
+                        return float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+            except (OSError, ValueError, IndexError):
+                continue
+        return None
+
+    def _run(self):
+        while not self._stop.is_set():
+            v = self._read()
+            if v is not None:
+                self.samples.append(v)
+            time.sleep(self.period)
+
+    def __enter__(self):
+        if self.paths:
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        if self.paths:
+            self._thread.join(timeout=1.0)
+
+    def summary(self):
+        if not self.samples:
+            return None
+        xs = sorted(self.samples)
+        return {"median_mhz": xs[len(xs) // 2], "min_mhz": xs[0], "max_mhz": xs[-1], "samples": len(xs),
+                "source": "pp_dpm_sclk (active level) sampled during the timed steps"}
+
+
+def parity_gate(w, step_fn, hidden2d, weight, shifted, old, ref, adv, rows_n=64):
+    """Before anything is timed: one step of the path on the benchmark's own inputs against the oracle.
+    `rows_n` sampled token rows (logprob, entropy, and the dHidden row when the workload has a backward) and the
+    loss.  The oracle forms the sampled rows' logits on the host from the same bf16 inputs in fp32; the loss is
+    its objective on the [T] logprob vector; its autograd gives the per-token gradient the dHidden rows must
+    show.  Returns the errors and whether they are inside the tolerances of the parity tests."""
+    import torch
+    from oracle import grpo_oracle as O
+    p = w.params
+    T, V = w.T, w.V
+    lp_all, ent_all, loss, dH = step_fn()          # what the timed steps compute, from the timed entry point
+    gsel = torch.Generator().manual_seed(17)
+    valid = torch.nonzero(shifted != -100).reshape(-1).cpu()
+    rows = valid[torch.randperm(valid.numel(), generator=gsel)[:rows_n]]
+    W_c = weight.detach().float().cpu()
+    hs_rows = hidden2d[rows.to(hidden2d.device)].detach().float().cpu().requires_grad_(not p["forward_only"])
+    y_rows = shifted[rows.to(shifted.device)].cpu()
+    x = hs_rows @ W_c.t()
+    want_lp = O.logprobs_from_logits(x, y_rows)
+    want_ent = O.entropy_from_logits(x.detach())
+    res = {"rows": int(rows.numel()),
+           "max_abs_dlogprob": float((lp_all[rows.to(lp_all.device)].cpu() - want_lp.detach()).abs().max()),
+           "max_abs_dentropy": float((ent_all[rows.to(ent_all.device)].cpu() - want_ent).abs().max()),
+           "tolerance": {"dlogprob": 2e-3, "dentropy": 5e-3, "loss_rel": 1e-3, "dH_rows_cosine": 0.999}}
+    ok = res["max_abs_dlogprob"] <= 2e-3 and res["max_abs_dentropy"] <= 5e-3
+    if not p["forward_only"]:
+        lp_c = lp_all.double().cpu().requires_grad_(True)
+        want = O.grpo_objective_from_logprobs(lp_c, shifted.cpu(), old.double().cpu(), adv.double().cpu(), p["clip_low"],
+                                              p["clip_high"], p["clip_ratio_c"], ref.double().cpu(), p["kl_beta"],
+                                              "sample_mean", w.cu_seqlens.cpu())
+        want[0].backward()
+        res["loss"] = float(loss.detach())
+        res["loss_oracle"] = float(want[0])
+        res["loss_rel_err"] = abs(float(loss.detach()) - float(want[0])) / max(abs(float(want[0])), 1e-30)
+        g_rows = lp_c.grad[rows].float()
+        (want_lp * g_rows).sum().backward()
+        got = dH.reshape(T, -1)[rows.to(dH.device)].float().cpu()
+        res["dH_rows_cosine"] = float(torch.nn.functional.cosine_similarity(got.flatten(), hs_rows.grad.flatten(), dim=0))
+        ok = ok and res["loss_rel_err"] <= 1e-3 and res["dH_rows_cosine"] >= 0.999
+    res["passed"] = bool(ok)
+    return res
 
 
 def attention_line(args):
@@ -228,10 +320,13 @@ def hbm_line(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="cfg1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true", help="skip the oracle check that precedes the timed steps")
+    ap.add_argument("--keep-logits", choices=["auto", "on", "off"], default="auto",
+                    help="keep the bf16 logits for the backward (auto: when supported and memory allows) or recompute them")
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed steps, run one 1 GiB device copy (reference point for traffic counters)")
     ap.add_argument("--seed", type=int, default=0)
@@ -264,6 +359,7 @@ def main():
     fwd_only = p["forward_only"]
     labels = w.labels
     shifted = ops.shift_labels(labels).reshape(-1)
+    keep_logits = {"auto": None, "on": True, "off": False}[args.keep_logits]
 
     # inputs of the objective: advantages from the group kernel, old/ref = current logprob + noise
     adv_s = ops.group_advantages(w.rewards, w.group_offsets, p["adv_eps"])
@@ -272,38 +368,65 @@ def main():
         lp0, _, _ = ops.lmhead_logprob_fwd(w.hidden.reshape(T, H), w.weight, None, shifted)
     old = lp0 + w.noise_old
     ref = lp0 + w.noise_ref
-    hidden = w.hidden.clone().requires_grad_(not fwd_only)
-    weight = w.weight.clone().requires_grad_(not fwd_only)
 
-    def step():
+    # Two input sets at different addresses, used in turn: no step finds the previous step's operands in a cache.
+    class Inputs:
+        def __init__(self):
+            self.hidden = w.hidden.clone().requires_grad_(not fwd_only)
+            self.weight = w.weight.clone().requires_grad_(not fwd_only)
+            self.old, self.ref, self.adv, self.labels = old.clone(), ref.clone(), adv.clone(), labels.clone()
+            self.cu = w.cu_seqlens.clone()
+    sets = [Inputs(), Inputs()]
+
+    def step(k=0):
+        s = sets[k % len(sets)]
         if fwd_only:
             with torch.no_grad():
-                return G.fused_log_probs_and_entropy_fn(weight, None, hidden, labels)
-        hidden.grad = None
-        weight.grad = None
-        out = G.grpo_loss_and_entropy_ce_fn(weight, None, hidden, labels, 1.0, old, adv, p["clip_low"], p["clip_high"],
-                                            p["clip_ratio_c"], loss_chunksize=p["chunk"], ref_logprobs=ref,
-                                            kl_beta=p["kl_beta"], loss_agg_mode="sample_mean", cu_seqlens=w.cu_seqlens)
+                return G.fused_log_probs_and_entropy_fn(s.weight, None, s.hidden, s.labels)
+        s.hidden.grad = None
+        s.weight.grad = None
+        out = G.grpo_loss_and_entropy_ce_fn(s.weight, None, s.hidden, s.labels, 1.0, s.old, s.adv, p["clip_low"],
+                                            p["clip_high"], p["clip_ratio_c"], loss_chunksize=p["chunk"],
+                                            ref_logprobs=s.ref, kl_beta=p["kl_beta"], loss_agg_mode="sample_mean",
+                                            cu_seqlens=s.cu, keep_logits=keep_logits)
         out[0].backward()
         return out
 
-    for _ in range(args.warmup):
-        step()
+    # ---- parity on the same inputs, before timing ----
+    def gate_step():
+        out = step(0)
+        torch.cuda.synchronize()
+        if fwd_only:
+            return out[0], out[1], None, None
+        return out[2] + old, out[1], out[0], sets[0].hidden.grad        # log_ratio = lp - old
+    parity = None
+    if not args.no_parity:
+        parity = parity_gate(w, gate_step, w.hidden.reshape(T, H), w.weight, shifted, old, ref, adv)
+        if not parity["passed"]:
+            print("bench.py: parity check failed, nothing timed: " + json.dumps(parity), file=sys.stderr)
+            sys.exit(1)
+
+    for i in range(args.warmup):
+        step(i)
     torch.cuda.synchronize()
-    # dominant kernel: the forward statistics kernel (one launch per step = all T tokens x all V rows), timed
-    # inside the timed steps with HIP events recorded on the launch stream around the library call
-    # (the bracket also holds the per-token combine kernel, some tens of microseconds).
+    # Per-kernel times inside the timed steps: HIP events recorded on the launch stream around the forward's
+    # library call (the bracket also holds the per-token combine kernel, some tens of microseconds) and, inside the
+    # library, around each launch of the backward.
     fwd_events = []
     ops.set_fwd_event_sink(fwd_events)
+    if not fwd_only:
+        ops.phase_timing_begin()
     step_events = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    t0 = time.perf_counter()
-    step_events[0].record()
-    for i in range(args.steps):
-        step()
-        step_events[i + 1].record()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    with ClockSampler() as clock:
+        t0 = time.perf_counter()
+        step_events[0].record()
+        for i in range(args.steps):
+            step(i)
+            step_events[i + 1].record()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
     ops.set_fwd_event_sink(None)
+    phase_ms, phase_n, dropped = ops.phase_timing_end() if not fwd_only else ({}, {}, 0)
     per_step = sorted(step_events[i].elapsed_time(step_events[i + 1]) for i in range(args.steps))
     ms = dt / args.steps * 1e3
     tok_s = T / (ms / 1e3)
@@ -316,9 +439,31 @@ def main():
         torch.cuda.synchronize()
         dst.copy_(src)
         torch.cuda.synchronize()
-    flops_launch = 2.0 * T * H * V
-    achieved = flops_launch / (k_ms * 1e-3) / 1e12
-    alg_flops_step = (2.0 if fwd_only else 6.0) * T * H * V
+    thv = 2.0 * T * H * V
+    achieved = thv / (k_ms * 1e-3) / 1e12
+    alg_flops_step = (1.0 if fwd_only else 3.0) * thv
+    kept = (not fwd_only) and phase_n.get("dlogits", 0) == args.steps and phase_n.get("dh", 0) == args.steps
+    executed = (1.0 if fwd_only else (3.0 if kept else 4.0)) * thv
+
+    def phase(kernel, total_ms, flops, note=None):
+        per = total_ms / args.steps
+        d = {"kernel": kernel, "ms": per, "flops": flops,
+             "frac": (flops / (per * 1e-3) / 1e12 / PEAK_BF16_TFLOPS) if (flops and per > 0) else None}
+        if note:
+            d["note"] = note
+        return d
+    phases = [phase("lmhead_fwd_kernel" + (" (keeps bf16 logits)" if kept else "") + " + combine", k_ms * args.steps, thv)]
+    if not fwd_only:
+        if kept:
+            phases.append(phase("kept_logits_to_dlogits_kernel", phase_ms["dlogits"], 0.0,
+                                f"HBM-bound: {4.0 * T * V / 1e9:.1f} GB per launch = "
+                                f"{4.0 * T * V / (phase_ms['dlogits'] / args.steps * 1e-3) / 1e12:.2f} TB/s"))
+        else:
+            phases.append(phase(f"lmhead_ds_kernel x {phase_n['dlogits'] // args.steps} panels (recomputes the logits)",
+                                phase_ms["dlogits"], thv, "executed, not algorithmic, work"))
+        phases.append(phase(f"gemm_store_kernel dHidden x {phase_n['dh'] // args.steps}", phase_ms["dh"], thv))
+        phases.append(phase(f"gemm_store_kernel dW x {phase_n['dw'] // args.steps}", phase_ms["dw"], thv))
+    prof = PROFILED_TRAFFIC.get((args.config, bool(kept)))
 
     line = {
         "metric": "packed tokens/sec fused logprob+GRPO fwd/bwd (Qwen2.5-1.5B shape); MFMA % peak",
@@ -328,17 +473,28 @@ def main():
         "config": {"workload": f"{args.config}: T={T} packed tokens, H={H}, V={V}, "
                                f"{'forward only' if fwd_only else 'forward+backward (dHidden, dW)'}, "
                                f"{w.n_samples} samples, chunk hint {p['chunk']}",
-                   "tokens": T, "hidden": H, "vocab": V, "samples": w.n_samples},
+                   "tokens": T, "hidden": H, "vocab": V, "samples": w.n_samples,
+                   "backward": None if fwd_only else ("bf16 logits kept for the backward" if kept else "logits recomputed in the backward"),
+                   "input_sets_rotated": len(sets)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
-                     "kernel": "lmhead_fwd_kernel (+ per-token combine)", "kernel_ms": k_ms,
+                     "frac": achieved / PEAK_BF16_TFLOPS,
+                     "frac_at_held_clock": (achieved / (PEAK_BF16_TFLOPS * clock.summary()["median_mhz"] / PEAK_CLOCK_MHZ))
+                     if clock.summary() else None,
+                     "traffic": prof[0] if prof else None,
+                     "traffic_source": (prof[1] + " (rocprofv3 --pmc runs of this command; not measured in this run)") if prof else None,
+                     "kernel": phases[0]["kernel"], "kernel_ms": k_ms,
                      "kernel_launches_timed": len(fwd_events),
-                     "algorithmic_flops_per_launch": flops_launch},
+                     "algorithmic_flops_per_launch": thv,
+                     "phases": phases, "phase_brackets_dropped": dropped,
+                     "peak_note": f"published peak = {PEAK_CLOCK_MHZ:.0f} MHz x 256 CUs x 4096 flop/cycle; the clock the "
+                                  "device held during the timed steps is under 'clock'"},
+        "clock": clock.summary(),
+        "parity": parity,
         "ms_per_step_median": per_step[len(per_step) // 2], "ms_per_step_min": per_step[0],
         "path_mfma_frac": alg_flops_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "path_algorithmic_tflops": alg_flops_step / (ms * 1e-3) / 1e12,
-        # what the matrix pipeline executes: the backward recomputes the logits once (nothing [T x V] is kept)
-        "path_executed_tflops": (2.0 if fwd_only else 8.0) * T * H * V / (ms * 1e-3) / 1e12,
+        # what the matrix pipeline executes: with kept logits the three algorithmic products, otherwise a fourth
+        "path_executed_tflops": executed / (ms * 1e-3) / 1e12,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.config, p["chunk"], args.seed)

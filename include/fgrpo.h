@@ -132,6 +132,20 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
                           void* dH_out, void* dW_out, void* dbias_out,
                           void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- diagnostics: GPU time per phase of the backward ------------------------------------------------------
+ * Between fgrpo_phase_timing_begin() and fgrpo_phase_timing_end() every fgrpo_lmhead_bwd / fgrpo_lmhead_bwd_kept
+ * call of the process (whatever thread makes it: autograd runs backwards on its own) brackets its launches with
+ * HIP events on the call's stream (the library creates FGRPO_MAX_TIMED_PHASES event pairs on first use; later
+ * brackets are counted as dropped).  Meant for one stream at a time.  _end waits
+ * for the last event and returns, per phase, the summed milliseconds and the number of brackets:
+ * phase 0 = dLogits (recomputing kernel, or the in-place pass over kept logits), 1 = dHidden product,
+ * 2 = dW product, 3 = everything else (operand staging, bias sums).  Returns the number of dropped brackets
+ * (0 = all timed) or a negative error.  Timing is off unless begun; no counterpart in the reference. */
+#define FGRPO_NUM_PHASES 4
+#define FGRPO_MAX_TIMED_PHASES 1024
+int fgrpo_phase_timing_begin(void);
+int fgrpo_phase_timing_end(float* ms_by_phase, int* brackets_by_phase);
+
 /* ---- per-token GRPO objective -------------------------------------------------
  * Replaces the tail of grpo_loss_and_entropy_ce_fn (grpo_loss.py:318-348):
  * ratio, dual clip, masked mean.  old_lp NULL => ratio 1 (grpo_loss.py:318-319).
