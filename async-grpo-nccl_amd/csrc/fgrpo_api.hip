@@ -433,7 +433,14 @@ bool keep_supported(const Tuning& tn, int T, int H, int V, int dtype) {
   const long long th = (long long)((T + 255) / 256) * (H / 256), vh = (long long)((V + 255) / 256) * (H / 256);
   return th >= num_cus() / 2 && vh >= num_cus() / 2;
 }
-size_t keep_bytes(int T, int V) { return (size_t)round_up(V, 256) * (size_t)round_up(T, 256) * sizeof(bf16_t); }
+// Layout of the kept buffer: the column-blocked bf16 numerators, then the per-token references (fp32), then the
+// overflow flag (one int in its own 256 bytes).
+size_t keep_block_bytes(int T, int V) { return (size_t)round_up(V, 256) * (size_t)round_up(T, 256) * sizeof(bf16_t); }
+size_t keep_bytes(int T, int V) { return keep_block_bytes(T, V) + (size_t)round_up(T, 256) * sizeof(float) + 256; }
+float* keep_ref2_of(void* keep, int T, int V) { return (float*)((char*)keep + keep_block_bytes(T, V)); }
+int* keep_flag_of(void* keep, int T, int V) {
+  return (int*)((char*)keep + keep_block_bytes(T, V) + (size_t)round_up(T, 256) * sizeof(float));
+}
 
 int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
                       int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
@@ -475,6 +482,13 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   if (keep) {
     p.keep = (bf16_t*)keep;
     p.keep_blk = (long long)pl.tiles_t * kCfg[8].bn * 256;
+    float* ref2 = keep_ref2_of(keep, T, V);
+    int* flag = keep_flag_of(keep, T, V);
+    KeepRefParams r{(const bf16_t*)hidden, (const bf16_t*)weight, p.bias, (const long long*)labels, T, H, V, inv_temp, ref2, flag};
+    hipLaunchKernelGGL(keep_reference_kernel, dim3((T + 3) / 4), dim3(256), 0, st, r);
+    HIP_TRY(hipGetLastError());
+    p.keep_ref2 = ref2;
+    p.keep_flag = flag;
     rc = launch_fwd_keep(p, st);
   } else {
     rc = launch_fwd_variant(pl.variant, p, st);
@@ -772,13 +786,36 @@ void kept_panels(const Tuning& tn, int T, int H, int V, int& panel, int& npanels
 }
 }  // namespace
 
+namespace {
+struct KeptBwdPlan {
+  float* row_scale;       // [T]
+  bf16_t* hidden_scaled;  // [T x H]
+  float* dh_acc;          // [T x H] fp32, panels > 1 only
+  size_t bytes;
+};
+void plan_kept_bwd(KeptBwdPlan& pl, void* ws, int T, int H) {
+  Carver cv(ws);
+  pl.row_scale = cv.take<float>((size_t)T);
+  pl.hidden_scaled = cv.take<bf16_t>((size_t)T * H);
+  pl.dh_acc = cv.take<float>((size_t)T * H);     // always sized: a concurrent set_tuning must not make it short
+  pl.bytes = cv.total();
+}
+}  // namespace
+
 size_t fgrpo_lmhead_bwd_kept_workspace(int T, int H, int V, int dtype) {
   if (T <= 0 || H <= 0 || V <= 0 || dtype != FGRPO_BF16) return 0;
-  int panel = 0, np = 0;
-  kept_panels(g_tune, T, H, V, panel, np);
-  // sized for any panel count: a concurrent set_tuning must not turn a sufficient workspace into a short one
-  (void)np;
-  return (size_t)round_up((long long)T * H * (long long)sizeof(float), 256);
+  KeptBwdPlan pl;
+  plan_kept_bwd(pl, nullptr, T, H);
+  return pl.bytes;
+}
+
+int fgrpo_keep_overflowed(const void* logits_keep, int T, int V, void* stream) {
+  if (!logits_keep || T <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "keep_overflowed: bad argument");
+  int flag = 0;
+  HIP_TRY(hipMemcpyAsync(&flag, keep_flag_of(const_cast<void*>(logits_keep), T, V), sizeof(int), hipMemcpyDeviceToHost,
+                         (hipStream_t)stream));
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return flag != 0 ? 1 : 0;
 }
 
 int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bias, const int64_t* labels,
@@ -793,26 +830,25 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
   if (!keep_supported(tn, T, H, V, dtype))
     return fail(FGRPO_ERR_UNSUPPORTED, "lmhead_bwd_kept: needs bf16, H %% 256 == 0 and a device-filling problem (T=%d H=%d V=%d)", T, H, V);
   if (!logits_keep || !aligned16(logits_keep) || logits_keep_bytes < keep_bytes(T, V))
-    return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: logits buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
+    return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: kept buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
   if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: dbias requested without a bias");
   if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "lmhead_bwd_kept: hidden/weight must be 16-byte aligned");
   if (!dH_out && !dW_out && !dbias_out) return 0;
-  const int Tpad = (int)round_up(T, 256), Vpad = (int)round_up(V, 256);
+  KeptBwdPlan pl;
+  plan_kept_bwd(pl, ws, T, H);
+  if (!ws || !aligned16(ws) || ws_bytes < pl.bytes)
+    return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: workspace null, misaligned or smaller than %zu bytes", pl.bytes);
+  const int Tpad = (int)round_up(T, 256);
   const long long blk = (long long)Tpad * 256;
-  bf16_t* ds = (bf16_t*)logits_keep;
+  bf16_t* ek = (bf16_t*)logits_keep;
   int panel = 0, npanels = 0;
   kept_panels(tn, T, H, V, panel, npanels);
-  float* dh_acc = nullptr;
-  if (dH_out && npanels > 1) {
-    if (!ws || !aligned16(ws) || ws_bytes < (size_t)T * H * sizeof(float))
-      return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: workspace null, misaligned or smaller than %zu bytes", (size_t)T * H * sizeof(float));
-    dh_acc = (float*)ws;
-  }
 
-  KeptParams k{ds, blk, Tpad, T, V, (const long long*)labels, lse, g, gout_dev, inv_temp};
   {
     PhaseScope ph(kPhaseDlogits, st);
-    hipLaunchKernelGGL(kept_logits_to_dlogits_kernel, dim3((unsigned)((Vpad / 256) * (Tpad / kKeptRows))), dim3(256), 0, st, k);
+    KeepPrepParams k{ek, blk, keep_ref2_of(logits_keep, T, V), (const long long*)labels, lse, g, gout_dev, inv_temp,
+                     (const bf16_t*)hidden, T, H, V, pl.row_scale, dW_out ? pl.hidden_scaled : nullptr};
+    hipLaunchKernelGGL(keep_backward_prep_kernel, dim3((T + 3) / 4), dim3(256), 0, st, k);
   }
   HIP_TRY(hipGetLastError());
 
@@ -820,9 +856,9 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
   for (int pi = 0; pi < npanels; ++pi) {
     const int v0 = pi * panel;
     const int rows = (V - v0) < panel ? (V - v0) : panel;      // vocabulary rows of W / dW in this panel
-    const int kv = (int)round_up(rows, 256);                   // dLogits columns of the panel (zero past V)
-    bf16_t* ds_p = ds + (long long)(v0 / 256) * blk;
-    if (dH_out) {   // dH[T x H] (+)= dS[T x kv] W[v0 : v0+rows, H]: A column-blocked K-contiguous, B = W read in place
+    const int kv = (int)round_up(rows, 256);                   // columns of the panel (zero past V)
+    bf16_t* ek_p = ek + (long long)(v0 / 256) * blk;
+    if (dH_out) {   // dH[T x H] (+)= diag(a) E'[T x kv] W[v0 : v0+rows, H]: A column-blocked K-contiguous, B = W read in place
       StoreParams s;
       memset(&s, 0, sizeof(s));
       s.g.M = T;
@@ -831,23 +867,24 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       s.g.a_blk = blk;
       s.g.ldb = H;
       s.g.nseg = 1;
-      s.g.seg[0] = GemmSeg{ds_p, (const bf16_t*)weight + (size_t)v0 * H, kv};
+      s.g.seg[0] = GemmSeg{ek_p, (const bf16_t*)weight + (size_t)v0 * H, kv};
       s.g.kb_valid = rows;
       s.ldc = H;
       s.alpha = 1.f;
+      s.row_scale = pl.row_scale;
       const bool first = (pi == 0), last = (pi == npanels - 1);
-      s.c_in = first ? nullptr : dh_acc;
+      s.c_in = first ? nullptr : pl.dh_acc;
       if (last)
         s.c_out_bf16 = (bf16_t*)dH_out;
       else
-        s.c_out_f32 = dh_acc;
+        s.c_out_f32 = pl.dh_acc;
       {
         PhaseScope ph(kPhaseDh, st);
         rc = run_store_gemm_kmajor(tn, s, false, true, st);
       }
       if (rc) return rc;
     }
-    if (dW_out) {   // dW[v0 : v0+rows, H] = dS^T[rows x Tpad] hidden[Tpad x H]: the token is the contraction row of both
+    if (dW_out) {   // dW[v0 : v0+rows, H] = E'^T[rows x Tpad] (diag(a) hidden)[Tpad x H]: the token is the contraction row of both
       StoreParams s;
       memset(&s, 0, sizeof(s));
       s.g.M = rows;
@@ -856,7 +893,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       s.g.a_blk = blk;
       s.g.ldb = H;
       s.g.nseg = 1;
-      s.g.seg[0] = GemmSeg{ds_p, (const bf16_t*)hidden, Tpad};
+      s.g.seg[0] = GemmSeg{ek_p, pl.hidden_scaled, Tpad};
       s.g.kb_valid = T;
       s.ldc = H;
       s.alpha = 1.f;
@@ -869,8 +906,9 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
     }
   }
   if (dbias_out) {
-    hipLaunchKernelGGL(panel_col_sum_kernel, dim3((V + 63) / 64), dim3(256), 0, st, ds, (const bf16_t*)nullptr,
-                       (long long)Vpad, blk, T, V, (float*)nullptr, (bf16_t*)dbias_out);
+    PhaseScope ph(kPhaseOther, st);
+    hipLaunchKernelGGL(keep_col_sum_kernel, dim3((V + 63) / 64), dim3(256), 0, st, ek, blk, pl.row_scale, T, V,
+                       (bf16_t*)dbias_out);
     HIP_TRY(hipGetLastError());
   }
   return 0;

@@ -439,7 +439,11 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   constexpr int D = C::NSTAGE - 1;              // K steps of loads in flight
   constexpr int LPT = C::PA + C::PB;            // loads per thread per K step
   static_assert(D >= 1 && D <= 4 && LPT * (D - 1) < 64, "pipeline depth");
-  const int tid = threadIdx.x;
+  // The per-lane offsets below are cheap to derive and expensive to keep: a caller that runs this loop once per
+  // tile with an epilogue in between would otherwise carry two dozen loop-invariant registers through that
+  // epilogue.  The empty asm makes the thread id opaque, so they are recomputed per call.
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront-uniform: LDS targets stay scalar
   const int wm = wave / C::WN, wn = wave % C::WN;

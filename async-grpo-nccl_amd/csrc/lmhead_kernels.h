@@ -46,12 +46,22 @@ struct FwdParams {
   int tiles_v, tiles_t, nsplit, group_t;
   float4* part;              // [nsplit][T] : (m, s, sx, unused)
   float* xt;                 // [T] target logit (written only where a valid label exists)
-  // KEEP kernels only: the raw products x = W h + b (before the temperature), rounded to bf16, for the backward
-  // that does not recompute them.  Column-blocked [V/256][keep_rows][256]: element (t, v) at
+  // KEEP kernels only: the soft-max numerators for the backward that does not recompute the logits,
+  //   E[t, v] = exp(x_tv / temperature - ref_t)   (bf16; x = W h + b),
+  // against a per-token reference chosen BEFORE the sweep (keep_ref2 = ref_t * log2(e); +huge for tokens that take no
+  // gradient, whose rows are then stored as exact zeros).  The probability is E[t, v] * exp(ref_t - lse_t): one
+  // factor per token, which the gradient GEMMs apply to their output rows / to the other operand, so the buffer
+  // feeds them as it is.  Column-blocked [V/256][keep_rows][256]: element (t, v) at
   // (v / 256) * keep_blk + t * 256 + v % 256, keep_blk = keep_rows * 256, keep_rows = token tiles * BN.
+  // keep_flag: set to 1 when some row's running maximum exceeds its reference by more than kKeepHeadroom2 (the stored
+  // values may then have overflowed and the caller must recompute instead).
   bf16_t* keep;
   long long keep_blk;
+  const float* keep_ref2;    // [T]
+  int* keep_flag;
 };
+
+constexpr float kKeepHeadroom2 = 120.f;   // log2 units: exp2(120) * (values <= 1) stays finite in bf16 / fp32
 
 // One 32-token x WTM-entry slab of bf16 values (the sub-tile column block j of a wavefront in the LM-head
 // orientation: lane = token, 16 vocabulary rows per 32x32 block) written to a column-blocked buffer through the
@@ -61,22 +71,22 @@ struct FwdParams {
 // n so that the 32 lanes of a write hit 32 different slots.  LDS traffic is inline assembly (the compiler would
 // otherwise wait for the direct-to-LDS loads of the next tile that are in flight); LDS operations of one wavefront
 // complete in order, so one wait before the stores is enough.  `out` points at (first token of the slab, first
-// vocabulary entry of the wavefront's rows) in the block; pk(i, q) returns the packed entries
-// i*32 + 8*q + 4*(lane/32) + 0..3 of this lane's token.
-template <class C, class PK>
-__device__ __forceinline__ void store_slab_via_patch(char* patch, bf16_t* out, int lane_v, PK&& pk) {
+// vocabulary entry of the wavefront's rows) in the block.
+// patch_write_quad: entries i*32 + 8*q + 4*(lane/32) + 0..3 of this lane's token (8 bytes) into the patch;
+// patch_flush: the whole slab out, after every quad of the slab has been written.
+template <class C>
+__device__ __forceinline__ void patch_write_quad(char* patch, int lane_v, int i, int q, uint2 v) {
   constexpr int ROWP = C::WTM * 2;                       // patch row: one token's WTM entries
   constexpr int NSLOT = ROWP / 8;                        // 8-byte slots per row
+  const int slot = ((i * 32 + 8 * q) >> 2) + (lane_v >> 5);
+  lds_write_b64_asm(lds_addr(patch) + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3), v.x, v.y);
+}
+template <class C>
+__device__ __forceinline__ void patch_flush(char* patch, bf16_t* out, int lane_v) {
+  constexpr int ROWP = C::WTM * 2;
+  constexpr int NSLOT = ROWP / 8;
   constexpr int PPT = ROWP / 16, TPP = 64 / PPT;         // 16-byte pieces per token, tokens per store instruction
   static_assert(64 % PPT == 0 && 32 % TPP == 0 && (NSLOT & (NSLOT - 1)) == 0, "epilogue patch");
-#pragma unroll
-  for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint2 v = pk(i, q);
-      const int slot = ((i * 32 + 8 * q) >> 2) + (lane_v >> 5);
-      lds_write_b64_asm(lds_addr(patch) + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3), v.x, v.y);
-    }
   u32x4_t pv[32 / TPP];
 #pragma unroll
   for (int r = 0; r < 32 / TPP; ++r) {
@@ -117,6 +127,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
   const int col0 = tt * C::BN;
 
   float m_run[C::TN], s_run[C::TN], sx_run[C::TN];
+  float ref2[C::TN];         // KEEP only
   int y[C::TN];
 #pragma unroll
   for (int j = 0; j < C::TN; ++j) {
@@ -126,6 +137,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
     const int n = col0 + acc_col<C>(wn, j, lane);
     long long lab = (n < T) ? p.labels[n] : -1;
     y[j] = (lab >= 0 && lab < V) ? (int)lab : -1;
+    if constexpr (KEEP) ref2[j] = (n < T) ? p.keep_ref2[n] : -kNegBig;
   }
 
   // KEEP: the wavefront's patch lives behind LDS buffer 0, which the prefetch of the next tile may already be filling
@@ -181,19 +193,6 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
       // a slot that has seen only masked rows keeps (m, s, sx) = (kNegBig, 0, 0):
       // x*xs - mb would otherwise be the rounding residue of two huge terms
       const float mb = (mn > 0.5f * kNegBig) ? mn * xs : 0.f;
-      float s = s_run[j] * alpha, sx = sx_run[j] * alpha;
-#pragma unroll
-      for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float x = acc[i][j][r];
-          const float e = fast_exp2(__builtin_fmaf(x, xs, -mb));
-          s += e;
-          sx = __builtin_fmaf(e, x, sx);
-        }
-      m_run[j] = mn;
-      s_run[j] = s;
-      sx_run[j] = sx;
       // target logit: rows of this lane are lane_row0 + i*32 + 8*(r/4) + (r%4)
       const int yrel = y[j] - row0 - wm * C::WTM - 4 * (lane >> 5);
       if (y[j] >= 0 && yrel >= 0 && yrel < C::WTM) {
@@ -209,18 +208,48 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
           }
         if (hit) p.xt[col0 + acc_col<C>(wn, j, lane)] = xv * p.inv_temp;
       }
+      // KEEP: the exponential computed for the statistics (relative to the running maximum) times one factor per
+      // token and tile re-bases it on the token's fixed reference; it replaces the accumulator it came from
+      float kf = 0.f;
       if constexpr (KEEP) {
-        // the addresses are recomputed per tile on purpose (hoisted they would sit in registers across the main loop)
-        int lane_v = lane;
-        asm volatile("" : "+v"(lane_v));
-        bf16_t* out = p.keep + (long long)vt * p.keep_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
-        store_slab_via_patch<C>(patch, out, lane_v, [&](int i, int q) {
-          uint2 pk;
-          pk.x = pack_bf16x2(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
-          pk.y = pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
-          return pk;
-        });
+        const float d2 = mb - ref2[j];
+        kf = fast_exp2(d2);
+        if (d2 > kKeepHeadroom2 && ref2[j] < 0.5f * -kNegBig) *p.keep_flag = 1;
       }
+      float s = s_run[j] * alpha, sx = sx_run[j] * alpha;
+      // KEEP: the patch addresses are recomputed per tile on purpose (hoisted they would sit in registers across the
+      // main loop); every quad goes to the patch as soon as its statistics are folded in
+      int lane_v = lane;
+      if constexpr (KEEP) asm volatile("" : "+v"(lane_v));
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float ek[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const float x = acc[i][j][q * 4 + c];
+            const float e = fast_exp2(__builtin_fmaf(x, xs, -mb));
+            s += e;
+            sx = __builtin_fmaf(e, x, sx);
+            ek[c] = e * kf;
+          }
+          if constexpr (KEEP) {
+            uint2 pk;
+            pk.x = pack_bf16x2(ek[0], ek[1]);
+            pk.y = pack_bf16x2(ek[2], ek[3]);
+            patch_write_quad<C>(patch, lane_v, i, q, pk);
+            // pin the running sums here: left alone the compiler first computes all 64 exponentials of the column
+            // (to feed the patch writes) and folds them into the sums afterwards, which keeps all of them in registers
+            asm volatile("" : "+v"(s), "+v"(sx));
+          }
+        }
+      m_run[j] = mn;
+      s_run[j] = s;
+      sx_run[j] = sx;
+      if constexpr (KEEP)
+        patch_flush<C>(patch, p.keep + (long long)vt * p.keep_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM,
+                       lane_v);
     }
   }
 
@@ -491,6 +520,7 @@ struct StoreParams {
   const float* alpha_dev;  // optional device scalar multiplied into alpha
   int tiles_m, tiles_n, group_m;
   int wide_stores;         // ldc and the output / addend bases allow 16-byte pieces (set by the launcher)
+  const float* row_scale;  // optional [M]: output row m is multiplied by row_scale[m] (after alpha, before c_in)
 };
 
 // Output is either fp32 or bf16 (never both); rows/cols past M/N are skipped.
@@ -511,6 +541,7 @@ __device__ __forceinline__ void store_tile(const StoreParams& p, f32x16_t (&acc)
           if (rr < mrem) {
             const long long o = o0 + (long long)rr * p.ldc;
             float v = acc[i][j][r] * alpha;
+            if (p.row_scale) v *= p.row_scale[row0 + wm * C::WTM + 4 * (lane >> 5) + rr];
             if (HAS_IN) v += p.c_in[o];
             if (OUT_BF16)
               p.c_out_bf16[o] = f32_to_bf16_rn(v);
@@ -566,6 +597,11 @@ __device__ __forceinline__ void store_tile_lds(const StoreParams& p, f32x16_t (&
       }
       if (m >= p.g.M || n0 >= p.g.N) continue;
       const long long o = (long long)m * p.ldc + n0;
+      if (p.row_scale) {
+        const float rs = p.row_scale[m];
+#pragma unroll
+        for (int e = 0; e < PIECE; ++e) v[e] *= rs;
+      }
       if (n_full) {
         if (HAS_IN) {
 #pragma unroll

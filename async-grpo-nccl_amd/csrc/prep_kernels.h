@@ -147,82 +147,120 @@ __global__ void panel_row_sum_kernel(const bf16_t* vt_hi, const bf16_t* vt_lo, l
 
 
 // ---------------------------------------------------------------------------
-// Backward without recomputation: the forward kept x = W h + b (bf16, column-blocked [V/256][rows][256]); this
-// kernel turns the buffer into dLogits in place,
-//   dS[t, v] = c_t * (1[v == y_t] - exp(x_tv / temperature - lse_t)),  c_t = g_t * gout / temperature,
-// which the two gradient GEMMs then read where it lies.  Rows with c_t == 0 (ignored labels, zero gradient, padding
-// rows t >= T) are written as zeros without being read.  HBM-bound: 2 bytes read and 2 written per logit.
-// One work-group = 64 token rows of one 256-column block (32 KiB, contiguous); a row is 32 lanes x 16 bytes.
+// Kept soft-max numerators (forward KEEP kernel): the small kernels around them.
+//
+// keep_reference_kernel, before the forward: the per-token reference of the stored exponentials,
+//   ref_t = x_t[y_t] / temperature + kKeepOffset   (x_t[y_t] = W[y_t] . h_t + b[y_t], a dot product per token),
+// written as ref_t * log2(e); +huge for tokens with an ignored or invalid label (their rows are stored as zeros).
+// Stored values are exp(x_tv/temperature - ref_t) = p_v / p_y * exp(-kKeepOffset): finite in bf16 as long as the
+// target's log-probability is above -(88 + kKeepOffset) = -128 nats; the forward kernel raises a flag otherwise.
+//
+// keep_backward_prep_kernel, before the gradient GEMMs: with s_t = exp(ref_t - lse_t) the probability is
+// p_tv = E[t, v] * s_t, so dLogits[t, v] = c_t (1[v = y_t] - p_tv) = a_t * E'[t, v] with
+//   a_t = -c_t * s_t,   E' = E except E'[t, y_t] = (p_y - 1) / s_t  (written in place, from the fp32 lse, not from
+//   the stored bf16 value),   c_t = g_t * gout / temperature.
+// dHidden = diag(a) (E' W): the row factor goes into the GEMM's epilogue; dW = E'^T (diag(a) hidden): the kernel
+// writes the scaled copy of hidden.  One work-group of 256 threads per 4 tokens (a wavefront per token).
 // ---------------------------------------------------------------------------
-struct KeptParams {
-  bf16_t* x;                 // in: kept logits, out: dLogits
-  long long blk;             // elements between column blocks (= rows * 256)
-  int rows;                  // token rows per block (multiple of 64, >= T)
-  int T, V;
+constexpr float kKeepOffset = 40.f;
+
+struct KeepRefParams {
+  const bf16_t* hidden;      // [T][H]
+  const bf16_t* weight;      // [V][H]
+  const float* bias;         // [V] fp32 or null
+  const long long* labels;   // shifted labels [T]
+  int T, H, V;
+  float inv_temp;
+  float* ref2;               // [T] out
+  int* flag;                 // cleared here (one int)
+};
+
+__global__ __launch_bounds__(256) void keep_reference_kernel(const KeepRefParams p) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *p.flag = 0;
+  if (t >= p.T) return;
+  const long long lab = p.labels[t];
+  if (lab < 0 || lab >= p.V) {                 // ignored (-100) or invalid: no gradient, row stored as zeros
+    if (lane == 0) p.ref2[t] = -kNegBig;
+    return;
+  }
+  const u32x4_t* h = (const u32x4_t*)(p.hidden + (long long)t * p.H);
+  const u32x4_t* w = (const u32x4_t*)(p.weight + lab * p.H);
+  float acc = 0.f;
+  for (int c = lane; c < p.H / 8; c += 64) {   // H is a multiple of 8 (checked by the caller)
+    const u32x4_t a = h[c], b = w[c];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc = __builtin_fmaf(__uint_as_float(a[e] << 16), __uint_as_float(b[e] << 16), acc);
+      acc = __builtin_fmaf(__uint_as_float(a[e] & 0xffff0000u), __uint_as_float(b[e] & 0xffff0000u), acc);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if (lane == 0) p.ref2[t] = ((acc + (p.bias ? p.bias[lab] : 0.f)) * p.inv_temp + kKeepOffset) * kLog2e;
+}
+
+struct KeepPrepParams {
+  bf16_t* e;                 // kept numerators, column-blocked (element (t, y_t) is patched)
+  long long blk;             // elements between column blocks
+  const float* ref2;         // [T]
   const long long* labels;   // shifted labels [T]
   const float* lse;          // [T]
   const float* gtok;         // [T]
   const float* gout;         // device scalar or null
   float inv_temp;
+  const bf16_t* hidden;      // [T][H]
+  int T, H, V;
+  float* row_scale;          // [T] out: a_t
+  bf16_t* hidden_scaled;     // [T][H] out: a_t * hidden[t], or null
 };
 
-constexpr int kKeptRows = 64;
+__global__ __launch_bounds__(256) void keep_backward_prep_kernel(const KeepPrepParams p) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= p.T) return;
+  const long long lab = p.labels[t];
+  float a = 0.f;
+  if (lab >= 0 && lab < p.V) {
+    const float c = p.gtok[t] * (p.gout ? *p.gout : 1.f) * p.inv_temp;
+    const float d2 = p.ref2[t] - p.lse[t] * kLog2e;        // log2 s_t
+    a = -c * fast_exp2(d2);
+    if (lane == 0) {
+      // p_y - 1 from the fp32 quantities: log p_y = x_y/temperature - lse = (ref - offset) - lse
+      const float lp = (d2 * (1.f / kLog2e)) - kKeepOffset;
+      const float pm1 = expm1f(lp);
+      p.e[(lab >> 8) * p.blk + (long long)t * 256 + (lab & 255)] = f32_to_bf16_rn(pm1 * fast_exp2(-d2));
+    }
+  }
+  if (lane == 0) p.row_scale[t] = a;
+  if (p.hidden_scaled) {
+    const u32x4_t* h = (const u32x4_t*)(p.hidden + (long long)t * p.H);
+    u32x4_t* o = (u32x4_t*)(p.hidden_scaled + (long long)t * p.H);
+    for (int cidx = lane; cidx < p.H / 8; cidx += 64) {
+      const u32x4_t v = h[cidx];
+      u32x4_t r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        r[e] = pack_bf16x2(a * __uint_as_float(v[e] << 16), a * __uint_as_float(v[e] & 0xffff0000u));
+      o[cidx] = r;
+    }
+  }
+}
 
-__global__ __launch_bounds__(256) void kept_logits_to_dlogits_kernel(const KeptParams p) {
-  __shared__ float s_c[kKeptRows], s_l2[kKeptRows];
-  __shared__ int s_y[kKeptRows];
-  const int chunks = p.rows / kKeptRows;
-  const int vb = blockIdx.x / chunks, t0 = (blockIdx.x - vb * chunks) * kKeptRows;
-  const int tid = threadIdx.x;
-  if (tid < kKeptRows) {
-    const int t = t0 + tid;
-    float c = 0.f, l2 = 0.f;
-    int y = -1;
-    if (t < p.T) {
-      const long long lab = p.labels[t];
-      if (lab != -100) {
-        c = p.gtok[t] * (p.gout ? *p.gout : 1.f) * p.inv_temp;
-        l2 = p.lse[t] * kLog2e;
-        y = (lab >= 0 && lab < p.V) ? (int)lab - vb * 256 : -1;    // column inside this block, or out of range
-      }
-    }
-    s_c[tid] = c;
-    s_l2[tid] = l2;
-    s_y[tid] = y;
+// dbias from the kept numerators: out[v] = sum_t a_t * E'[t][v].  One block owns 64 columns; its four row groups
+// are combined in a fixed order.
+__global__ void keep_col_sum_kernel(const bf16_t* e, long long blk, const float* row_scale, int T, int V,
+                                    bf16_t* out_bf16) {
+  __shared__ float red[4][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + tx;
+  float s = 0.f;
+  if (c < V) {
+    const bf16_t* col = e + (long long)(c >> 8) * blk + (c & 255);
+    for (int t = ty; t < T; t += 4) s = __builtin_fmaf(row_scale[t], bf16_to_f32(col[(long long)t * 256]), s);
   }
+  red[ty][tx] = s;
   __syncthreads();
-  const float xs = p.inv_temp * kLog2e;
-  const int r0 = tid >> 5, cpos = (tid & 31) * 8;          // row inside a pass of 8 rows, first column of the lane
-  u32x4_t* base = (u32x4_t*)(p.x + (long long)vb * p.blk + (long long)t0 * 256) + tid;   // + pass * 256 pieces
-  u32x4_t v[kKeptRows / 8];
-#pragma unroll
-  for (int ps = 0; ps < kKeptRows / 8; ++ps)
-    if (s_c[ps * 8 + r0] != 0.f) v[ps] = __builtin_nontemporal_load(base + ps * 256);
-#pragma unroll
-  for (int ps = 0; ps < kKeptRows / 8; ++ps) {
-    const int r = ps * 8 + r0;
-    const float c = s_c[r];
-    u32x4_t o = {0u, 0u, 0u, 0u};
-    if (c != 0.f) {
-      const float nc = -c, l2 = s_l2[r];
-      const int yrel = s_y[r] - cpos;                       // 0..7 when the target sits in this lane's piece
-      float d[8];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t w = v[ps][e];
-        const float x0 = __uint_as_float(w << 16), x1 = __uint_as_float(w & 0xffff0000u);
-        d[2 * e] = nc * fast_exp2(__builtin_fmaf(x0, xs, -l2));
-        d[2 * e + 1] = nc * fast_exp2(__builtin_fmaf(x1, xs, -l2));
-      }
-      if (yrel >= 0 && yrel < 8) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) d[e] += (e == yrel) ? c : 0.f;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(d[2 * e], d[2 * e + 1]);
-    }
-    __builtin_nontemporal_store(o, base + ps * 256);
-  }
+  if (ty == 0 && c < V) out_bf16[c] = f32_to_bf16_rn((red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]));
 }
 
 }  // namespace fgrpo

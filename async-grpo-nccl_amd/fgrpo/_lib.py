@@ -35,6 +35,7 @@ SIGNATURES = {
     "fgrpo_keep_supported": (_i, [_i, _i, _i, _i]),
     "fgrpo_logits_keep_bytes": (_sz, [_i, _i]),
     "fgrpo_logprob_fwd_keep": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp]),
+    "fgrpo_keep_overflowed": (_i, [_vp, _i, _i, _vp]),
     "fgrpo_lmhead_bwd_kept_workspace": (_sz, [_i, _i, _i, _i]),
     "fgrpo_lmhead_bwd_kept": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp,
                                    _vp, _sz, _vp]),

@@ -99,7 +99,7 @@ def lmhead_logprob_fwd(hidden: torch.Tensor, weight: torch.Tensor, bias: Optiona
                        want_entropy: bool = True, want_lse: bool = True, keep: bool = False):
     """hidden [T,H], weight [V,H] (same dtype, bf16 or fp32), labels_shifted [T] int64
     -> (lp [T] fp32, entropy [T] fp32 | None, lse [T] fp32 | None); with ``keep`` a fourth result, the uint8 buffer
-    holding the bf16 logits in the library's blocked layout, for ``lmhead_bwd_kept``."""
+    holding the bf16 soft-max numerators in the library's blocked layout, for ``lmhead_bwd_kept``."""
     dev = _require_cuda(hidden, weight, bias, labels_shifted)
     lib = _lib.load()
     if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
@@ -205,10 +205,21 @@ def lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torc
     return dH, dW, db
 
 
+def keep_overflowed(kept: torch.Tensor, T: int, V: int) -> bool:
+    """True when the forward flagged that the kept values may have overflowed (a scored token whose log-probability
+    is below -128): the caller must then take the recomputing backward.  Waits for the current stream."""
+    with torch.cuda.device(kept.device):
+        rc = _lib.load().fgrpo_keep_overflowed(_ptr(kept), int(T), int(V), _stream())
+    if rc < 0:
+        _lib.check(rc, "keep_overflowed")
+    return rc != 0
+
+
 def lmhead_bwd_kept(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torch.Tensor], temperature: float,
                     kept: torch.Tensor, need_dh: bool, need_dw: bool, need_db: bool):
-    """The backward on the logits the forward kept (``lmhead_logprob_fwd(..., keep=True)``): ``kept`` is turned into
-    dLogits in place (its contents are spent afterwards), then dH / dW / dbias come from one GEMM each."""
+    """The backward on the soft-max numerators the forward kept (``lmhead_logprob_fwd(..., keep=True)``): one
+    element per row of ``kept`` is patched in place, then dH / dW / dbias come from one GEMM each reading the buffer
+    as it lies.  The caller has checked ``keep_overflowed(kept, T, V)``."""
     dev = _require_cuda(hidden, weight, labels_shifted, lse, g, kept)
     lib = _lib.load()
     T, H = hidden.shape
@@ -228,7 +239,7 @@ def lmhead_bwd_kept(hidden, weight, bias, labels_shifted, lse, g, gout: Optional
     db = torch.empty(V, dtype=weight.dtype, device=dev) if (need_db and bias is not None) else None
     if not (need_dh or need_dw or db is not None):
         return dH, dW, db
-    ws = _ws(lib.fgrpo_lmhead_bwd_kept_workspace(T, H, V, code) if need_dh else 0, dev)
+    ws = _ws(lib.fgrpo_lmhead_bwd_kept_workspace(T, H, V, code), dev)
     with torch.cuda.device(dev):
         rc = lib.fgrpo_lmhead_bwd_kept(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(labels_shifted), _ptr(lse), _ptr(g),
                                        _ptr(gout), 1.0 / float(temperature), T, H, V, code,
@@ -594,6 +605,8 @@ def panel_elems_bound(T: int, V: int, loss_chunksize: Optional[int]) -> int:
 def _bwd_rows(h_used, weight, bias, y_used, lse, g_full, gout, temperature, need, panel_hint, idx, hidden_shape,
               kept=None):
     g_used = g_full if idx is None else g_full.reshape(-1).index_select(0, idx)
+    if kept is not None and keep_overflowed(kept, h_used.shape[0], weight.shape[0]):
+        kept = None                                # out of the kept values' range: recompute (exact for any input)
     if kept is not None:
         dH, dW, db = lmhead_bwd_kept(h_used, weight, bias, y_used, lse, g_used, gout, temperature, kept, need[0],
                                      need[1], need[2])
@@ -616,7 +629,7 @@ class _LMHeadLogprob(torch.autograd.Function):
                                                                needs_grad, keep_logits)
         ctx.save_for_backward(h_used, weight, bias if bias is not None else hidden.new_empty(0), y_used, lse,
                               idx if idx is not None else hidden.new_empty(0))
-        ctx.kept = kept       # consumed by the one backward (a second backward through this node recomputes)
+        ctx.kept = kept       # released by the first backward (a second backward through this node recomputes)
         ctx.has_bias = bias is not None
         ctx.compacted = idx is not None
         ctx.hidden_shape = tuple(hidden.shape)
@@ -648,7 +661,7 @@ class _FusedGRPOLoss(torch.autograd.Function):
         needs_grad = any(ctx.needs_input_grad[:3])
         lp, ent, lse, h_used, y_used, kept = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx,
                                                                needs_grad, keep_logits)
-        ctx.kept = kept       # consumed by the one backward (a second backward through this node recomputes)
+        ctx.kept = kept       # released by the first backward (a second backward through this node recomputes)
         loss, g, lr, c1, l1, l2, scal = grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
                                                       clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
                                                       denom_override)

@@ -326,7 +326,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check that precedes the timed steps")
     ap.add_argument("--keep-logits", choices=["auto", "on", "off"], default="auto",
-                    help="keep the bf16 logits for the backward (auto: when supported and memory allows) or recompute them")
+                    help="keep the [T x V] bf16 soft-max numerators for the backward (auto: when supported and memory allows) "
+                         "or recompute the logits there")
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed steps, run one 1 GiB device copy (reference point for traffic counters)")
     ap.add_argument("--seed", type=int, default=0)
@@ -452,12 +453,13 @@ def main():
         if note:
             d["note"] = note
         return d
-    phases = [phase("lmhead_fwd_kernel" + (" (keeps bf16 logits)" if kept else "") + " + combine", k_ms * args.steps, thv)]
+    phases = [phase("lmhead_fwd_kernel" + (" (keeps the bf16 soft-max numerators)" if kept else "") + " + combine",
+                    k_ms * args.steps, thv)]
     if not fwd_only:
         if kept:
-            phases.append(phase("kept_logits_to_dlogits_kernel", phase_ms["dlogits"], 0.0,
-                                f"HBM-bound: {4.0 * T * V / 1e9:.1f} GB per launch = "
-                                f"{4.0 * T * V / (phase_ms['dlogits'] / args.steps * 1e-3) / 1e12:.2f} TB/s"))
+            phases.append(phase("keep_backward_prep_kernel", phase_ms["dlogits"], 0.0,
+                                "per-token factors, one patched element per row, scaled copy of hidden "
+                                f"({4.0 * T * H / 1e6:.0f} MB): no pass over [T x V]"))
         else:
             phases.append(phase(f"lmhead_ds_kernel x {phase_n['dlogits'] // args.steps} panels (recomputes the logits)",
                                 phase_ms["dlogits"], thv, "executed, not algorithmic, work"))
@@ -474,7 +476,7 @@ def main():
                                f"{'forward only' if fwd_only else 'forward+backward (dHidden, dW)'}, "
                                f"{w.n_samples} samples, chunk hint {p['chunk']}",
                    "tokens": T, "hidden": H, "vocab": V, "samples": w.n_samples,
-                   "backward": None if fwd_only else ("bf16 logits kept for the backward" if kept else "logits recomputed in the backward"),
+                   "backward": None if fwd_only else ("bf16 soft-max numerators kept for the backward" if kept else "logits recomputed in the backward"),
                    "input_sets_rotated": len(sets)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS,

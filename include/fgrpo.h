@@ -99,19 +99,26 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
                      long long panel_elems_hint,
                      void* workspace, size_t workspace_bytes, void* stream);
 
-/* ---- the same forward / backward pair WITHOUT recomputation: the logits are kept --------------------------
+/* ---- the same forward / backward pair WITHOUT recomputation: the soft-max numerators are kept ---------------
  * The reference keeps every chunk's logits alive for autograd (grpo_loss.py:286-313: 9.96 GB of bf16 at T = 32768,
  * V = 151936) and its backward reads them back; fgrpo_lmhead_bwd instead recomputes them (a fourth [T x V x H]
- * product).  Where memory allows - 288 GB of HBM per MI355X - this pair does what the reference does:
- * fgrpo_logprob_fwd_keep is fgrpo_logprob_fwd that also writes x = W h + b (before the temperature, rounded to
- * bf16 exactly as the reference's bf16 logits are) into `logits_keep`, and fgrpo_lmhead_bwd_kept turns that buffer
- * IN PLACE into dLogits (one HBM-bound pass) and runs each gradient product as one launch over the whole
- * vocabulary: 6 instead of 8 T*H*V products per step, dH written once.  The workspace (T*H*4 bytes) is only
- * touched when the tuning key keep_panels splits the products into vocabulary panels (fp32 dH accumulator);
- * NULL is accepted otherwise.  lp / entropy / lse are computed from the fp32 accumulators and are bit-identical
- * to fgrpo_logprob_fwd's.
- * logits_keep: fgrpo_logits_keep_bytes(T, V) bytes, 16-byte aligned, laid out in 256-column blocks
- * [ceil(V/256)][round_up(T,256)][256] bf16; its contents after fgrpo_lmhead_bwd_kept are dLogits (not an output).
+ * product).  Where memory allows - 288 GB of HBM per MI355X - this pair keeps a [T x V] bf16 matrix as the
+ * reference does, in the form the backward needs: fgrpo_logprob_fwd_keep is fgrpo_logprob_fwd that also writes
+ *   E[t, v] = exp(x_tv / temperature - ref_t),   ref_t = x_t[y_t] / temperature + 40,
+ * the exponential its statistics compute anyway, re-based on a per-token reference fixed before the sweep (a dot
+ * product per token).  The probability is E[t, v] * exp(ref_t - lse_t), so dLogits = diag(a) E' with one factor
+ * a_t per token and E' = E but for the target's element of each row, which fgrpo_lmhead_bwd_kept patches in place:
+ * no pass over [T x V] is needed and the two gradient products read the buffer as it lies (dH = diag(a) E' W with
+ * the factor in the epilogue, dW = E'^T (diag(a) hidden)): 6 instead of 8 T*H*V products per step.  The buffer
+ * survives the backward (a second backward may reuse it).  lp / entropy / lse are computed as in
+ * fgrpo_logprob_fwd and are bit-identical to its results.
+ * Range: E holds p_v / p_y * exp(-40) in bf16, finite as long as log p_y > -128 for every scored token; the
+ * forward raises a flag in the buffer otherwise, fgrpo_keep_overflowed() reads it (it waits for `stream`), and the
+ * caller must then use fgrpo_lmhead_bwd.  Rows of ignored tokens are stored as exact zeros.
+ * logits_keep: fgrpo_logits_keep_bytes(T, V) bytes, 16-byte aligned: [ceil(V/256)][round_up(T,256)][256] bf16,
+ * then the references and the flag.  workspace of the backward: fgrpo_lmhead_bwd_kept_workspace bytes (the token
+ * factors, the scaled copy of hidden, and an fp32 dH accumulator used only when the tuning key keep_panels splits
+ * the products into vocabulary panels).
  * Supported (fgrpo_keep_supported() != 0): bf16, H a multiple of 256, enough tiles to fill the device; anything
  * else returns FGRPO_ERR_UNSUPPORTED - use the recomputing pair.  dH_out / dW_out / dbias_out as in
  * fgrpo_lmhead_bwd. */
@@ -123,6 +130,9 @@ int fgrpo_logprob_fwd_keep(const void* hidden, const void* weight, const void* b
                            float* lp_out, float* ent_out, float* lse_out,
                            void* logits_keep, size_t logits_keep_bytes,
                            void* workspace, size_t workspace_bytes, void* stream);
+/* 1 when the kept values may have overflowed (use fgrpo_lmhead_bwd), 0 when they are good, negative on error.
+ * Synchronises `stream`. */
+int fgrpo_keep_overflowed(const void* logits_keep, int T, int V, void* stream);
 size_t fgrpo_lmhead_bwd_kept_workspace(int T, int H, int V, int dtype);
 int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bias,
                           const int64_t* labels_shifted, const float* lse, const float* g,

@@ -1,5 +1,6 @@
-"""The forward/backward pair that keeps the bf16 logits (as the reference's autograd does, grpo_loss.py:286-313)
-instead of recomputing them, and the whole path at the full benchmark sizes through the drop-in's own entry point.
+"""The forward/backward pair that keeps a [T x V] bf16 matrix for the backward (as the reference's autograd keeps
+its logits, grpo_loss.py:286-313) instead of recomputing the logits - here the soft-max numerators against a
+per-token reference - and the whole path at the full benchmark sizes through the drop-in's own entry point.
 
 Small device-filling shapes are compared with the CPU oracle outright.  At the full sizes the oracle cannot form
 [T x V] in seconds: the per-token logprobs (pinned against sampled oracle rows in test_gpu_parity) feed the oracle's
@@ -41,8 +42,9 @@ def test_kept_logits_with_bias_and_temperature(dev):
 
 
 def test_kept_forward_is_bit_identical_and_backward_close_to_recompute(dev):
-    """Keeping the logits changes nothing in the forward (statistics come from the fp32 accumulators either way);
-    the backward differs from the recomputing one only by the bf16 rounding of the kept logits."""
+    """Keeping the numerators changes nothing in the forward (statistics come from the fp32 accumulators either
+    way); the backward differs from the recomputing one only by bf16 rounding (of the kept values there, of
+    dLogits here)."""
     from fgrpo import ops
     w = filling_workload(13, tokens=8192 + 64)           # token count past a multiple of 256
     hs, W = w.hidden.reshape(w.T, w.H).to(dev), w.weight.to(dev)
@@ -75,7 +77,6 @@ def test_kept_logits_panel_split_matches_single_launch(dev):
     g = torch.randn(w.T, generator=torch.Generator().manual_seed(3)).to(dev) / w.T
     lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
     dH1, dW1, _ = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
-    kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)[3]
     _lib.set_tuning(keep_panels=3)
     try:
         dH3, dW3, _ = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
@@ -83,6 +84,53 @@ def test_kept_logits_panel_split_matches_single_launch(dev):
         _lib.set_tuning(keep_panels=0)
     assert torch.equal(dW1, dW3)
     assert cos(dH1, dH3) >= 0.99999
+
+
+def test_kept_values_out_of_range_fall_back_to_recomputation(dev):
+    """The kept numerators are exp(x_v - x_target - 40) in bf16: a scored token whose log-probability is below
+    -128 would overflow them.  The forward flags it, and the backward then recomputes: same gradients, bit for
+    bit, as with keep_logits=False; the forward's own outputs never depend on the kept values."""
+    from fgrpo import ops
+    T, H, V = 8192, 1024, 8192
+    gen = torch.Generator().manual_seed(21)
+    hs = torch.ones(T, H).bfloat16()
+    W = (torch.randn(V, H, generator=gen) * 0.01).bfloat16()
+    W[7] = 0.25                                        # logit 256 for entry 7 on every row; the targets sit near 0
+    y = torch.randint(8, V, (T,), generator=gen)
+    adv = torch.randn(T, generator=gen)
+    hs_d, W_d, y_d, adv_d = hs.to(dev), W.to(dev), y.to(dev), adv.to(dev)
+    lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs_d, W_d, None, y_d, 1.0, keep=True)
+    assert ops.keep_overflowed(kept, T, V)
+    assert (lp < -128).all() and torch.isfinite(lp).all() and torch.isfinite(lse).all()
+    grads = []
+    for keep in (True, False):
+        h = hs_d.clone().requires_grad_(True)
+        w = W_d.clone().requires_grad_(True)
+        out = ops.fused_grpo_loss(h, w, None, y_d, None, adv_d, keep_logits=keep)
+        out[0].backward()
+        grads.append((h.grad, w.grad, out[0].detach()))
+    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
+    assert torch.equal(grads[0][2], grads[1][2]) and torch.isfinite(grads[0][1].float()).all()
+    # and an ordinary batch does not raise the flag
+    W2 = (torch.randn(V, H, generator=gen) * 0.05).bfloat16().to(dev)
+    kept2 = ops.lmhead_logprob_fwd(torch.randn(T, H, generator=gen).bfloat16().to(dev), W2, None, y_d, 1.0, keep=True)[3]
+    assert not ops.keep_overflowed(kept2, T, V)
+
+
+def test_kept_buffer_survives_the_backward(dev):
+    """The backward patches one element per row with a value computed from scratch and otherwise only reads the
+    buffer: running it twice on the same buffer gives the same gradients."""
+    from fgrpo import ops
+    w = filling_workload(15)
+    hs, W = w.hidden.reshape(w.T, w.H).to(dev), w.weight.to(dev)
+    y = ops.shift_labels(w.labels.to(dev)).reshape(-1)
+    g = torch.randn(w.T, generator=torch.Generator().manual_seed(4)).to(dev) / w.T
+    lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
+    a = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
+    b = ops.lmhead_bwd_kept(hs, W, None, y, lse, 2 * g, None, 1.0, kept, True, True, False)
+    c = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
+    assert torch.equal(a[0], c[0]) and torch.equal(a[1], c[1])
+    assert cos(b[0], a[0]) >= 0.99999 and abs(b[1].float().norm().item() / a[1].float().norm().item() - 2.0) < 1e-2
 
 
 def test_keep_refuses_what_it_cannot_do(dev):
