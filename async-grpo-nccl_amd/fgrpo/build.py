@@ -18,8 +18,10 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(HERE), "csrc")
 LIB_PATH = os.environ.get("FGRPO_LIB", os.path.join(CSRC, "libfgrpo.so"))
-USAGE_PATH = os.path.join(CSRC, "resource_usage.json")
-OBJ_DIR = os.path.join(CSRC, "build")
+# an alternative output (FGRPO_LIB, for side-by-side builds) keeps its own objects and report
+_ALT = "" if LIB_PATH == os.path.join(CSRC, "libfgrpo.so") else "_" + os.path.splitext(os.path.basename(LIB_PATH))[0]
+USAGE_PATH = os.path.join(CSRC, f"resource_usage{_ALT}.json")
+OBJ_DIR = os.path.join(CSRC, "build" + _ALT)
 
 SOURCES = ["fgrpo_api.hip", "launch_lmhead.hip", "launch_gemm.hip", "launch_attn.hip"]
 

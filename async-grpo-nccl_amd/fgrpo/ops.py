@@ -537,8 +537,14 @@ COMPACT_MIN_TOKENS = 2048
 COMPACT_MAX_VALID_FRACTION = 0.9
 
 
-def _valid_rows(labels_shifted: torch.Tensor, compact: bool):
+def _valid_rows(labels_shifted: torch.Tensor, compact):
+    """Row indices the projection runs on, or None for all rows.  ``compact`` is False, True (find the rows whose
+    shifted label is valid: one host sync for their number) or an int64 tensor that already lists them in
+    ascending order (no sync; the caller vouches that it holds exactly the positions with a valid label)."""
     T = labels_shifted.numel()
+    if torch.is_tensor(compact):
+        idx = compact.reshape(-1).to(device=labels_shifted.device, dtype=torch.int64)
+        return idx if 0 < idx.numel() < T else None
     if not compact or T < COMPACT_MIN_TOKENS:
         return None
     mask = labels_shifted.reshape(-1) != -100
@@ -718,7 +724,7 @@ def grpo_loss_from_logprobs(lp, labels_shifted, old_lp, adv, ref_lp=None, cu_seq
 
 def lmhead_logprob(hidden, weight, bias, labels_shifted, temperature=1.0, panel_hint=0,
                    compact=False, keep_logits=None) -> Tuple[torch.Tensor, torch.Tensor]:
-    return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint), bool(compact),
+    return _LMHeadLogprob.apply(hidden, weight, bias, labels_shifted, float(temperature), int(panel_hint), compact if torch.is_tensor(compact) else bool(compact),
                                 keep_logits)
 
 
@@ -729,8 +735,8 @@ def fused_grpo_loss(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp=No
     ``keep_logits``: None = the module default (``KEEP_LOGITS``), True / False / "auto"."""
     return _FusedGRPOLoss.apply(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens,
                                 float(temperature), float(clip_low), float(clip_high), float(clip_ratio_c),
-                                float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint), bool(compact),
-                                keep_logits)
+                                float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint),
+                                compact if torch.is_tensor(compact) else bool(compact), keep_logits)
 
 
 # --------------------------------------------------------------------------- packed variable-length attention

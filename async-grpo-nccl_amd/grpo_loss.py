@@ -210,7 +210,7 @@ def fused_log_probs_and_entropy_fn(
                                                    per_token_fn, None)
     shifted = ops.shift_labels(labels).reshape(-1)
     lp, ent = ops.lmhead_logprob(hs, w, b, shifted, temperature,
-                                 compact=bool(unused_kwargs.get("compact_masked_tokens", False)),
+                                 compact=unused_kwargs.get("compact_masked_tokens", False),
                                  keep_logits=unused_kwargs.get("keep_logits", None))
     return lp, ent
 
@@ -256,7 +256,7 @@ def grpo_loss_and_entropy_ce_fn(
     loss_agg_mode = unused_kwargs.get("loss_agg_mode", "token_mean")
     cu_seqlens = unused_kwargs.get("cu_seqlens", None)
     num_samples_total = unused_kwargs.get("num_samples_total", None)
-    compact = bool(unused_kwargs.get("compact_masked_tokens", False))
+    compact = unused_kwargs.get("compact_masked_tokens", False)      # True / False, or the int64 row indices themselves
 
     shifted = ops.shift_labels(labels).reshape(-1)
     w, b, hs = _prep(lm_head_weights, lm_head_bias, hidden_states)
@@ -414,8 +414,12 @@ def compute_dual_clip_grpo_loss(
     # Shapes alone (no sync) tell when prompts are a sizeable part of the batch: output_indices lists exactly the
     # positions whose shifted label is valid (sample_processing_utils.py:29-67).  The LM head then skips the rest.
     extra = {}
-    if 0 < int(output_indices.numel()) < ops.COMPACT_MAX_VALID_FRACTION * int(labels.numel()):
-        extra["compact_masked_tokens"] = True
+    if ops.COMPACT_MIN_TOKENS <= int(labels.numel()) and \
+            0 < int(output_indices.numel()) < ops.COMPACT_MAX_VALID_FRACTION * int(labels.numel()):
+        # output_indices are the rows themselves when every labelled token is an output token (their host-side
+        # counts agree): nothing to count on the device then; otherwise the rows are found from the labels
+        n_host = minibatch.get("_num_output_tokens_non_masked_host", None)
+        extra["compact_masked_tokens"] = output_indices if (n_host is not None and int(n_host) == int(output_indices.numel())) else True
     grpo_output = policy_model(
         input_ids=batch_ids,
         attention_mask=minibatch.get("attention_mask", None),
@@ -438,8 +442,15 @@ def compute_dual_clip_grpo_loss(
         stats_dev = ops.grpo_metrics(output_indices, grpo_output.neg_log_ratio, grpo_output.entropy, old_entropy,
                                      advantages, grpo_output.loss_unclipped, grpo_output.loss_clipped,
                                      clip_low, clip_high)
-        host = torch.cat([stats_dev, grpo_output.loss.detach().double().reshape(1)]).cpu().tolist()
-    st, loss_sum = host[:-1], float(host[-1])
+        # the one device-to-host copy of this function: diagnostics, loss value and the batch's sample count
+        num_samples_tensor = minibatch.get("num_samples", None)
+        tail = [grpo_output.loss.detach().double().reshape(1)]
+        if torch.is_tensor(num_samples_tensor):
+            tail.append(num_samples_tensor.detach().double().reshape(1).to(stats_dev.device))
+        host = torch.cat([stats_dev] + tail).cpu().tolist()
+    st, loss_sum = host[:ops._lib.NUM_STATS], float(host[ops._lib.NUM_STATS])
+    num_samples = int(host[ops._lib.NUM_STATS + 1]) if len(host) > ops._lib.NUM_STATS + 1 else \
+        (int(num_samples_tensor) if num_samples_tensor is not None else 0)
     n = st[0]
     mean = (lambda s: s / n) if n > 0 else (lambda s: 0.0)
 
@@ -450,11 +461,6 @@ def compute_dual_clip_grpo_loss(
         return max(s2 / n - m * m, 0.0) ** 0.5
 
     expected_out = int(output_indices.numel())
-    try:
-        num_samples_tensor = minibatch.get("num_samples", None)
-        num_samples = int(num_samples_tensor.item()) if num_samples_tensor is not None else 0
-    except Exception:
-        num_samples = 0
 
     metrics = {
         "loss": loss_sum,

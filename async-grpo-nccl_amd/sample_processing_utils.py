@@ -18,6 +18,75 @@ import torch
 from fgrpo import ops
 
 
+class PackedLogProbs:
+    """Wire format of the logprob worker's result: ONE pinned fp32 host buffer ``[2, T]`` (row 0 per-token
+    logprobs, row 1 per-token entropies; row 1 is absent, ``[1, T]``, when no entropies were produced) plus int32
+    ``offsets [n + 1]`` into it, sample i owning ``offsets[i]:offsets[i+1]``.  The reference ships a Python list of
+    floats per sample instead (gpu_process_worker.py:1694-1703), stores the lists on the samples
+    (logprob_worker.py:112-121) and re-tensors them in the trainer (sample_processing_utils.py:180-193).
+    ``attach`` puts views of the buffer on the samples; ``post_process_batch`` recognises samples that are
+    consecutive slices of one buffer and moves them with a single copy, no per-sample loop."""
+
+    def __init__(self, buffer: torch.Tensor, offsets):
+        if buffer.dim() != 2 or buffer.shape[0] not in (1, 2) or buffer.dtype != torch.float32 or buffer.is_cuda:
+            raise ValueError("PackedLogProbs: buffer must be a host fp32 tensor [1 or 2, T]")
+        self.buffer = buffer
+        self.offsets = np.ascontiguousarray(np.asarray(offsets, dtype=np.int32))
+        if self.offsets.ndim != 1 or self.offsets.size < 1 or int(self.offsets[-1]) != buffer.shape[1] or \
+                (np.diff(self.offsets) < 0).any() or int(self.offsets[0]) != 0:
+            raise ValueError("PackedLogProbs: offsets must rise from 0 to the buffer's length")
+
+    def __len__(self) -> int:
+        return self.offsets.size - 1
+
+    @property
+    def has_entropies(self) -> bool:
+        return self.buffer.shape[0] == 2
+
+    def sample(self, i: int):
+        """(logprobs view, entropies view | None) of sample i, numpy views of the buffer."""
+        a, b = int(self.offsets[i]), int(self.offsets[i + 1])
+        view = self.buffer.numpy()
+        return view[0, a:b], (view[1, a:b] if self.has_entropies else None)
+
+    def to_lists(self) -> List[dict]:
+        """The reference's list form (gpu_process_worker.py:1694-1703)."""
+        out = []
+        for i in range(len(self)):
+            lp, ent = self.sample(i)
+            out.append({"logprobs": lp.tolist(), "entropies": ent.tolist() if ent is not None else None})
+        return out
+
+    def attach(self, samples: list) -> None:
+        """What the controller does with the worker's result (logprob_worker.py:112-121), on views: sample i gets
+        ``sample_logprobs`` / ``sample_entropies`` and a note of where in which buffer they live."""
+        if len(samples) != len(self):
+            raise ValueError(f"PackedLogProbs: {len(self)} results for {len(samples)} samples")
+        for i, s in enumerate(samples):
+            lp, ent = self.sample(i)
+            s["sample_logprobs"] = lp
+            s["sample_entropies"] = ent
+            s["_packed_logprobs"] = (self, i)
+
+
+def _packed_run(batched_questions):
+    """(PackedLogProbs, first, last + 1) when the samples are consecutive entries of one packed result whose views
+    they still carry, else None."""
+    first = batched_questions[0].get("_packed_logprobs") if batched_questions else None
+    if first is None:
+        return None
+    packed, i0 = first
+    for k, s in enumerate(batched_questions):
+        ref = s.get("_packed_logprobs")
+        if ref is None or ref[0] is not packed or ref[1] != i0 + k:
+            return None
+        lp = s.get("sample_logprobs")
+        a, b = int(packed.offsets[i0 + k]), int(packed.offsets[i0 + k + 1])
+        if not isinstance(lp, np.ndarray) or lp.size != b - a or (lp.size and not np.shares_memory(lp, packed.buffer.numpy())):
+            return None                           # the field was replaced after attach: take the general route
+    return packed, i0, i0 + len(batched_questions)
+
+
 def _fill(dst: np.ndarray, batched_questions, key: str, lens, default=None) -> None:
     """Writes the per-token values ``s[key]`` of every sample into consecutive pieces of ``dst`` (a numpy view of
     the staging buffer).  Python lists go through ``np.fromiter`` (about half the cost of ``torch.as_tensor`` per
@@ -80,10 +149,12 @@ def get_input_for_logprobs(batched_questions, output_indices, device):
     _fill(view[1], batched_questions, "sample_position_ids", lens)
     if have_labels:
         _fill(view[2], batched_questions, "labels", lens)
+        get_input_for_logprobs.last_scored = int(np.count_nonzero(view[2] != -100))
     dev = host.to(device, non_blocking=True)
     if have_labels:
         return dev[0:1], dev[1:2], dev[2:3]
     il, ol = _lens(batched_questions)
+    get_input_for_logprobs.last_scored = int(ol.sum())
     return dev[0:1], dev[1:2], ops.build_labels(dev[0:1], il, ol)
 
 
@@ -129,15 +200,25 @@ def post_process_batch(batched_questions, device, constant_length_samples=None):
     else:
         output_lens_broadcasted = torch.full((total,), float(constant_length_samples), device=device, dtype=torch.float32)
 
-    # old-policy logprobs and entropies (zeros where a sample carries none): one pinned buffer, one copy
-    lp_lens = [len(s["sample_logprobs"]) for s in batched_questions]
-    n_lp = sum(lp_lens)
-    stage = torch.empty((2, n_lp), dtype=torch.float32).pin_memory() if n_lp else torch.empty((2, 0), dtype=torch.float32)
-    sv = stage.numpy()
-    _fill(sv[0], batched_questions, "sample_logprobs", lp_lens)
-    _fill(sv[1], batched_questions, "sample_entropies", lp_lens, default=0.0)
-    stage_dev = stage.to(device, non_blocking=True)
-    reference_output_logprobs, reference_output_entropies = stage_dev[0], stage_dev[1]
+    # old-policy logprobs and entropies (zeros where a sample carries none)
+    run = _packed_run(batched_questions)
+    if run is not None:
+        # consecutive slices of one pinned result buffer: one copy of the column range, no per-sample work
+        packed, i0, i1 = run
+        a, b = int(packed.offsets[i0]), int(packed.offsets[i1])
+        stage_dev = packed.buffer[:, a:b].to(device, non_blocking=True)
+        reference_output_logprobs = stage_dev[0]
+        reference_output_entropies = stage_dev[1] if packed.has_entropies else torch.zeros_like(stage_dev[0])
+    else:
+        # lists (the reference's form) or loose arrays: one pinned staging buffer, one copy
+        lp_lens = [len(s["sample_logprobs"]) for s in batched_questions]
+        n_lp = sum(lp_lens)
+        stage = torch.empty((2, n_lp), dtype=torch.float32).pin_memory() if n_lp else torch.empty((2, 0), dtype=torch.float32)
+        sv = stage.numpy()
+        _fill(sv[0], batched_questions, "sample_logprobs", lp_lens)
+        _fill(sv[1], batched_questions, "sample_entropies", lp_lens, default=0.0)
+        stage_dev = stage.to(device, non_blocking=True)
+        reference_output_logprobs, reference_output_entropies = stage_dev[0], stage_dev[1]
 
     batch_ids, batch_position_ids, labels = get_input_for_logprobs(batched_questions, output_indices, device)
 
@@ -170,6 +251,9 @@ def post_process_batch(batched_questions, device, constant_length_samples=None):
         "labels": labels.contiguous(),
         # not in the reference: segment boundaries, so that the loss can aggregate per sample
         "cu_seqlens": cu,
+        # not in the reference: the labelled-token count as a host integer (known while the labels are packed), so
+        # that the trainer's all-masked check needs no device read
+        "_num_output_tokens_non_masked_host": float(get_input_for_logprobs.last_scored),
     }
     for k, key in enumerate(counters):
         out[key] = counter_vec[k]

@@ -15,7 +15,7 @@ import numpy as np
 import torch
 
 from grpo_loss import compute_dual_clip_grpo_loss, make_grpo_forward
-from sample_processing_utils import _fill, post_process_batch
+from sample_processing_utils import PackedLogProbs, _fill, post_process_batch
 
 
 def prepare_actor_module(model, config=None, mode: str = "training", use_varlen_attention: bool = True):
@@ -47,7 +47,11 @@ class TrainerHarness:
         self.actor_module_fsdp.train()
         batch = post_process_batch(worker_batch, self.device)
         # single GPU: an all-masked batch contributes nothing (gpu_process_worker.py:979-985)
-        if self.fsdp_world_size == 1 and float(batch["num_output_tokens_non_masked"].item()) == 0:
+        # (the count is known on the host from packing the labels; the device scalar is only read when it is not)
+        n_scored = batch.get("_num_output_tokens_non_masked_host")
+        if n_scored is None:
+            n_scored = float(batch["num_output_tokens_non_masked"].item())
+        if self.fsdp_world_size == 1 and n_scored == 0:
             return {"loss": 0.0, "pg_clip": 0, "kl_div": 0.0, "entropy": 0.0}
         cfg = self.config
         with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
@@ -59,10 +63,11 @@ class TrainerHarness:
         # n_real / (minibatch_target // world) before backward (gpu_process_worker.py:1006-1025)
         n_real = sum(1 for s in worker_batch if not s.get("dummy", False))
         target = int(getattr(cfg, "train_minibatch_sample_size", 0) or 0)
-        if self.fsdp_world_size > 0:
-            target = max(1, target // self.fsdp_world_size) if target else 0
-        if target > 0 and n_real != target:
-            loss = loss * (float(n_real) / float(target))
+        if self.fsdp_world_size and self.fsdp_world_size > 0:
+            target = max(1, target // self.fsdp_world_size)          # an unset target of 0 becomes 1, as in the reference
+        scale = float(n_real) / float(target) if target > 0 else 1.0
+        if scale != 1.0:
+            loss = loss * scale
         loss.backward()
         self._mb_count_since_last_step += 1
         return metrics
@@ -76,11 +81,16 @@ class LogProbHarness:
         self.device = torch.device(device)
 
     @torch.no_grad()
-    def compute_log_probs_from_samples(self, samples: list) -> List[dict]:
+    def compute_log_probs_from_samples(self, samples: list, packed: bool = False):
+        """Per-sample logprobs and entropies of ``samples`` (dicts with ``sample_ids`` and ``labels``).
+        Default: the reference's result, a list of ``{"logprobs": [float], "entropies": [float] | None}``
+        (gpu_process_worker.py:1694-1703).  ``packed=True``: a ``PackedLogProbs`` - one pinned fp32 buffer
+        ``[2, T]`` filled by a single device-to-host copy, plus int32 offsets - whose ``to_lists()`` equals the
+        default result bit for bit and which ``post_process_batch`` takes without a per-sample loop."""
         self.actor_module_fsdp.eval()
         lens = [len(s["sample_ids"]) for s in samples]
         total = sum(lens)
-        host = torch.empty((3, total), dtype=torch.long)
+        host = torch.empty((3, total), dtype=torch.long).pin_memory() if total else torch.empty((3, 0), dtype=torch.long)
         view = host.numpy()
         _fill(view[0], samples, "sample_ids", lens)
         _fill(view[2], samples, "labels", lens, default=-100)
@@ -88,15 +98,15 @@ class LogProbHarness:
         for k in lens:
             view[1, off:off + k] = np.arange(k)
             off += k
-        dev = host.to(self.device)
+        dev = host.to(self.device, non_blocking=True)
         out = self.actor_module_fsdp(input_ids=dev[0:1], attention_mask=None, position_ids=dev[1:2], labels=dev[2:3])
-        # one device->host copy for the whole batch, then split on the host
-        lp = out.loss.detach().float().cpu()
+        # one device->host copy for the whole batch into one pinned buffer
         ent = getattr(out, "entropy", None)
-        ent = ent.detach().float().cpu() if ent is not None else None
-        res, off = [], 0
-        for k in lens:
-            res.append({"logprobs": lp[off:off + k].tolist(),
-                        "entropies": ent[off:off + k].tolist() if ent is not None else None})
-            off += k
-        return res
+        rows = 2 if ent is not None else 1
+        buf = torch.empty((rows, total), dtype=torch.float32).pin_memory() if total else torch.empty((rows, 0), dtype=torch.float32)
+        stacked = out.loss.detach().float().reshape(1, -1) if ent is None else \
+            torch.stack((out.loss.detach().float().reshape(-1), ent.detach().float().reshape(-1)))
+        buf.copy_(stacked, non_blocking=True)
+        torch.cuda.current_stream(self.device).synchronize()
+        result = PackedLogProbs(buf, np.concatenate(([0], np.cumsum(lens))))
+        return result if packed else result.to_lists()

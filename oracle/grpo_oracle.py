@@ -383,10 +383,16 @@ def pack_samples(samples: List[dict]) -> Dict[str, torch.Tensor]:
 
 
 def scale_microbatch_loss(loss, num_real_samples: int, train_minibatch_sample_size: int, world: int = 1):
-    """loss * n_real / (minibatch_target // world).  Reference:
-    gpu_process_worker.py:1006-1025."""
-    local_target = max(1, int(train_minibatch_sample_size) // max(world, 1)) if train_minibatch_sample_size else 0
-    return loss * (float(num_real_samples) / float(local_target)) if local_target > 0 else loss
+    """loss * n_real / local_target with local_target = max(1, minibatch_target // world) when world > 0 (so an
+    unset target of 0 becomes 1 and the loss is scaled by n_real), the plain target when world is 0, and no scaling
+    when that leaves 0.  Reference: gpu_process_worker.py:1006-1025."""
+    local_target = int(train_minibatch_sample_size or 0)
+    if world and world > 0:
+        local_target = max(1, local_target // world)
+    if local_target <= 0:
+        return loss
+    scale = float(num_real_samples) / float(local_target)
+    return loss * scale if scale != 1.0 else loss
 
 
 def split_logprobs_per_sample(flat_lp: torch.Tensor, flat_ent: Optional[torch.Tensor], lens: Sequence[int]):

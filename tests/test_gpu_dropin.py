@@ -51,7 +51,8 @@ def make_samples(n=6, V=512, seed=0):
                             input_len=li, output_len=lo, advantage=float(rng.normal()),
                             sample_logprobs=(-rng.random(li + lo) * 0.2 - math.log(V)).tolist(),
                             sample_entropies=(rng.random(li + lo) + 5).tolist() if i % 2 == 0 else None,
-                            reward=float(i % 2), modified_reward=None, delimiter_not_found=False,
+                            reward=float(i % 2), modified_reward=(0.25 * i - 0.5 if i % 3 == 1 else None),
+                            delimiter_not_found=bool(i % 2 == 1),
                             truncated_sample=bool(i % 3 == 0), __uid__=100 + i))
     return samples
 
@@ -67,6 +68,9 @@ def test_post_process_batch_matches_oracle(dev):
         assert g.dtype == v.dtype and g.shape == v.shape, k
         assert torch.equal(g, v), k
     assert got["uids"].tolist() == [100 + i for i in range(len(samples))]
+    # samples 1 and 4 carry a modified reward (sample_processing_utils.py:167-168, 209-212)
+    assert got["num_modified_samples"].item() == 2.0 and got["total_modified_reward"].item() == (-0.25) + 0.5
+    assert got["delimiter_not_found"].item() == 1.0 and got["total_non_modified_reward"].item() == 0.0 + 0.0 + 1.0 + 1.0
     cu = got["cu_seqlens"].cpu()
     assert torch.equal(cu, O.cu_seqlens_from_position_ids(want["batch_position_ids"]))
     const = spu.post_process_batch(samples, dev, constant_length_samples=7)
@@ -268,6 +272,45 @@ def test_eval_forward_and_logprob_worker(dev):
         G.make_grpo_forward(TinyLM().to(dev), mode="bogus").forward(input_ids=ids.to(dev), position_ids=pos.to(dev), labels=labels.to(dev))
 
 
+def test_packed_logprob_wire_format_round_trip(dev):
+    """compute_log_probs_from_samples(packed=True): one pinned fp32 buffer [2, T] + int32 offsets.  Its list form
+    equals the default result bit for bit, and post_process_batch builds the same batch from attached views (one
+    copy of a column range) as from the lists (per-sample conversion) - also for a sub-run of the samples, and it
+    falls back to the general route when the samples are not consecutive slices of one buffer."""
+    import sample_processing_utils as spu
+    from workers import LogProbHarness
+    model, G = _patched(dev, "eval", temperature=0.9)
+    samples = make_samples(7, seed=11)
+    h = LogProbHarness(model, dev)
+    lists = h.compute_log_probs_from_samples(samples)
+    packed = h.compute_log_probs_from_samples(samples, packed=True)
+    assert isinstance(packed, spu.PackedLogProbs) and len(packed) == 7 and packed.has_entropies
+    assert packed.buffer.is_pinned() and packed.buffer.dtype == torch.float32 and packed.buffer.shape[0] == 2
+    assert packed.offsets.dtype == np.int32 and packed.offsets.tolist() == np.concatenate(([0], np.cumsum([len(s["sample_ids"]) for s in samples]))).tolist()
+    assert packed.to_lists() == lists                                   # bit for bit: float lists compare exactly
+
+    a = [dict(s) for s in samples]
+    for s, r in zip(a, lists):                                          # what the reference's controller stores
+        s["sample_logprobs"], s["sample_entropies"] = r["logprobs"], r["entropies"]
+    b = [dict(s) for s in samples]
+    packed.attach(b)
+    for sub in (slice(0, 7), slice(2, 6)):
+        from_lists = spu.post_process_batch(a[sub], dev)
+        from_packed = spu.post_process_batch(b[sub], dev)
+        assert spu._packed_run(b[sub]) is not None
+        for k, v in from_lists.items():
+            if torch.is_tensor(v):
+                assert torch.equal(v, from_packed[k]), k
+    shuffled = [b[3], b[1], b[2]]
+    assert spu._packed_run(shuffled) is None
+    got = spu.post_process_batch(shuffled, dev)
+    want = spu.post_process_batch([a[3], a[1], a[2]], dev)
+    assert torch.equal(got["reference_output_logprobs"], want["reference_output_logprobs"])
+    assert torch.equal(got["reference_output_entropies"], want["reference_output_entropies"])
+    b[4]["sample_logprobs"] = list(b[4]["sample_logprobs"])            # replaced after attach: general route again
+    assert spu._packed_run(b[3:6]) is None
+
+
 @pytest.mark.parametrize("entropy_coeff", [0.0, 0.01])
 def test_training_forward_metrics_and_backward(dev, entropy_coeff):
     import sample_processing_utils as spu
@@ -344,6 +387,13 @@ def test_trainer_harness_scaling_and_dummy(dev):
     g2 = model.model.proj.weight.grad.clone()
     ratio = (g1.float().norm() / g2.float().norm()).item()
     assert abs(ratio - 0.25) < 0.02
+    # an unset target becomes max(1, 0 // world) = 1: the loss is scaled by the number of real samples
+    # (gpu_process_worker.py:1013-1020)
+    model.zero_grad()
+    cfg.train_minibatch_sample_size = 0
+    tr.compute_gradients(samples, 0)
+    g3 = model.model.proj.weight.grad.clone()
+    assert abs((g3.float().norm() / g2.float().norm()).item() - 4.0) < 0.3
     assert tr.compute_gradients([{"dummy": True}], 0) == {"loss": 0.0, "pg_clip": 0, "kl_div": 0.0, "entropy": 0.0}
 
 

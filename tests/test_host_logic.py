@@ -126,3 +126,29 @@ def test_product_modules_never_import_the_oracle():
             if f.endswith((".py", ".h", ".hip")):
                 text = open(os.path.join(dirpath, f), encoding="utf-8").read()
                 assert "oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_packed_logprobs_container():
+    """The wire format of the logprob worker's result on the host side: validation, views, list form."""
+    import sample_processing_utils as spu
+    buf = torch.arange(12, dtype=torch.float32).reshape(2, 6)
+    p = spu.PackedLogProbs(buf, [0, 2, 2, 6])
+    assert len(p) == 3 and p.has_entropies and p.offsets.dtype == np.int32
+    lp, ent = p.sample(2)
+    assert lp.tolist() == [2.0, 3.0, 4.0, 5.0] and ent.tolist() == [8.0, 9.0, 10.0, 11.0]
+    assert np.shares_memory(lp, buf.numpy())
+    assert p.to_lists() == [{"logprobs": [0.0, 1.0], "entropies": [6.0, 7.0]}, {"logprobs": [], "entropies": []},
+                            {"logprobs": [2.0, 3.0, 4.0, 5.0], "entropies": [8.0, 9.0, 10.0, 11.0]}]
+    only_lp = spu.PackedLogProbs(buf[:1], [0, 6])
+    assert not only_lp.has_entropies and only_lp.to_lists() == [{"logprobs": [0.0, 1.0, 2.0, 3.0, 4.0, 5.0], "entropies": None}]
+    samples = [{}, {}, {}]
+    p.attach(samples)
+    assert spu._packed_run(samples) == (p, 0, 3) and spu._packed_run(samples[1:]) == (p, 1, 3)
+    assert spu._packed_run([samples[2], samples[0]]) is None and spu._packed_run([{}]) is None
+    for bad in ([0, 7], [1, 6], [0, 4, 3, 6]):
+        with pytest.raises(ValueError):
+            spu.PackedLogProbs(buf, bad)
+    with pytest.raises(ValueError):
+        spu.PackedLogProbs(buf.double(), [0, 6])
+    with pytest.raises(ValueError):
+        p.attach([{}])

@@ -249,6 +249,14 @@ def test_metrics_hand_computed():
     # clipped > unclipped: A=-2, r<0.8 -> clipped = 1.6 > unclipped = 1.21 -> 1 hit
     assert m["pg_clip"] == 1.0
     assert m["loss_per_token"] == 0.25 / 3 and m["loss_per_sample"] == 0.125
+    # population standard deviation of the advantages {1, 0, -2}: mean -1/3
+    assert abs(m["adv_std"] - math.sqrt(((4 / 3) ** 2 + (1 / 3) ** 2 + (5 / 3) ** 2) / 3)) < 1e-6
+    assert m["old_policy_entropy"] == 0.0 and m["entropy_coeff"] == 0.0       # nothing given: zeros
+    old_ent = torch.tensor([0.5, 1.5, 4.0, 100.0])
+    m2 = O.dual_clip_metrics(0.25, ent, lr, unclipped, clipped, adv, oi, None, 0.2, 0.2, old_entropy=old_ent,
+                             num_samples=2, entropy_coeff=0.01)
+    assert abs(m2["old_policy_entropy"] - 2.0) < 1e-7 and m2["entropy_coeff"] == 0.01      # mean over the indexed positions only
+    assert m2["adv_std"] == m["adv_std"] and m2["kl_div"] == m["kl_div"]
 
 
 # ------------------------------------------------------------------ batch shaping
@@ -305,8 +313,54 @@ def test_pack_samples_keys_and_values():
     assert b["num_output_tokens_non_masked"].item() == 5 and b["num_samples"].item() == 2
     assert b["total_non_modified_reward"].item() == 1.0 and b["truncated_sample"].item() == 1.0
     assert b["reference_output_entropies"].abs().sum() == 0
+    assert b["total_modified_reward"].item() == 0.0 and b["num_modified_samples"].item() == 0.0
+    assert b["delimiter_not_found"].item() == 0.0
+
+
+def test_pack_samples_modified_rewards():
+    """sample_processing_utils.py:167-168, 209-212: samples whose modified_reward is set are counted apart - their
+    modified rewards and delimiter flags are summed, the others contribute their plain reward; total_reward_rank
+    sums the plain reward of all."""
+    spec = [  # (input_len, output_len, reward, modified_reward, delimiter_not_found)
+        (2, 3, 1.0, None, False), (1, 2, 0.5, 0.25, True), (3, 1, 0.0, -1.0, False), (1, 1, 2.0, None, True),
+        (2, 2, 1.5, 0.0, True)]
+    samples = []
+    for i, (li, lo, r, mr, dnf) in enumerate(spec):
+        ids = list(range(10 * i, 10 * i + li + lo))
+        samples.append(dict(sample_ids=ids, sample_position_ids=list(range(li + lo)), labels=O.make_labels(ids, li, lo),
+                            input_len=li, output_len=lo, advantage=float(i), sample_logprobs=[-1.0] * (li + lo),
+                            sample_entropies=[0.5] * (li + lo) if i % 2 else None,
+                            reward=r, modified_reward=mr, delimiter_not_found=dnf, truncated_sample=False))
+    b = O.pack_samples(samples)
+    assert b["num_modified_samples"].item() == 3.0                      # modified_reward = 0.0 still counts as set
+    assert b["total_modified_reward"].item() == 0.25 - 1.0 + 0.0
+    assert b["total_non_modified_reward"].item() == 1.0 + 2.0
+    assert b["delimiter_not_found"].item() == 2.0                       # flags of the modified samples only
+    assert b["total_reward_rank"].item() == 1.0 + 0.5 + 0.0 + 2.0 + 1.5
+    # entropies: given lists where present, zeros of the logprob length elsewhere
+    want_ent = sum(([0.5] * (li + lo) if i % 2 else [0.0] * (li + lo) for i, (li, lo, *_r) in enumerate(spec)), [])
+    assert b["reference_output_entropies"].tolist() == want_ent
 
 
 def test_loss_scaling():
+    """gpu_process_worker.py:1013-1025: local_target = max(1, target // world) whenever world > 0."""
     assert O.scale_microbatch_loss(2.0, 6, 128, world=2) == 2.0 * 6 / 64
-    assert O.scale_microbatch_loss(2.0, 6, 0) == 2.0
+    assert O.scale_microbatch_loss(2.0, 6, 0) == 2.0 * 6          # unset target: max(1, 0 // 1) = 1
+    assert O.scale_microbatch_loss(2.0, 6, 3, world=8) == 2.0 * 6  # 3 // 8 = 0 -> 1
+    assert O.scale_microbatch_loss(2.0, 6, 6, world=1) == 2.0      # scale exactly 1: loss untouched
+    assert O.scale_microbatch_loss(2.0, 6, 0, world=0) == 2.0      # no world, no target: no scaling
+    assert O.scale_microbatch_loss(2.0, 6, 12, world=0) == 1.0
+
+
+def test_split_logprobs_per_sample_hand_case():
+    """gpu_process_worker.py:1694-1703: torch.split by sample length, then python lists."""
+    lp = torch.tensor([-0.5, -1.5, 0.0, -2.0, -3.0, -0.25])
+    ent = torch.tensor([1.0, 2.0, 3.0, 4.0, 5.0, 6.0])
+    got = O.split_logprobs_per_sample(lp, ent, [2, 1, 3])
+    assert got == [{"logprobs": [-0.5, -1.5], "entropies": [1.0, 2.0]},
+                   {"logprobs": [0.0], "entropies": [3.0]},
+                   {"logprobs": [-2.0, -3.0, -0.25], "entropies": [4.0, 5.0, 6.0]}]
+    assert all(isinstance(v, float) for s in got for v in s["logprobs"] + s["entropies"])
+    none = O.split_logprobs_per_sample(lp, None, [6])
+    assert none == [{"logprobs": lp.tolist(), "entropies": None}]
+    assert O.split_logprobs_per_sample(lp[:0], None, []) == []
