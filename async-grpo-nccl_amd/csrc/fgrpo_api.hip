@@ -283,8 +283,15 @@ int run_store_gemm_kmajor(const Tuning& tn, StoreParams p, bool akm, bool bkm, h
   // a K-major tile is read 256 columns wide without clamping: the rows must hold them
   if (g.a_blk != 0 && (g.lda != 256 || g.a_blk % 8 || g.a_blk < 256LL * (akm ? g.seg[0].K : g.M)))
     return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): column-blocked A needs lda = 256 and blocks that hold every row");
-  if (akm && g.a_blk == 0 && (long long)p.tiles_m * Cfg8::BM > g.lda) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): lda < padded M");
-  if (bkm && (long long)p.tiles_n * Cfg8::BN > g.ldb) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): ldb < padded N");
+  // A K-major tile is read 256 columns wide without clamping.  Rows shorter than the padded width are fine: the
+  // excess columns of a row are the start of the next one (values that only reach output columns past M / N, which
+  // are never stored) and, past the last existing row, zeros from the buffer descriptor's bound.  The rows must
+  // hold the logical width, though.
+  if (akm && g.a_blk == 0 && g.M > g.lda) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): lda < M");
+  if (bkm && g.N > g.ldb) return fail(FGRPO_ERR_BAD_ARG, "gemm(k-major): ldb < N");
+  // the kernel bounds its reads by the rows that exist: "all of them" must be said as a number
+  if (akm && p.g.ka_valid <= 0) p.g.ka_valid = g.seg[0].K;
+  if (bkm && p.g.kb_valid <= 0) p.g.kb_valid = g.seg[0].K;
   if (256LL * g.lda * 2 >= (1LL << 32) || 256LL * g.ldb * 2 >= (1LL << 32))
     return fail(FGRPO_ERR_UNSUPPORTED, "gemm(k-major): leading dimension too large");
   {
@@ -343,7 +350,7 @@ long long default_panel_elems(int T, int V) {
 // (three launches' tails and one pass over the fp32 dH accumulator, measured at about 0.15 of such a round).
 // Measured at T=32768, H=1536, V=151936: 8 panels (450 tiles, 1.76 rounds each) 39.1 ms, 7 panels (510 tiles) 38.2.
 int fit_panel_count(int np_min, int H, int V) {
-  const int cus = num_cus(), hT = H / 256, max_np = (V + 255) / 256;
+  const int cus = num_cus(), hT = (H + 255) / 256, max_np = (V + 255) / 256;
   if ((long long)((V + np_min - 1) / np_min + 255) / 256 * hT < cus / 2) return np_min;   // small problems: the small-tile path
   int best = np_min;
   long long best_cost = -1;
@@ -377,7 +384,7 @@ void plan_bwd(const Tuning& tn, BwdPlan& pl, void* ws, int T, int H, int V, int 
   if (cols < 256) cols = 256;
   int np = (int)((V + cols - 1) / cols);
   if (np < 1) np = 1;
-  if (!pl.f32 && H % 256 == 0) np = fit_panel_count(np, H, V);
+  if (!pl.f32 && H % 64 == 0) np = fit_panel_count(np, H, V);
   pl.panel = (int)round_up((V + np - 1) / np, 256);
   pl.npanels = (V + pl.panel - 1) / pl.panel;
   pl.copy_ops = pl.f32 || (H % 64 != 0);
@@ -394,9 +401,11 @@ void plan_bwd(const Tuning& tn, BwdPlan& pl, void* ws, int T, int H, int V, int 
   // In-place (K-major) gradient GEMMs: bf16 operands used as they are, H a multiple of the tile width, and
   // enough tiles to fill the device (small problems keep the small-tile path).
   {
-    const long long th = (long long)((T + 255) / 256) * (H / 256);
-    const long long vh = (long long)(((V < pl.panel ? V : pl.panel) + 255) / 256) * (H / 256);
-    pl.kmajor = tn.bwd_kmajor && !pl.copy_ops && H % 256 == 0 && pl.bm == 256 && pl.bn % 64 == 0 &&
+    // (H need not be a multiple of the 256-column tile: the last tile reads past the end of each row into the next
+    // one - inside the buffer descriptor, zeros beyond it - and those output columns are never stored)
+    const long long th = (long long)((T + 255) / 256) * ((H + 255) / 256);
+    const long long vh = (long long)(((V < pl.panel ? V : pl.panel) + 255) / 256) * ((H + 255) / 256);
+    pl.kmajor = tn.bwd_kmajor && !pl.copy_ops && H % 64 == 0 && pl.bm == 256 && pl.bn % 64 == 0 &&
                 th >= num_cus() / 2 && vh >= num_cus() / 2;
     pl.kmajor_dh = pl.kmajor && tn.bwd_kmajor >= 2;
   }
@@ -428,9 +437,9 @@ namespace {
 // Conditions of the kept-logits pair: the forward on the 256x256x64 two-buffer tile with operands used in place,
 // both gradient GEMMs on operands read where they lie.
 bool keep_supported(const Tuning& tn, int T, int H, int V, int dtype) {
-  if (dtype != FGRPO_BF16 || T <= 0 || V <= 0 || H <= 0 || H % 256 != 0) return false;
+  if (dtype != FGRPO_BF16 || T <= 0 || V <= 0 || H <= 0 || H % 64 != 0) return false;
   if (pick_variant(tn, 8, V, T) != 8) return false;
-  const long long th = (long long)((T + 255) / 256) * (H / 256), vh = (long long)((V + 255) / 256) * (H / 256);
+  const long long th = (long long)((T + 255) / 256) * ((H + 255) / 256), vh = (long long)((V + 255) / 256) * ((H + 255) / 256);
   return th >= num_cus() / 2 && vh >= num_cus() / 2;
 }
 // Layout of the kept buffer: the column-blocked bf16 numerators, then the per-token references (fp32), then the
@@ -764,7 +773,7 @@ int fgrpo_logprob_fwd_keep(const void* hidden, const void* weight, const void* b
                            void* stream) {
   if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd_keep: T=%d H=%d V=%d", T, H, V);
   if (!keep_supported(g_tune, T, H, V, dtype))
-    return fail(FGRPO_ERR_UNSUPPORTED, "logprob_fwd_keep: needs bf16, H %% 256 == 0 and a device-filling problem (T=%d H=%d V=%d)", T, H, V);
+    return fail(FGRPO_ERR_UNSUPPORTED, "logprob_fwd_keep: needs bf16, H %% 64 == 0 and a device-filling problem (T=%d H=%d V=%d)", T, H, V);
   if (!logits_keep || !aligned16(logits_keep) || logits_keep_bytes < keep_bytes(T, V))
     return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd_keep: logits buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
   return logprob_fwd_impl(hidden, weight, bias, labels, inv_temp, T, H, V, dtype, lp_out, ent_out, lse_out, ws, ws_bytes,
@@ -828,7 +837,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
   if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: inv_temperature must be positive");
   const Tuning tn = g_tune;
   if (!keep_supported(tn, T, H, V, dtype))
-    return fail(FGRPO_ERR_UNSUPPORTED, "lmhead_bwd_kept: needs bf16, H %% 256 == 0 and a device-filling problem (T=%d H=%d V=%d)", T, H, V);
+    return fail(FGRPO_ERR_UNSUPPORTED, "lmhead_bwd_kept: needs bf16, H %% 64 == 0 and a device-filling problem (T=%d H=%d V=%d)", T, H, V);
   if (!logits_keep || !aligned16(logits_keep) || logits_keep_bytes < keep_bytes(T, V))
     return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: kept buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
   if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: dbias requested without a bias");

@@ -848,13 +848,18 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   const long long lda2 = g.lda * 2, ldb2 = g.ldb * 2;
   long long a_rem = (AKM && g.ka_valid > 0) ? g.ka_valid : (1LL << 40);   // k rows of A that exist from Ap on
   long long b_rem = (BKM && g.kb_valid > 0) ? g.kb_valid : (1LL << 40);
-  auto bytes_of = [](long long rows, long long ld2) -> uint32_t {
+  // bytes from a descriptor's base (first k row of the step, first column of the tile) to the end of the operand:
+  // `rows` k rows of ld2 bytes, less the tile's column offset - the last tile of a row width that is not a multiple
+  // of 256 reads past the end of every row, which must not carry past the end of the last one
+  auto bytes_of = [](long long rows, long long ld2, long long col_bytes) -> uint32_t {
     if (rows <= 0) return 0u;
-    const long long bts = rows * ld2;
+    const long long bts = rows * ld2 - col_bytes;
+    if (bts <= 0) return 0u;
     return (rows > (1LL << 31) || bts > 0xffffffffLL) ? 0xffffffffu : (uint32_t)bts;
   };
-  __amdgpu_buffer_rsrc_t rsa = make_rsrc(Ap, AKM ? bytes_of(a_rem, lda2) : 0xffffffffu);
-  __amdgpu_buffer_rsrc_t rsb = make_rsrc(Bp, BKM ? bytes_of(b_rem, ldb2) : 0xffffffffu);
+  const long long a_col = (AKM && g.a_blk == 0) ? (long long)row0 * 2 : 0, b_col = BKM ? (long long)col0 * 2 : 0;
+  __amdgpu_buffer_rsrc_t rsa = make_rsrc(Ap, AKM ? bytes_of(a_rem, lda2, a_col) : 0xffffffffu);
+  __amdgpu_buffer_rsrc_t rsb = make_rsrc(Bp, BKM ? bytes_of(b_rem, ldb2, b_col) : 0xffffffffu);
   uint32_t ka = 0, kb = 0;                      // running K byte offset of a K-contiguous operand
   const int dst_w = wave * 1024;                // both layouts: one load fills 1 KiB, loads i are NW KiB apart
 
@@ -873,7 +878,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
       if constexpr (AKM) {
         Ap += (long long)C::BK * lda2;
         a_rem -= C::BK;
-        rsa = make_rsrc(Ap, bytes_of(a_rem, lda2));
+        rsa = make_rsrc(Ap, bytes_of(a_rem, lda2, a_col));
       } else {
         ka += C::BK * 2;
         if (--ablk_left == 0) {
@@ -888,7 +893,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
       if constexpr (BKM) {
         Bp += (long long)C::BK * ldb2;
         b_rem -= C::BK;
-        rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2));
+        rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2, b_col));
       } else {
         kb += C::BK * 2;
       }

@@ -34,6 +34,17 @@ def test_kept_logits_against_oracle(dev, mode):
     check(want, got, o, g, f32=False)
 
 
+@pytest.mark.parametrize("keep", [True, False])
+def test_hidden_size_that_is_not_a_multiple_of_the_tile(dev, keep):
+    """H = 896 (the 0.5B model's width, 3.5 tiles of 256): the gradient products still read W, hidden and the
+    [T x V] buffer where they lie; both the kept and the recomputing backward against the oracle."""
+    from fgrpo import ops
+    w = filling_workload(16, H=896)
+    assert ops.keep_supported(w.T, w.H, w.V, torch.bfloat16)
+    want, got, o, g, _, _ = run_case(w, dev, "north_star", keep_logits=keep)
+    check(want, got, o, g, f32=False)
+
+
 def test_kept_logits_with_bias_and_temperature(dev):
     w = filling_workload(12)
     bias = (torch.randn(w.V, generator=torch.Generator().manual_seed(9)) * 0.3).to(w.dtype)

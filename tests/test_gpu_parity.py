@@ -183,10 +183,15 @@ def test_bias_and_temperature(dev):
     ("ab", 700, 512, 320, 300),
     ("ab", 1024, 1536, 1024, 1000),
     ("a", 512, 300, 192, 0),
+    ("b", 512, 896, 256, 0),          # rows of 896 columns: the last 256-column tile reads into the next row
+    ("ab", 600, 896, 320, 290),
+    ("b", 300, 328, 192, 0),
 ])
 def test_contraction_major_gemm_against_torch(dev, layout, M, N, K, k_valid):
     """C = A B^T with A and/or B stored [K][M] / [K][N]; fp32 accumulation of bf16 products is exact up to
-    summation order, so the fp32 matmul of the same bf16 numbers is the reference."""
+    summation order, so the fp32 matmul of the same bf16 numbers is the reference.  The K-major B operand is an
+    exact-size allocation: a row width that is not a multiple of 256 makes the last tile read past the end of each
+    row, which the kernel bounds by the end of the operand."""
     from fgrpo import ops
     gen = torch.Generator(device="cpu").manual_seed(11)
     kr = k_valid if k_valid else K
