@@ -61,7 +61,13 @@ struct GemmOperands {
   // down the rows of one block (K-major use) then reads one sequential stream, and a tile that walks along
   // the columns (K-contiguous use) reads 128 KiB contiguous pieces.
   long long a_blk;
+  // gemm_mainloop_km with both operands K-major only: the contraction may skip whole K steps (64 rows each) that
+  // are known to contribute nothing.  k_runs (device memory, written by an earlier launch on the stream) =
+  // {number of runs R, K steps in all runs, start_0 .. start_{kRunCap-1}, end_0 .. end_{kRunCap-1}}: run r covers
+  // the K steps start_r <= k < end_r, runs ascending and disjoint.  Null = every K step.
+  const int* k_runs;
 };
+constexpr int kRunCap = 4096;   // runs a k_runs list can hold (more live/dead alternations than that: pass null)
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int NST_ = 2, bool DMA_ = false>
 struct TileCfg {
@@ -863,7 +869,22 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   uint32_t ka = 0, kb = 0;                      // running K byte offset of a K-contiguous operand
   const int dst_w = wave * 1024;                // both layouts: one load fills 1 KiB, loads i are NW KiB apart
 
-  const int nk_total = g.seg[0].K / C::BK;
+  // run list (both operands K-major only): the issue cursor walks the listed K steps; the compute side never
+  // knows, it consumes LDS buffers in the order they were filled
+  const int* runs = (AKM && BKM) ? g.k_runs : nullptr;
+  const int n_runs = runs ? runs[0] : 0;
+  const int nk_total = runs ? runs[1] : g.seg[0].K / C::BK;
+  int run_idx = 0, run_left = 0, cur_step = 0;
+  if (runs != nullptr && n_runs > 0) {
+    cur_step = runs[2];
+    run_left = runs[2 + kRunCap] - cur_step;
+    Ap += (long long)cur_step * C::BK * lda2;
+    Bp += (long long)cur_step * C::BK * ldb2;
+    a_rem -= (long long)cur_step * C::BK;
+    b_rem -= (long long)cur_step * C::BK;
+    rsa = make_rsrc(Ap, bytes_of(a_rem, lda2, a_col));
+    rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2, b_col));
+  }
   const long long a_blk_bytes = (!AKM) ? g.a_blk * 2 : 0;
   int ablk_left = 256 / C::BK;
   auto issue_one = [&](int stage, int idx) {
@@ -875,9 +896,19 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsb, FGRPO_LDS_PTR(base + REG + dst_w + (idx - C::PA) * C::NW * 1024), 16,
                                                (int)boff[idx - C::PA], (int)kb, 0, FGRPO_DMA_AUX);
     if (idx == LPT - 1) {                        // next K step
+      long long jump = 1;                        // K steps from this one to the next one to fetch
+      if constexpr (AKM && BKM) {
+        if (runs != nullptr && --run_left == 0 && run_idx + 1 < n_runs) {   // this run is done: on to the next
+          ++run_idx;
+          const int s = runs[2 + run_idx];
+          jump = s - cur_step;
+          run_left = runs[2 + kRunCap + run_idx] - s;
+        }
+        cur_step += (int)jump;
+      }
       if constexpr (AKM) {
-        Ap += (long long)C::BK * lda2;
-        a_rem -= C::BK;
+        Ap += jump * C::BK * lda2;
+        a_rem -= jump * C::BK;
         rsa = make_rsrc(Ap, bytes_of(a_rem, lda2, a_col));
       } else {
         ka += C::BK * 2;
@@ -891,8 +922,8 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
         }
       }
       if constexpr (BKM) {
-        Bp += (long long)C::BK * ldb2;
-        b_rem -= C::BK;
+        Bp += jump * C::BK * ldb2;
+        b_rem -= jump * C::BK;
         rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2, b_col));
       } else {
         kb += C::BK * 2;

@@ -7,7 +7,7 @@ namespace fgrpo {
 namespace {
 template <class C>
 int launch_store(const StoreParams& p, hipStream_t st) {
-  return launch_tile_kernel<gemm_store_kernel<C, false, false>, C>(p, p.tiles_m * p.tiles_n, st);
+  return launch_tile_kernel<gemm_store_kernel<C, false, false>, C>(p, p.nblocks, st);
 }
 }  // namespace
 
@@ -18,7 +18,7 @@ int launch_store_variant(int variant, const StoreParams& p, hipStream_t st) {
 }
 
 int launch_store_kmajor(bool akm, bool bkm, const StoreParams& p, hipStream_t st) {
-  const int nb = p.tiles_m * p.tiles_n;
+  const int nb = p.nblocks;
   if (akm && bkm) return launch_tile_kernel<gemm_store_kernel<Cfg8, true, true>, Cfg8>(p, nb, st);
   if (akm) return launch_tile_kernel<gemm_store_kernel<Cfg8, true, false>, Cfg8>(p, nb, st);
   if (bkm) return launch_tile_kernel<gemm_store_kernel<Cfg8, false, true>, Cfg8>(p, nb, st);

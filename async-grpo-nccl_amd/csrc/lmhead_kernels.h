@@ -518,9 +518,12 @@ struct StoreParams {
   long long ldc;
   float alpha;
   const float* alpha_dev;  // optional device scalar multiplied into alpha
-  int tiles_m, tiles_n, group_m;
+  int tiles_m, tiles_n, group_m;   // group_m == 0: row tiles dealt round-robin to the XCDs (see gemm_store_kernel)
+  int nblocks;                     // work-groups to launch (set by the launcher's caller)
   int wide_stores;         // ldc and the output / addend bases allow 16-byte pieces (set by the launcher)
   const float* row_scale;  // optional [M]: output row m is multiplied by row_scale[m] (after alpha, before c_in)
+  const int* m_tile_live;  // optional [tiles_m] (BM = 256 rows per tile): 0 = every row of the tile has row_scale 0,
+                           // the contraction is skipped and the tile is written as zeros (or as c_in)
 };
 
 // Output is either fp32 or bf16 (never both); rows/cols past M/N are skipped.
@@ -637,22 +640,37 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
 
-  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int per_group = p.group_m * p.tiles_n;
-  const int grp = lid / per_group;
-  const int first_m = grp * p.group_m;
-  const int gsz = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
-  const int w = lid - grp * per_group;
-  const int tm = first_m + w % gsz;
-  const int tn = w / gsz;
+  int tm, tn;
+  if (p.group_m > 0) {
+    // every XCD walks one contiguous range of tiles, group_m row tiles x all column tiles at a time
+    const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int per_group = p.group_m * p.tiles_n;
+    const int grp = lid / per_group;
+    const int first_m = grp * p.group_m;
+    const int gsz = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
+    const int w = lid - grp * per_group;
+    tm = first_m + w % gsz;
+    tn = w / gsz;
+  } else {
+    // row tiles dealt round-robin to the XCDs (work-group b runs on XCD b % 8), all column tiles of a row tile side
+    // by side on one XCD: neighbouring row tiles - which are dead or alive together when whole samples carry no
+    // gradient - land on different XCDs, so skipped tiles thin every XCD's share instead of emptying some
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    tm = (idx / p.tiles_n) * 8 + xcd;
+    tn = idx % p.tiles_n;
+    if (tm >= p.tiles_m) return;
+  }
   const int row0 = tm * C::BM, col0 = tn * C::BN;
 
   f32x16_t acc[C::TM][C::TN];
   zero_acc<C>(acc);
-  if constexpr (AKM || BKM)
-    gemm_mainloop_km<C, AKM, BKM>(p.g, row0, col0, smem, acc);
-  else
-    run_mainloop<C>(p.g, row0, col0, smem, acc);
+  const bool dead = p.m_tile_live != nullptr && p.m_tile_live[tm] == 0;     // work-group uniform
+  if (!dead) {
+    if constexpr (AKM || BKM)
+      gemm_mainloop_km<C, AKM, BKM>(p.g, row0, col0, smem, acc);
+    else
+      run_mainloop<C>(p.g, row0, col0, smem, acc);
+  }
 
   const float alpha = p.alpha * (p.alpha_dev ? *p.alpha_dev : 1.f);
   const int mode = (p.c_in ? 1 : 0) | (p.c_out_bf16 ? 2 : 0);

@@ -263,4 +263,77 @@ __global__ void keep_col_sum_kernel(const bf16_t* e, long long blk, const float*
   if (ty == 0 && c < V) out_bf16[c] = f32_to_bf16_rn((red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]));
 }
 
+// Which parts of the token axis carry a gradient at all (row factor a_t != 0): zero-advantage samples and ignored
+// labels form long stretches of dead rows, which the gradient GEMMs skip - the dHidden product by 256-row tile
+// (m_tile_live), the dW product, whose contraction runs over the tokens, by K step of 64 rows (k_runs: the list of
+// live runs gemm_mainloop_km walks).  One work-group; thread i owns a contiguous piece of the 64-row chunks.
+// If the rows alternate more often than the list can hold, k_runs[0] is written as one run over everything
+// (the products are then merely not shortened).
+struct KeepLiveParams {
+  const float* row_scale;    // [T]
+  int T;
+  int n_chunks;              // ceil(T / 64), at most kLiveMaxChunks
+  int k_steps;               // K steps of the dW product (round_up(T, 256) / 64)
+  int* k_runs;               // [2 + 2 * kRunCap]
+  int* m_tile_live;          // [ceil(T / 256)]
+};
+constexpr int kLiveMaxChunks = 32768;      // 2 M tokens: beyond that nothing is skipped (the lists say "all live")
+
+__global__ __launch_bounds__(1024) void keep_live_runs_kernel(const KeepLiveParams p) {
+  __shared__ unsigned char live[kLiveMaxChunks];
+  __shared__ int starts_before[1024 + 1], live_before[1024 + 1];
+  const int tid = threadIdx.x;
+  // chunk flags: one wavefront per chunk, 64 rows each
+  for (int c = tid >> 6; c < p.n_chunks; c += 16) {
+    const int t = c * 64 + (tid & 63);
+    const bool on = t < p.T && p.row_scale[t] != 0.f;
+    const bool any = __builtin_amdgcn_ballot_w64(on) != 0;
+    if ((tid & 63) == 0) live[c] = any ? 1 : 0;
+  }
+  __syncthreads();
+  for (int m = tid; m * 4 < p.n_chunks; m += 1024) {
+    int any = 0;
+    for (int c = m * 4; c < m * 4 + 4 && c < p.n_chunks; ++c) any |= live[c];
+    p.m_tile_live[m] = any;
+  }
+  const int per = (p.n_chunks + 1023) / 1024;
+  const int c0 = tid * per, c1 = (c0 + per < p.n_chunks ? c0 + per : p.n_chunks);
+  int ns = 0, nl = 0;
+  for (int c = c0; c < c1; ++c) {
+    nl += live[c];
+    ns += live[c] && (c == 0 || !live[c - 1]);
+  }
+  starts_before[tid + 1] = ns;
+  live_before[tid + 1] = nl;
+  if (tid == 0) starts_before[0] = live_before[0] = 0;
+  __syncthreads();
+  if (tid == 0) {        // 1024 additions: a serial scan is fine here
+    for (int i = 1; i <= 1024; ++i) {
+      starts_before[i] += starts_before[i - 1];
+      live_before[i] += live_before[i - 1];
+    }
+  }
+  __syncthreads();
+  const int n_runs = starts_before[1024], n_live = live_before[1024];
+  if (n_runs > kRunCap) {                  // too fragmented for the list: one run over every K step
+    if (tid == 0) {
+      p.k_runs[0] = 1;
+      p.k_runs[1] = p.k_steps;
+      p.k_runs[2] = 0;
+      p.k_runs[2 + kRunCap] = p.k_steps;
+    }
+    return;
+  }
+  if (tid == 0) {
+    p.k_runs[0] = n_runs;
+    p.k_runs[1] = n_live;
+  }
+  int k = starts_before[tid];              // runs that start before this thread's piece
+  for (int c = c0; c < c1; ++c) {
+    if (!live[c]) continue;
+    if (c == 0 || !live[c - 1]) p.k_runs[2 + k++] = c;                       // run k starts here
+    if (c + 1 >= p.n_chunks || !live[c + 1]) p.k_runs[2 + kRunCap + k - 1] = c + 1;   // and the current run ends here
+  }
+}
+
 }  // namespace fgrpo

@@ -118,7 +118,7 @@ class ClockSampler:
                 "source": "pp_dpm_sclk (active level) sampled during the timed steps"}
 
 
-def parity_gate(w, step_fn, hidden2d, weight, shifted, old, ref, adv, rows_n=64):
+def parity_gate(w, step_fn, hidden2d, weight, shifted, old, ref, adv, north_star=True, rows_n=64):
     """Before anything is timed: one step of the path on the benchmark's own inputs against the oracle.
     `rows_n` sampled token rows (logprob, entropy, and the dHidden row when the workload has a backward) and the
     loss.  The oracle forms the sampled rows' logits on the host from the same bf16 inputs in fp32; the loss is
@@ -145,9 +145,13 @@ def parity_gate(w, step_fn, hidden2d, weight, shifted, old, ref, adv, rows_n=64)
     ok = res["max_abs_dlogprob"] <= 2e-3 and res["max_abs_dentropy"] <= 5e-3
     if not p["forward_only"]:
         lp_c = lp_all.double().cpu().requires_grad_(True)
-        want = O.grpo_objective_from_logprobs(lp_c, shifted.cpu(), old.double().cpu(), adv.double().cpu(), p["clip_low"],
-                                              p["clip_high"], p["clip_ratio_c"], ref.double().cpu(), p["kl_beta"],
-                                              "sample_mean", w.cu_seqlens.cpu())
+        if north_star:
+            want = O.grpo_objective_from_logprobs(lp_c, shifted.cpu(), old.double().cpu(), adv.double().cpu(),
+                                                  p["clip_low"], p["clip_high"], p["clip_ratio_c"], ref.double().cpu(),
+                                                  p["kl_beta"], "sample_mean", w.cu_seqlens.cpu())
+        else:
+            want = O.grpo_objective_from_logprobs(lp_c, shifted.cpu(), old.double().cpu(), adv.double().cpu(),
+                                                  p["clip_low"], p["clip_high"], p["clip_ratio_c"])
         want[0].backward()
         res["loss"] = float(loss.detach())
         res["loss_oracle"] = float(want[0])
@@ -325,6 +329,14 @@ def main():
     ap.add_argument("--config", default="cfg1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check that precedes the timed steps")
+    ap.add_argument("--objective", choices=["north_star", "reference"], default="north_star",
+                    help="north_star: KL to the reference policy + mean over samples of per-sample token means (every "
+                         "scored token has a gradient); reference: the reference's own objective, token mean without "
+                         "KL (grpo_loss.py:318-348) - tokens of zero-advantage groups then have no gradient and the "
+                         "backward skips them")
+    ap.add_argument("--reward-p", type=float, default=None,
+                    help="probability of reward 1 per sample (default: the configuration's); with --objective reference "
+                         "it sets the share of zero-advantage groups")
     ap.add_argument("--keep-logits", choices=["auto", "on", "off"], default="auto",
                     help="keep the [T x V] bf16 soft-max numerators for the backward (auto: when supported and memory allows) "
                          "or recompute the logits there")
@@ -354,13 +366,15 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = make_workload(args.config, seed=args.seed, device=dev)
+    w = make_workload(args.config, seed=args.seed, device=dev,
+                      overrides=None if args.reward_p is None else dict(reward_p=args.reward_p))
     p = w.params
     T, H, V = w.T, w.H, w.V
     fwd_only = p["forward_only"]
     labels = w.labels
     shifted = ops.shift_labels(labels).reshape(-1)
     keep_logits = {"auto": None, "on": True, "off": False}[args.keep_logits]
+    north_star = args.objective == "north_star"
 
     # inputs of the objective: advantages from the group kernel, old/ref = current logprob + noise
     adv_s = ops.group_advantages(w.rewards, w.group_offsets, p["adv_eps"])
@@ -386,10 +400,10 @@ def main():
                 return G.fused_log_probs_and_entropy_fn(s.weight, None, s.hidden, s.labels)
         s.hidden.grad = None
         s.weight.grad = None
+        extra = dict(ref_logprobs=s.ref, kl_beta=p["kl_beta"], loss_agg_mode="sample_mean", cu_seqlens=s.cu) if north_star else {}
         out = G.grpo_loss_and_entropy_ce_fn(s.weight, None, s.hidden, s.labels, 1.0, s.old, s.adv, p["clip_low"],
                                             p["clip_high"], p["clip_ratio_c"], loss_chunksize=p["chunk"],
-                                            ref_logprobs=s.ref, kl_beta=p["kl_beta"], loss_agg_mode="sample_mean",
-                                            cu_seqlens=s.cu, keep_logits=keep_logits)
+                                            keep_logits=keep_logits, **extra)
         out[0].backward()
         return out
 
@@ -402,7 +416,7 @@ def main():
         return out[2] + old, out[1], out[0], sets[0].hidden.grad        # log_ratio = lp - old
     parity = None
     if not args.no_parity:
-        parity = parity_gate(w, gate_step, w.hidden.reshape(T, H), w.weight, shifted, old, ref, adv)
+        parity = parity_gate(w, gate_step, w.hidden.reshape(T, H), w.weight, shifted, old, ref, adv, north_star)
         if not parity["passed"]:
             print("bench.py: parity check failed, nothing timed: " + json.dumps(parity), file=sys.stderr)
             sys.exit(1)
@@ -476,6 +490,11 @@ def main():
                                f"{'forward only' if fwd_only else 'forward+backward (dHidden, dW)'}, "
                                f"{w.n_samples} samples, chunk hint {p['chunk']}",
                    "tokens": T, "hidden": H, "vocab": V, "samples": w.n_samples,
+                   "objective": None if fwd_only else (
+                       "north_star: dual clip + k3 KL to the reference policy, mean over samples of per-sample token means"
+                       if north_star else "reference: dual clip, token mean, no KL (grpo_loss.py:318-348)"),
+                   "tokens_without_gradient": None if fwd_only else float(((adv == 0) | (shifted == -100)).float().mean()) if not north_star
+                   else float((shifted == -100).float().mean()),
                    "backward": None if fwd_only else ("bf16 soft-max numerators kept for the backward" if kept else "logits recomputed in the backward"),
                    "input_sets_rotated": len(sets)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",

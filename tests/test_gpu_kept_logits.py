@@ -144,6 +144,44 @@ def test_kept_buffer_survives_the_backward(dev):
     assert cos(b[0], a[0]) >= 0.99999 and abs(b[1].float().norm().item() / a[1].float().norm().item() - 2.0) < 1e-2
 
 
+@pytest.mark.parametrize("pattern", ["groups", "all_dead", "alternating", "tail"])
+def test_rows_without_gradient_are_skipped_exactly(dev, pattern):
+    """Zero-advantage samples give long stretches of tokens with g_t = 0 (the reference logs their share as
+    adv_zero_frac, grpo_loss.py:450).  The kept-path backward skips them - dHidden by 256-row tile, dW by 64-row
+    step of its contraction - and must produce the very same gradients as without skipping: leaving out exact
+    zeros changes no fp32 sum."""
+    from fgrpo import _lib, ops
+    w = filling_workload(17, tokens=8192 + 300)
+    T = w.T
+    hs, W = w.hidden.reshape(T, w.H).to(dev), w.weight.to(dev)
+    y = ops.shift_labels(w.labels.to(dev)).reshape(-1)
+    g = torch.randn(T, generator=torch.Generator().manual_seed(5)).to(dev) / T
+    if pattern == "groups":                       # dead stretches that start and end anywhere
+        for a, b in ((0, 700), (1500, 1501), (2048, 4096), (5000, 5063), (6000, 8300)):
+            g[a:b] = 0
+    elif pattern == "all_dead":
+        g.zero_()
+    elif pattern == "alternating":                # every other 64-row step dead: many short runs
+        g.view(-1)[: (T // 128) * 128].view(-1, 2, 64)[:, 1, :] = 0
+    else:                                         # only the very last rows live
+        g[: T - 5] = 0
+    lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
+    res = {}
+    for skip in (1, 0):
+        _lib.set_tuning(keep_skip_dead=skip)
+        try:
+            res[skip] = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
+        finally:
+            _lib.set_tuning(keep_skip_dead=1)
+    assert torch.equal(res[1][0], res[0][0]) and torch.equal(res[1][1], res[0][1])
+    assert (res[1][0][g == 0] == 0).all()
+    if pattern == "all_dead":
+        assert (res[1][1] == 0).all()
+    else:
+        dH0, dW0, _ = ops.lmhead_bwd(hs, W, None, y, lse, g, None, 1.0, True, True, False, 0)
+        assert cos(res[1][0], dH0) >= 0.9999 and cos(res[1][1], dW0) >= 0.9999
+
+
 def test_keep_refuses_what_it_cannot_do(dev):
     from fgrpo import ops
     hs = torch.randn(512, 192, device=dev).bfloat16()
