@@ -102,7 +102,9 @@ __device__ __forceinline__ void patch_flush(char* patch, bf16_t* out, int lane_v
     const int m = tok & (NSLOT - 1);
     u32x4_t v = pv[r];
     if (m & 1) v = u32x4_t{v[2], v[3], v[0], v[1]};       // odd rows hold the two slots of a piece swapped
-    *(u32x4_t*)(out + (long long)tok * 256 + piece * 8) = v;
+    // non-temporal: the buffer is written once and read by a later launch; stored normally its 10 GB push the
+    // operand tiles out of the L2s (forward kernel at T=32768, H=1536, V=151936: 14.46 ms, non-temporal 12.65)
+    __builtin_nontemporal_store(v, (u32x4_t*)(out + (long long)tok * 256 + piece * 8));
   }
 }
 
@@ -487,7 +489,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
             const int m = tok & (NSLOT - 1);
             u32x4_t v = pv[r];
             if (m & 1) v = u32x4_t{v[2], v[3], v[0], v[1]};       // odd rows hold the two slots of a piece swapped
-            *(u32x4_t*)(out + (long long)tok * 256 + piece * 8) = v;
+            __builtin_nontemporal_store(v, (u32x4_t*)(out + (long long)tok * 256 + piece * 8));   // see patch_flush
           }
         }
       };

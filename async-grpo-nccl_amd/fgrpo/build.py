@@ -93,7 +93,7 @@ def check_resource_usage(usage: dict) -> list:
 def _compile(src: str, verbose: bool):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [hipcc, *HIPCC_FLAGS, *os.environ.get("FGRPO_EXTRA_FLAGS", "").split(), "-c", os.path.join(CSRC, src), "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
