@@ -445,13 +445,14 @@ bool keep_supported(const Tuning& tn, int T, int H, int V, int dtype) {
   const long long th = (long long)((T + 255) / 256) * ((H + 255) / 256), vh = (long long)((V + 255) / 256) * ((H + 255) / 256);
   return th >= num_cus() / 2 && vh >= num_cus() / 2;
 }
-// Layout of the kept buffer: the column-blocked bf16 numerators, then the per-token references (fp32), then the
-// overflow flag (one int in its own 256 bytes).
+// Layout of the kept buffer: the column-blocked bf16 numerators, then the per-token references and target logits
+// (fp32 each), then the overflow flag (one int in its own 256 bytes).
 size_t keep_block_bytes(int T, int V) { return (size_t)round_up(V, 256) * (size_t)round_up(T, 256) * sizeof(bf16_t); }
-size_t keep_bytes(int T, int V) { return keep_block_bytes(T, V) + (size_t)round_up(T, 256) * sizeof(float) + 256; }
+size_t keep_bytes(int T, int V) { return keep_block_bytes(T, V) + 2 * (size_t)round_up(T, 256) * sizeof(float) + 256; }
 float* keep_ref2_of(void* keep, int T, int V) { return (float*)((char*)keep + keep_block_bytes(T, V)); }
+float* keep_xy_of(void* keep, int T, int V) { return keep_ref2_of(keep, T, V) + round_up(T, 256); }
 int* keep_flag_of(void* keep, int T, int V) {
-  return (int*)((char*)keep + keep_block_bytes(T, V) + (size_t)round_up(T, 256) * sizeof(float));
+  return (int*)((char*)keep + keep_block_bytes(T, V) + 2 * (size_t)round_up(T, 256) * sizeof(float));
 }
 
 int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
@@ -496,7 +497,17 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
     p.keep_blk = (long long)pl.tiles_t * kCfg[8].bn * 256;
     float* ref2 = keep_ref2_of(keep, T, V);
     int* flag = keep_flag_of(keep, T, V);
-    KeepRefParams r{(const bf16_t*)hidden, (const bf16_t*)weight, p.bias, (const long long*)labels, T, H, V, inv_temp, ref2, flag};
+    // the reference's sample of the vocabulary: the plain forward kernel over the first rows of W; only the maxima
+    // of its per-split partials are used (the main launch below overwrites the partials afterwards)
+    FwdParams sp = p;
+    const int vs = V < kKeepSampleRows ? V : kKeepSampleRows;
+    sp.g.M = vs;
+    sp.tiles_v = (vs + kCfg[8].bm - 1) / kCfg[8].bm;
+    sp.nsplit = sp.tiles_v < pl.nsplit ? sp.tiles_v : pl.nsplit;
+    rc = launch_fwd_variant(8, sp, st);
+    if (rc) return rc;
+    KeepRefParams r{(const bf16_t*)hidden, (const bf16_t*)weight, p.bias, (const long long*)labels, T, H, V, inv_temp,
+                    pl.part, sp.nsplit, ref2, keep_xy_of(keep, T, V), flag};
     hipLaunchKernelGGL(keep_reference_kernel, dim3((T + 3) / 4), dim3(256), 0, st, r);
     HIP_TRY(hipGetLastError());
     p.keep_ref2 = ref2;
@@ -864,7 +875,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
 
   {
     PhaseScope ph(kPhaseDlogits, st);
-    KeepPrepParams k{ek, blk, keep_ref2_of(logits_keep, T, V), (const long long*)labels, lse, g, gout_dev, inv_temp,
+    KeepPrepParams k{ek, blk, keep_ref2_of(logits_keep, T, V), keep_xy_of(logits_keep, T, V), (const long long*)labels, lse, g, gout_dev, inv_temp,
                      (const bf16_t*)hidden, T, H, V, pl.row_scale, dW_out ? pl.hidden_scaled : nullptr};
     hipLaunchKernelGGL(keep_backward_prep_kernel, dim3((T + 3) / 4), dim3(256), 0, st, k);
     HIP_TRY(hipGetLastError());

@@ -150,15 +150,19 @@ __global__ void panel_row_sum_kernel(const bf16_t* vt_hi, const bf16_t* vt_lo, l
 // Kept soft-max numerators (forward KEEP kernel): the small kernels around them.
 //
 // keep_reference_kernel, before the forward: the per-token reference of the stored exponentials,
-//   ref_t = x_t[y_t] / temperature + kKeepOffset   (x_t[y_t] = W[y_t] . h_t + b[y_t], a dot product per token),
-// written as ref_t * log2(e); +huge for tokens with an ignored or invalid label (their rows are stored as zeros).
-// Stored values are exp(x_tv/temperature - ref_t) = p_v / p_y * exp(-kKeepOffset): finite in bf16 as long as the
-// target's log-probability is above -(88 + kKeepOffset) = -128 nats; the forward kernel raises a flag otherwise.
+//   ref_t = max(x_t[y_t], max over a sample of the vocabulary of x_t[v]) / temperature + kKeepOffset
+// (x_t[y_t] = W[y_t] . h_t + b[y_t], a dot product per token; the sample's maxima come from a run of the forward
+// kernel over the first kKeepSampleRows rows of W, whose per-split partials this kernel merges), written as
+// ref_t * log2(e); +huge for tokens with an ignored or invalid label (their rows are stored as zeros).
+// Stored values are exp(x_tv/temperature - ref_t): finite in bf16 as long as the row's largest logit exceeds both
+// the target's and the sample's by less than 88 + kKeepOffset = 128 nats (temperature applied) - i.e. always for a
+// policy scoring tokens it could have sampled, and also for an untrained model with near-Gaussian logits; the
+// forward kernel raises a flag otherwise.
 //
 // keep_backward_prep_kernel, before the gradient GEMMs: with s_t = exp(ref_t - lse_t) the probability is
 // p_tv = E[t, v] * s_t, so dLogits[t, v] = c_t (1[v = y_t] - p_tv) = a_t * E'[t, v] with
-//   a_t = -c_t * s_t,   E' = E except E'[t, y_t] = (p_y - 1) / s_t  (written in place, from the fp32 lse, not from
-//   the stored bf16 value),   c_t = g_t * gout / temperature.
+//   a_t = -c_t * s_t,   E' = E except E'[t, y_t] = (p_y - 1) / s_t  (written in place, from the fp32 lse and target
+//   logit, not from the stored bf16 value),   c_t = g_t * gout / temperature.
 // dHidden = diag(a) (E' W): the row factor goes into the GEMM's epilogue; dW = E'^T (diag(a) hidden): the kernel
 // writes the scaled copy of hidden.  One work-group of 256 threads per 4 tokens (a wavefront per token).
 // ---------------------------------------------------------------------------
@@ -171,9 +175,13 @@ struct KeepRefParams {
   const long long* labels;   // shifted labels [T]
   int T, H, V;
   float inv_temp;
+  const float4* sample_part; // [sample_splits][T]: (max, ...) per split of the sample run, logit units
+  int sample_splits;
   float* ref2;               // [T] out
+  float* xy;                 // [T] out: the target's logit x_t[y_t] / temperature (0 for tokens without one)
   int* flag;                 // cleared here (one int)
 };
+constexpr int kKeepSampleRows = 512;
 
 __global__ __launch_bounds__(256) void keep_reference_kernel(const KeepRefParams p) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -181,7 +189,10 @@ __global__ __launch_bounds__(256) void keep_reference_kernel(const KeepRefParams
   if (t >= p.T) return;
   const long long lab = p.labels[t];
   if (lab < 0 || lab >= p.V) {                 // ignored (-100) or invalid: no gradient, row stored as zeros
-    if (lane == 0) p.ref2[t] = -kNegBig;
+    if (lane == 0) {
+      p.ref2[t] = -kNegBig;
+      p.xy[t] = 0.f;
+    }
     return;
   }
   const u32x4_t* h = (const u32x4_t*)(p.hidden + (long long)t * p.H);
@@ -197,13 +208,19 @@ __global__ __launch_bounds__(256) void keep_reference_kernel(const KeepRefParams
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
-  if (lane == 0) p.ref2[t] = ((acc + (p.bias ? p.bias[lab] : 0.f)) * p.inv_temp + kKeepOffset) * kLog2e;
+  if (lane == 0) {
+    float mx = (acc + (p.bias ? p.bias[lab] : 0.f)) * p.inv_temp;
+    p.xy[t] = mx;
+    for (int k = 0; k < p.sample_splits; ++k) mx = fmaxf(mx, p.sample_part[(long long)k * p.T + t].x);
+    p.ref2[t] = (mx + kKeepOffset) * kLog2e;
+  }
 }
 
 struct KeepPrepParams {
   bf16_t* e;                 // kept numerators, column-blocked (element (t, y_t) is patched)
   long long blk;             // elements between column blocks
   const float* ref2;         // [T]
+  const float* xy;           // [T] target logits (from keep_reference_kernel)
   const long long* labels;   // shifted labels [T]
   const float* lse;          // [T]
   const float* gtok;         // [T]
@@ -225,9 +242,8 @@ __global__ __launch_bounds__(256) void keep_backward_prep_kernel(const KeepPrepP
     const float d2 = p.ref2[t] - p.lse[t] * kLog2e;        // log2 s_t
     a = -c * fast_exp2(d2);
     if (lane == 0) {
-      // p_y - 1 from the fp32 quantities: log p_y = x_y/temperature - lse = (ref - offset) - lse
-      const float lp = (d2 * (1.f / kLog2e)) - kKeepOffset;
-      const float pm1 = expm1f(lp);
+      // p_y - 1 from the fp32 quantities: log p_y = x_y/temperature - lse
+      const float pm1 = expm1f(p.xy[t] - p.lse[t]);
       p.e[(lab >> 8) * p.blk + (long long)t * 256 + (lab & 255)] = f32_to_bf16_rn(pm1 * fast_exp2(-d2));
     }
   }

@@ -26,7 +26,8 @@ PEAK_CLOCK_MHZ = 2400.0
 # --copy-probe.  Not measured in the run that prints it: the figure belongs to the binary and workload named in the
 # profile summary it cites, and is None for workloads that were not profiled.
 PROFILED_TRAFFIC = {
-    # workload: (bytes per launch, summary under profiles/)
+    # (workload, numerators kept): (bytes per launch, summary under profiles/)
+    ("cfg1", True): (3.2489e+10, "profiles/lmhead_fwd_kernel_cfg1_traffic_pmc.txt"),
 }
 
 

@@ -98,16 +98,18 @@ def test_kept_logits_panel_split_matches_single_launch(dev):
 
 
 def test_kept_values_out_of_range_fall_back_to_recomputation(dev):
-    """The kept numerators are exp(x_v - x_target - 40) in bf16: a scored token whose log-probability is below
-    -128 would overflow them.  The forward flags it, and the backward then recomputes: same gradients, bit for
-    bit, as with keep_logits=False; the forward's own outputs never depend on the kept values."""
+    """The kept numerators are exp(x_v - ref - 40) in bf16 with ref = max(target logit, largest logit among the first
+    512 vocabulary entries): a row whose largest logit exceeds both by more than 128 would overflow them.  The
+    forward flags it, and the backward then recomputes: same gradients, bit for bit, as with keep_logits=False;
+    the forward's own outputs never depend on the kept values.  The same dominant entry INSIDE the sampled rows
+    raises no flag."""
     from fgrpo import ops
     T, H, V = 8192, 1024, 8192
     gen = torch.Generator().manual_seed(21)
     hs = torch.ones(T, H).bfloat16()
     W = (torch.randn(V, H, generator=gen) * 0.01).bfloat16()
-    W[7] = 0.25                                        # logit 256 for entry 7 on every row; the targets sit near 0
-    y = torch.randint(8, V, (T,), generator=gen)
+    W[4000] = 0.25                                     # logit 256 for entry 4000 on every row; the targets sit near 0
+    y = torch.randint(8, 3999, (T,), generator=gen)
     adv = torch.randn(T, generator=gen)
     hs_d, W_d, y_d, adv_d = hs.to(dev), W.to(dev), y.to(dev), adv.to(dev)
     lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs_d, W_d, None, y_d, 1.0, keep=True)
@@ -122,6 +124,12 @@ def test_kept_values_out_of_range_fall_back_to_recomputation(dev):
         grads.append((h.grad, w.grad, out[0].detach()))
     assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
     assert torch.equal(grads[0][2], grads[1][2]) and torch.isfinite(grads[0][1].float()).all()
+    # the dominant entry among the sampled rows: the reference follows it, nothing overflows
+    W1 = W.clone()
+    W1[4000] = W[4001]
+    W1[7] = 0.25
+    lp1, _, _, kept1 = ops.lmhead_logprob_fwd(hs_d, W1.to(dev), None, y_d, 1.0, keep=True)
+    assert not ops.keep_overflowed(kept1, T, V) and (lp1 < -128).all()
     # and an ordinary batch does not raise the flag
     W2 = (torch.randn(V, H, generator=gen) * 0.05).bfloat16().to(dev)
     kept2 = ops.lmhead_logprob_fwd(torch.randn(T, H, generator=gen).bfloat16().to(dev), W2, None, y_d, 1.0, keep=True)[3]
