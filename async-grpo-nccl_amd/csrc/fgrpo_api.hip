@@ -1044,7 +1044,7 @@ int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, co
   }
   hipLaunchKernelGGL(grpo_loss_tokens_kernel, dim3(nblocks), dim3(kLossThreads), 0, st, p);
   HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(grpo_loss_finalize_kernel, dim3(nblocks), dim3(kLossThreads), 0, st, p, nblocks);
+  hipLaunchKernelGGL(grpo_loss_finalize_kernel, dim3(std::min(nblocks, kFinalizeBlocks)), dim3(kLossThreads), 0, st, p, nblocks);
   HIP_TRY(hipGetLastError());
   return 0;
 }

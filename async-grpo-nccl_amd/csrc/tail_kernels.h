@@ -129,27 +129,43 @@ __global__ void build_labels_kernel(const long long* ids, const int* tok_off, co
 }
 
 // cu_seqlens from position ids: ordered list of the indices t with pos[t] == 0,
-// followed by T.  A single work-group walks the array in order; within a chunk
-// the rank of a hit is a ballot prefix, so the output order is the token order.
+// followed by T.  A single work-group walks the array in order, eight
+// consecutive tokens per thread and round; the rank of a hit is the prefix of
+// the per-thread counts, so the output order is the token order.
 // out has room for max_out entries; *count receives the number of boundaries
 // found + 1 (even when it exceeds max_out, in which case the tail is dropped).
 __global__ __launch_bounds__(1024) void segment_starts_kernel(const long long* pos, int T, int* out, int max_out,
                                                               int* count) {
+  constexpr int kPer = 8;                    // consecutive tokens per thread and round
   __shared__ int wave_cnt[16];
   __shared__ int base;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   if (threadIdx.x == 0) base = 0;
   __syncthreads();
-  for (int t0 = 0; t0 < T; t0 += 1024) {
-    const int t = t0 + threadIdx.x;
-    const bool hit = (t < T) && (pos[t] == 0);
-    const unsigned long long b = __ballot(hit);
-    const int rank = __popcll(b & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_cnt[wv] = __popcll(b);
+  for (long long t0 = 0; t0 < T; t0 += 1024 * kPer) {
+    const long long first = t0 + (long long)threadIdx.x * kPer;
+    unsigned hits = 0;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      if (first + i < T && pos[first + i] == 0) hits |= 1u << i;
+    const int mine = __popc(hits);
+    // exclusive prefix of the per-thread counts inside the wavefront
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) wave_cnt[wv] = incl;
     __syncthreads();
-    int off = base;
+    int off = base + incl - mine;
     for (int w = 0; w < wv; ++w) off += wave_cnt[w];
-    if (hit && off + rank < max_out) out[off + rank] = t;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      if (hits & (1u << i)) {
+        if (off < max_out) out[off] = (int)(first + i);
+        ++off;
+      }
     __syncthreads();
     if (threadIdx.x == 0) {
       int tot = 0;
@@ -279,7 +295,10 @@ __global__ __launch_bounds__(kLossThreads) void grpo_loss_tokens_kernel(const Lo
 }
 
 // Every block re-derives the totals from the block partials in the same order,
-// then scales its slice of g by the normaliser; block 0 publishes the scalars.
+// then scales its slices of g (a grid-stride walk: the launch holds at most
+// kFinalizeBlocks blocks, so the partials are re-read that many times at most)
+// by the normaliser; block 0 publishes the scalars.
+constexpr int kFinalizeBlocks = 256;
 __global__ __launch_bounds__(kLossThreads) void grpo_loss_finalize_kernel(const LossParams p, int nparts) {
   __shared__ double tot[3];
   if (threadIdx.x < 64) {
@@ -304,8 +323,8 @@ __global__ __launch_bounds__(kLossThreads) void grpo_loss_finalize_kernel(const 
   if (p.denom_override > 0.0) den = p.denom_override;
   if (den < 1.0) den = 1.0;
   const float norm = (float)(1.0 / den);
-  const int t = blockIdx.x * kLossThreads + threadIdx.x;
-  if (t < p.T) p.g[t] *= norm;
+  for (long long t = (long long)blockIdx.x * kLossThreads + threadIdx.x; t < p.T; t += (long long)gridDim.x * kLossThreads)
+    p.g[t] *= norm;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *p.loss = (float)(tot[0] / den);
     if (p.scal) {

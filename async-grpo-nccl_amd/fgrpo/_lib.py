@@ -74,6 +74,9 @@ def load() -> C.CDLL:
         raise RuntimeError(
             f"fgrpo: {LIB_PATH} is missing - build it with `python -m fgrpo.build` "
             "(hipcc --offload-arch=gfx950); there is no CPU or eager fallback")
+    # torch first: the wheel carries its own HIP runtime, and a process must hold one runtime only.  Loaded before
+    # torch, this library would bind the system's runtime while the tensors it is handed live in torch's.
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported

@@ -155,8 +155,8 @@ def parity_gate(w, step_fn, hidden2d, weight, shifted, old, ref, adv, north_star
                                                   p["clip_low"], p["clip_high"], p["clip_ratio_c"])
         want[0].backward()
         res["loss"] = float(loss.detach())
-        res["loss_oracle"] = float(want[0])
-        res["loss_rel_err"] = abs(float(loss.detach()) - float(want[0])) / max(abs(float(want[0])), 1e-30)
+        res["loss_oracle"] = float(want[0].detach())
+        res["loss_rel_err"] = abs(float(loss.detach()) - float(want[0].detach())) / max(abs(float(want[0].detach())), 1e-30)
         g_rows = lp_c.grad[rows].float()
         (want_lp * g_rows).sum().backward()
         got = dH.reshape(T, -1)[rows.to(dH.device)].float().cpu()
@@ -164,6 +164,40 @@ def parity_gate(w, step_fn, hidden2d, weight, shifted, old, ref, adv, north_star
         ok = ok and res["loss_rel_err"] <= 1e-3 and res["dH_rows_cosine"] >= 0.999
     res["passed"] = bool(ok)
     return res
+
+
+def library_yardstick(hidden2d, weight, fwd_only, reps=5):
+    """The vendor library's GEMM (torch.matmul -> hipBLASLt) on the products of the path, same shapes and dtype, on
+    this device right after the timed steps: logits = hidden . weight^T (written as bf16), and for the backward
+    dHidden = logits . weight and dW = logits^T . hidden with the logits standing in for dLogits.  Nothing of the
+    soft-max, the objective or the gather is in these times: they are what the matrix products alone cost through
+    the library, the yardstick for the fused kernels' fractions of peak."""
+    import torch
+    T, H = hidden2d.shape
+    V = weight.shape[0]
+    thv = 2.0 * T * H * V
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        ev[0].record()
+        for i in range(reps):
+            fn()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ms = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(reps))[reps // 2]
+        return {"ms": ms, "tflops": thv / (ms * 1e-3) / 1e12, "frac": thv / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+    logits = torch.empty(T, V, dtype=hidden2d.dtype, device=hidden2d.device)
+    out = {"what": "torch.matmul (hipBLASLt) on the same shapes, matrix products only, median of %d" % reps,
+           "logits": timed(lambda: torch.matmul(hidden2d, weight.t(), out=logits))}
+    if not fwd_only:
+        dh = torch.empty_like(hidden2d)
+        dw = torch.empty_like(weight)
+        out["dhidden"] = timed(lambda: torch.matmul(logits, weight, out=dh))
+        out["dweight"] = timed(lambda: torch.matmul(logits.t(), hidden2d, out=dw))
+        out["sum_ms"] = out["logits"]["ms"] + out["dhidden"]["ms"] + out["dweight"]["ms"]
+    return out
 
 
 def attention_line(args):
@@ -330,6 +364,8 @@ def main():
     ap.add_argument("--config", default="cfg1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check that precedes the timed steps")
+    ap.add_argument("--no-library-yardstick", action="store_true",
+                    help="skip timing the vendor GEMM library on the three products of the path (after the timed steps)")
     ap.add_argument("--objective", choices=["north_star", "reference"], default="north_star",
                     help="north_star: KL to the reference policy + mean over samples of per-sample token means (every "
                          "scored token has a gradient); reference: the reference's own objective, token mean without "
@@ -448,6 +484,10 @@ def main():
     tok_s = T / (ms / 1e3)
     k_ms = sum(a.elapsed_time(b) for a, b in fwd_events) / max(1, len(fwd_events))
 
+    yardstick = None
+    if not args.no_library_yardstick:
+        yardstick = library_yardstick(w.hidden.reshape(T, H).detach(), w.weight.detach(), fwd_only)
+
     if args.copy_probe:
         # a plain device copy of known size, so that one counter run holds the scale of FETCH_SIZE / WRITE_SIZE
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -508,6 +548,7 @@ def main():
                      "kernel_launches_timed": len(fwd_events),
                      "algorithmic_flops_per_launch": thv,
                      "phases": phases, "phase_brackets_dropped": dropped,
+                     "library_yardstick": yardstick,
                      "peak_note": f"published peak = {PEAK_CLOCK_MHZ:.0f} MHz x 256 CUs x 4096 flop/cycle; the clock the "
                                   "device held during the timed steps is under 'clock'"},
         "clock": clock.summary(),
