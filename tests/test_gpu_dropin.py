@@ -113,6 +113,14 @@ def test_segment_kernels(dev):
     pos = torch.cat([torch.arange(n) for n in (5, 1, 300, 64, 1000, 2)])[None].to(dev)
     cu = ops.cu_seqlens_from_position_ids(pos)
     assert torch.equal(cu.cpu(), O.cu_seqlens_from_position_ids(pos.cpu())) and cu.dtype == torch.int32
+    # several rounds of the walk (8192 tokens each), ragged end, dense and sparse hits, and the overflow report
+    gen = torch.Generator().manual_seed(5)
+    for lens in ([1] * 20001, torch.randint(1, 40, (1500,), generator=gen).tolist(), [8192, 8191, 1, 16385], [70001]):
+        pos2 = torch.cat([torch.arange(n) for n in lens])[None].to(dev)
+        got = ops.cu_seqlens_from_position_ids(pos2)
+        assert torch.equal(got.cpu(), O.cu_seqlens_from_position_ids(pos2.cpu())), len(lens)
+    with pytest.raises(RuntimeError, match="max_segments"):
+        ops.cu_seqlens_from_position_ids(pos, max_segments=3)
     vals = torch.randn(6, dtype=torch.float64)
     out = ops.segment_broadcast(vals.to(dev), cu, pos.numel())
     assert torch.equal(out.cpu(), torch.from_numpy(O.broadcast_values(vals.numpy(), [5, 1, 300, 64, 1000, 2])).float())

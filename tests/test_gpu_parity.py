@@ -460,6 +460,38 @@ def test_full_size_properties_and_sampled_rows(dev, name):
     assert col.abs().max().item() <= 1e-2 * dW.float().abs().sum(0).max().item()
 
 
+@pytest.mark.parametrize("mode", ["token_mean", "sample_mean"])
+def test_objective_on_a_million_tokens(dev, mode):
+    """The per-token objective and its normaliser beyond one pass of the normaliser's grid (256 blocks of 256
+    tokens): loss and d loss / d logprob against the oracle's tail on the same [T] vectors."""
+    from fgrpo import ops
+    T = 1_000_003
+    g = torch.Generator().manual_seed(21)
+    lens = []
+    while sum(lens) < T:
+        lens.append(int(torch.randint(1, 9000, (1,), generator=g)))
+    lens[-1] -= sum(lens) - T
+    cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32)
+    y = torch.randint(0, 1000, (T,), generator=g)
+    y[torch.rand(T, generator=g) < 0.3] = -100
+    y[cu[1:].long() - 1] = -100
+    lp = -torch.rand(T, generator=g) * 5
+    old = lp + torch.randn(T, generator=g) * 0.2
+    ref = lp + torch.randn(T, generator=g) * 0.05
+    adv = torch.randn(T, generator=g)
+    lp_o = lp.double().requires_grad_(True)
+    want = O.grpo_objective_from_logprobs(lp_o, y, old.double(), adv.double(), 0.2, 0.28, 3.0, ref.double(), 0.04, mode, cu)
+    want[0].backward()
+    lp_g = lp.to(dev).requires_grad_(True)
+    got = ops.grpo_loss_from_logprobs(lp_g, y.to(dev), old.to(dev), adv.to(dev), ref.to(dev), cu.to(dev), 0.2, 0.28, 3.0,
+                                      0.04, mode)
+    got[0].backward()
+    assert abs(got[0].item() - want[0].item()) <= 1e-5 * max(1.0, abs(want[0].item()))
+    scale = lp_o.grad.abs().max().item()
+    assert (lp_g.grad.cpu().double() - lp_o.grad).abs().max().item() <= 1e-5 * scale
+    assert (got[1].cpu().double() - want[1].detach()).abs().max().item() <= 1e-6
+
+
 def test_step_is_capturable_in_a_hip_graph(dev):
     """The library allocates nothing, synchronises nothing and clears its scratch with fill kernels, so a whole
     small step (projection + logprob, objective, backward) can be captured once and replayed: launch-bound sizes
