@@ -300,22 +300,30 @@ __global__ __launch_bounds__(kLossThreads) void grpo_loss_tokens_kernel(const Lo
 // by the normaliser; block 0 publishes the scalars.
 constexpr int kFinalizeBlocks = 256;
 __global__ __launch_bounds__(kLossThreads) void grpo_loss_finalize_kernel(const LossParams p, int nparts) {
+  __shared__ double part[3][kLossThreads / 64];
   __shared__ double tot[3];
-  if (threadIdx.x < 64) {
+  {
+    // all four wavefronts add their strided share, then one thread adds the four results: a fixed order
     double a = 0.0, b = 0.0, ne = 0.0;
-    for (int i = threadIdx.x; i < nparts; i += 64) {
+    for (int i = threadIdx.x; i < nparts; i += kLossThreads) {
       a += p.partial[2 * i];
       b += p.partial[2 * i + 1];
     }
     if (p.seg_cnt)
-      for (int i = threadIdx.x; i < p.nseq; i += 64) ne += (p.seg_cnt[i] > 0) ? 1.0 : 0.0;
+      for (int i = threadIdx.x; i < p.nseq; i += kLossThreads) ne += (p.seg_cnt[i] > 0) ? 1.0 : 0.0;
     a = wave_sum_d(a);
     b = wave_sum_d(b);
     ne = wave_sum_d(ne);
-    if (threadIdx.x == 0) {
-      tot[0] = a;
-      tot[1] = b;
-      tot[2] = ne;
+    if ((threadIdx.x & 63) == 0) {
+      part[0][threadIdx.x >> 6] = a;
+      part[1][threadIdx.x >> 6] = b;
+      part[2][threadIdx.x >> 6] = ne;
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+      double t = 0.0;
+      for (int w = 0; w < kLossThreads / 64; ++w) t += part[threadIdx.x][w];
+      tot[threadIdx.x] = t;
     }
   }
   __syncthreads();
