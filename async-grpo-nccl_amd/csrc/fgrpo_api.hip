@@ -298,7 +298,7 @@ int run_store_gemm_kmajor(const Tuning& tn, StoreParams p, bool akm, bool bkm, h
   {
     // group_m_auto: > 0 that many row tiles per raster group, < 0 row tiles dealt round-robin to the XCDs,
     // 0 the tuning default; a tuning key set for this GEMM overrides it
-    const int own = (akm && bkm) ? tn.dw_group_m : tn.dh_group_m;
+    const int own = akm ? tn.dw_group_m : tn.dh_group_m;
     p.group_m = own > 0 ? own : group_m_auto > 0 ? group_m_auto : group_m_auto < 0 ? 0 : (tn.gemm_group_m > 0 ? tn.gemm_group_m : 1);
   }
   p.wide_stores = can_store_wide(tn, p);
@@ -814,7 +814,7 @@ struct KeptBwdPlan {
   float* row_scale;       // [T]
   int* k_runs;            // live runs of the token axis for the dW product
   int* m_tile_live;       // live 256-row tiles for the dH product
-  bf16_t* hidden_scaled;  // [T x H]
+  bf16_t* hidden_scaled;  // [H x Tpad]: diag(a) hidden, transposed (the token contiguous), zero from T to Tpad
   float* dh_acc;          // [T x H] fp32, panels > 1 only
   size_t bytes;
 };
@@ -823,7 +823,7 @@ void plan_kept_bwd(KeptBwdPlan& pl, void* ws, int T, int H) {
   pl.row_scale = cv.take<float>((size_t)T);
   pl.k_runs = cv.take<int>((size_t)(2 + 2 * kRunCap));
   pl.m_tile_live = cv.take<int>((size_t)((T + 255) / 256));
-  pl.hidden_scaled = cv.take<bf16_t>((size_t)T * H);
+  pl.hidden_scaled = cv.take<bf16_t>((size_t)H * round_up(T, 256));
   pl.dh_acc = cv.take<float>((size_t)T * H);     // always sized: a concurrent set_tuning must not make it short
   pl.bytes = cv.total();
 }
@@ -876,9 +876,12 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
   {
     PhaseScope ph(kPhaseDlogits, st);
     KeepPrepParams k{ek, blk, keep_ref2_of(logits_keep, T, V), keep_xy_of(logits_keep, T, V), (const long long*)labels, lse, g, gout_dev, inv_temp,
-                     (const bf16_t*)hidden, T, H, V, pl.row_scale, dW_out ? pl.hidden_scaled : nullptr};
+                     (const bf16_t*)hidden, T, H, V, pl.row_scale};
     hipLaunchKernelGGL(keep_backward_prep_kernel, dim3((T + 3) / 4), dim3(256), 0, st, k);
     HIP_TRY(hipGetLastError());
+    if (dW_out)
+      hipLaunchKernelGGL(keep_scaled_transpose_kernel, dim3(Tpad / 64, H / 64), dim3(256), 0, st, (const bf16_t*)hidden,
+                         (const float*)pl.row_scale, T, H, Tpad, pl.hidden_scaled);
     if (skip_dead) {
       KeepLiveParams lv{pl.row_scale, T, (T + 63) / 64, Tpad / 64, pl.k_runs, pl.m_tile_live};
       hipLaunchKernelGGL(keep_live_runs_kernel, dim3(1), dim3(1024), 0, st, lv);
@@ -922,24 +925,25 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       }
       if (rc) return rc;
     }
-    if (dW_out) {   // dW[v0 : v0+rows, H] = E'^T[rows x Tpad] (diag(a) hidden)[Tpad x H]: the token is the contraction row of both
+    if (dW_out) {   // dW[v0 : v0+rows, H] = E'^T[rows x Tpad] (diag(a) hidden)^T[H x Tpad]^T: A read where the forward left it
+                    // (the token is its row), B a token-contiguous copy, so that only A needs transposing LDS reads
       StoreParams s;
       memset(&s, 0, sizeof(s));
       s.g.M = rows;
       s.g.N = H;
       s.g.lda = 256;
       s.g.a_blk = blk;
-      s.g.ldb = H;
+      s.g.ldb = Tpad;
       s.g.nseg = 1;
       s.g.seg[0] = GemmSeg{ek_p, pl.hidden_scaled, Tpad};
-      s.g.kb_valid = T;
+      s.g.ka_valid = T;
       s.g.k_runs = skip_dead ? pl.k_runs : nullptr;
       s.ldc = H;
       s.alpha = 1.f;
       s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
       {
         PhaseScope ph(kPhaseDw, st);
-        rc = run_store_gemm_kmajor(tn, s, true, true, st, 1);
+        rc = run_store_gemm_kmajor(tn, s, true, false, st, 1);
       }
       if (rc) return rc;
     }

@@ -61,7 +61,7 @@ struct GemmOperands {
   // down the rows of one block (K-major use) then reads one sequential stream, and a tile that walks along
   // the columns (K-contiguous use) reads 128 KiB contiguous pieces.
   long long a_blk;
-  // gemm_mainloop_km with both operands K-major only: the contraction may skip whole K steps (64 rows each) that
+  // gemm_mainloop_km with a K-major A only: the contraction may skip whole K steps (64 rows each) that
   // are known to contribute nothing.  k_runs (device memory, written by an earlier launch on the stream) =
   // {number of runs R, K steps in all runs, start_0 .. start_{kRunCap-1}, end_0 .. end_{kRunCap-1}}: run r covers
   // the K steps start_r <= k < end_r, runs ascending and disjoint.  Null = every K step.
@@ -869,9 +869,9 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   uint32_t ka = 0, kb = 0;                      // running K byte offset of a K-contiguous operand
   const int dst_w = wave * 1024;                // both layouts: one load fills 1 KiB, loads i are NW KiB apart
 
-  // run list (both operands K-major only): the issue cursor walks the listed K steps; the compute side never
+  // run list (A K-major; B either way): the issue cursor walks the listed K steps; the compute side never
   // knows, it consumes LDS buffers in the order they were filled
-  const int* runs = (AKM && BKM) ? g.k_runs : nullptr;
+  const int* runs = AKM ? g.k_runs : nullptr;
   const int n_runs = runs ? runs[0] : 0;
   const int nk_total = runs ? runs[1] : g.seg[0].K / C::BK;
   int run_idx = 0, run_left = 0, cur_step = 0;
@@ -879,11 +879,15 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
     cur_step = runs[2];
     run_left = runs[2 + kRunCap] - cur_step;
     Ap += (long long)cur_step * C::BK * lda2;
-    Bp += (long long)cur_step * C::BK * ldb2;
     a_rem -= (long long)cur_step * C::BK;
-    b_rem -= (long long)cur_step * C::BK;
     rsa = make_rsrc(Ap, bytes_of(a_rem, lda2, a_col));
-    rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2, b_col));
+    if constexpr (BKM) {
+      Bp += (long long)cur_step * C::BK * ldb2;
+      b_rem -= (long long)cur_step * C::BK;
+      rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2, b_col));
+    } else {
+      kb = (uint32_t)cur_step * C::BK * 2;
+    }
   }
   const long long a_blk_bytes = (!AKM) ? g.a_blk * 2 : 0;
   int ablk_left = 256 / C::BK;
@@ -897,7 +901,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
                                                (int)boff[idx - C::PA], (int)kb, 0, FGRPO_DMA_AUX);
     if (idx == LPT - 1) {                        // next K step
       long long jump = 1;                        // K steps from this one to the next one to fetch
-      if constexpr (AKM && BKM) {
+      if constexpr (AKM) {
         if (runs != nullptr && --run_left == 0 && run_idx + 1 < n_runs) {   // this run is done: on to the next
           ++run_idx;
           const int s = runs[2 + run_idx];
@@ -926,7 +930,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
         b_rem -= jump * C::BK;
         rsb = make_rsrc(Bp, bytes_of(b_rem, ldb2, b_col));
       } else {
-        kb += C::BK * 2;
+        kb += (uint32_t)jump * C::BK * 2;
       }
     }
   };

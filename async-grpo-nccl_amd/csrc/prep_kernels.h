@@ -229,7 +229,6 @@ struct KeepPrepParams {
   const bf16_t* hidden;      // [T][H]
   int T, H, V;
   float* row_scale;          // [T] out: a_t
-  bf16_t* hidden_scaled;     // [T][H] out: a_t * hidden[t], or null
 };
 
 __global__ __launch_bounds__(256) void keep_backward_prep_kernel(const KeepPrepParams p) {
@@ -248,17 +247,41 @@ __global__ __launch_bounds__(256) void keep_backward_prep_kernel(const KeepPrepP
     }
   }
   if (lane == 0) p.row_scale[t] = a;
-  if (p.hidden_scaled) {
-    const u32x4_t* h = (const u32x4_t*)(p.hidden + (long long)t * p.H);
-    u32x4_t* o = (u32x4_t*)(p.hidden_scaled + (long long)t * p.H);
-    for (int cidx = lane; cidx < p.H / 8; cidx += 64) {
-      const u32x4_t v = h[cidx];
-      u32x4_t r;
+}
+
+// B operand of the dW product, contraction-contiguous: out[h][t] = a_t * hidden[t][h] for t < T, zero up to Tpad
+// (the contraction runs over whole 64-token steps; the kept buffer's rows past T read as zero, and zero times a
+// stale value must not be a NaN).  64 x 64 tiles through LDS; H % 64 == 0, Tpad % 64 == 0.
+__global__ __launch_bounds__(256) void keep_scaled_transpose_kernel(const bf16_t* hidden, const float* row_scale, int T,
+                                                                    int H, int Tpad, bf16_t* out) {
+  __shared__ uint16_t tile[64][66];
+  const int t0 = blockIdx.x * 64, h0 = blockIdx.y * 64;
+  const int r = threadIdx.x >> 3, cidx = threadIdx.x & 7;
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        r[e] = pack_bf16x2(a * __uint_as_float(v[e] << 16), a * __uint_as_float(v[e] & 0xffff0000u));
-      o[cidx] = r;
+  for (int half = 0; half < 2; ++half) {
+    const int tl = r + 32 * half, t = t0 + tl;
+    u32x4_t v = {0u, 0u, 0u, 0u};
+    float a = 0.f;
+    if (t < T) {
+      v = *(const u32x4_t*)(hidden + (long long)t * H + h0 + 8 * cidx);
+      a = row_scale[t];
     }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t pk = pack_bf16x2(a * __uint_as_float(v[e] << 16), a * __uint_as_float(v[e] & 0xffff0000u));
+      tile[tl][8 * cidx + 2 * e] = (uint16_t)(pk & 0xffffu);
+      tile[tl][8 * cidx + 2 * e + 1] = (uint16_t)(pk >> 16);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int hl = r + 32 * half;
+    u32x4_t o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      o[e] = (uint32_t)tile[8 * cidx + 2 * e][hl] | ((uint32_t)tile[8 * cidx + 2 * e + 1][hl] << 16);
+    *(u32x4_t*)(out + (long long)(h0 + hl) * Tpad + t0 + 8 * cidx) = o;
   }
 }
 

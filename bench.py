@@ -513,7 +513,7 @@ def main():
     if not fwd_only:
         if kept:
             phases.append(phase("keep_backward_prep_kernel", phase_ms["dlogits"], 0.0,
-                                "per-token factors, one patched element per row, scaled copy of hidden "
+                                "per-token factors, one patched element per row, scaled transposed copy of hidden "
                                 f"({4.0 * T * H / 1e6:.0f} MB): no pass over [T x V]"))
         else:
             phases.append(phase(f"lmhead_ds_kernel x {phase_n['dlogits'] // args.steps} panels (recomputes the logits)",

@@ -117,7 +117,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
  * caller must then use fgrpo_lmhead_bwd.  Rows of ignored tokens are stored as exact zeros.
  * logits_keep: fgrpo_logits_keep_bytes(T, V) bytes, 16-byte aligned: [ceil(V/256)][round_up(T,256)][256] bf16,
  * then the references and the flag.  workspace of the backward: fgrpo_lmhead_bwd_kept_workspace bytes (the token
- * factors, the scaled copy of hidden, and an fp32 dH accumulator used only when the tuning key keep_panels splits
+ * factors, the scaled transposed copy of hidden, and an fp32 dH accumulator used only when the tuning key keep_panels splits
  * the products into vocabulary panels).
  * Supported (fgrpo_keep_supported() != 0): bf16, H a multiple of 64, enough tiles to fill the device; anything
  * else returns FGRPO_ERR_UNSUPPORTED - use the recomputing pair.  dH_out / dW_out / dbias_out as in
