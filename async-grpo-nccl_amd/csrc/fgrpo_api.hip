@@ -211,7 +211,13 @@ void plan_fwd(const Tuning& tn, FwdPlan& pl, void* ws, int T, int H, int V, int 
   const CfgInfo& c = kCfg[pl.variant];
   pl.tiles_v = (V + c.bm - 1) / c.bm;
   pl.tiles_t = (T + c.bn - 1) / c.bn;
-  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu, tn.fwd_nsplit);
+  // A work-group keeps its token tile and re-reads that tile's hidden slab for every vocabulary tile it walks; with
+  // four splits the device works on 8 XCDs x 8 token tiles = 16384 rows of hidden at a time.  From H = 6144 on that is
+  // more than 192 MB and no longer stays in the 256 MB cache in front of HBM next to the W stream: eight splits
+  // (4 token tiles per XCD) halve it (T=16384, H=8192, V=128256: 28.9 -> 24.9 ms; H=5120 and 3584 measure equal
+  // or better with four).
+  const int prefer = (16384LL * H * 2 > (192LL << 20)) ? 8 : 4;
+  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu, tn.fwd_nsplit, prefer);
   pl.Hp = (int)round_up(H, 64);
   pl.copy_ops = (dtype == FGRPO_F32) || (H % 64 != 0);
   Carver cv(ws);
@@ -298,8 +304,16 @@ int run_store_gemm_kmajor(const Tuning& tn, StoreParams p, bool akm, bool bkm, h
   {
     // group_m_auto: > 0 that many row tiles per raster group, < 0 row tiles dealt round-robin to the XCDs,
     // 0 the tuning default; a tuning key set for this GEMM overrides it
+    // Either way the 32 work-groups an XCD runs side by side should form a patch of row tiles x column tiles that is
+    // not a sliver: with more than 8 column tiles (H > 2048) a single row tile's columns would fill the XCD and
+    // every work-group would fetch a B slice of its own (measured at T=16384, H=8192, V=128256: 139 / 143 GB past
+    // the L2s for dHidden / dW against 53-66 GB for the vendor library's kernels), so 4 row tiles x 8 columns then.
     const int own = akm ? tn.dw_group_m : tn.dh_group_m;
-    p.group_m = own > 0 ? own : group_m_auto > 0 ? group_m_auto : group_m_auto < 0 ? 0 : (tn.gemm_group_m > 0 ? tn.gemm_group_m : 1);
+    const int wide = p.tiles_n > 8;
+    if (group_m_auto > 0 && wide) group_m_auto = 4;
+    p.group_m = own > 0 ? own : group_m_auto > 0 ? group_m_auto : group_m_auto < 0 ? 0 : (tn.gemm_group_m > 0 ? tn.gemm_group_m : (wide ? 4 : 1));
+    p.rr_cols = wide ? 8 : p.tiles_n;
+    p.rr_rows = wide ? 4 : 1;
   }
   p.wide_stores = can_store_wide(tn, p);
   p.nblocks = p.group_m > 0 ? p.tiles_m * p.tiles_n : 8 * ((p.tiles_m + 7) / 8) * p.tiles_n;
@@ -490,6 +504,7 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   p.tiles_t = pl.tiles_t;
   p.nsplit = pl.nsplit;
   p.group_t = tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
+  if (pl.nsplit >= 8 && p.group_t * pl.nsplit > 32) p.group_t = 32 / pl.nsplit > 0 ? 32 / pl.nsplit : 1;   // one XCD's 32 work-groups per patch
   p.part = pl.part;
   p.xt = pl.xt;
   if (keep) {

@@ -522,6 +522,7 @@ struct StoreParams {
   const float* alpha_dev;  // optional device scalar multiplied into alpha
   int tiles_m, tiles_n, group_m;   // group_m == 0: row tiles dealt round-robin to the XCDs (see gemm_store_kernel)
   int nblocks;                     // work-groups to launch (set by the launcher's caller)
+  int rr_rows, rr_cols;            // patch of the round-robin raster (group_m == 0): row tiles of the XCD x column tiles
   int wide_stores;         // ldc and the output / addend bases allow 16-byte pieces (set by the launcher)
   const float* row_scale;  // optional [M]: output row m is multiplied by row_scale[m] (after alpha, before c_in)
   const int* m_tile_live;  // optional [tiles_m] (BM = 256 rows per tile): 0 = every row of the tile has row_scale 0,
@@ -654,12 +655,22 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
     tm = first_m + w % gsz;
     tn = w / gsz;
   } else {
-    // row tiles dealt round-robin to the XCDs (work-group b runs on XCD b % 8), all column tiles of a row tile side
-    // by side on one XCD: neighbouring row tiles - which are dead or alive together when whole samples carry no
-    // gradient - land on different XCDs, so skipped tiles thin every XCD's share instead of emptying some
+    // row tiles dealt round-robin to the XCDs (work-group b runs on XCD b % 8): neighbouring row tiles - which are
+    // dead or alive together when whole samples carry no gradient - land on different XCDs, so skipped tiles thin
+    // every XCD's share instead of emptying some.  Inside an XCD the tiles come in patches of rr_rows of its row
+    // tiles x rr_cols column tiles (rr_rows * rr_cols = the XCD's 32 CUs; all column tiles when there are at most
+    // 8), rows fastest: the 32 work-groups running side by side share rr_rows A slices and rr_cols B slices.
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    tm = (idx / p.tiles_n) * 8 + xcd;
-    tn = idx % p.tiles_n;
+    const int rows_x = (p.tiles_m + 7) >> 3;                       // row tiles an XCD owns (the last ones may not exist)
+    const int per_group = p.rr_rows * p.tiles_n;
+    const int grp = idx / per_group;
+    const int first = grp * p.rr_rows;
+    const int gsz = (rows_x - first) < p.rr_rows ? (rows_x - first) : p.rr_rows;
+    const int w = idx - grp * per_group;
+    const int chunk = w / (gsz * p.rr_cols);                       // full column chunks before this one
+    const int w2 = w - chunk * gsz * p.rr_cols;
+    tm = (first + w2 % gsz) * 8 + xcd;
+    tn = chunk * p.rr_cols + w2 / gsz;
     if (tm >= p.tiles_m) return;
   }
   const int row0 = tm * C::BM, col0 = tn * C::BN;
