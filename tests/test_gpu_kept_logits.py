@@ -190,6 +190,35 @@ def test_rows_without_gradient_are_skipped_exactly(dev, pattern):
         assert cos(res[1][0], dH0) >= 0.9999 and cos(res[1][1], dW0) >= 0.9999
 
 
+@pytest.mark.parametrize("tokens", [4321, 13 * 256 + 17])
+def test_wide_hidden_takes_the_patch_rasters(dev, tokens):
+    """More than 8 column tiles (H = 2560: 10): the gradient GEMMs walk 4 x 8 tile patches per XCD - the grouped
+    raster for dW, the round-robin one for dHidden when dead rows are skipped - with row-tile counts that are no
+    multiple of the patch.  Against the oracle, and skipping against not skipping bit for bit."""
+    from fgrpo import _lib, ops
+    w = filling_workload(18, H=2560, V=4200, tokens=tokens, len_hi=500)
+    assert ops.keep_supported(w.T, w.H, w.V, torch.bfloat16)
+    want, got, o, g_, _, _ = run_case(w, dev, "north_star", keep_logits=True)
+    check(want, got, o, g_, f32=False)
+    T = w.T
+    hs, W = w.hidden.reshape(T, w.H).to(dev), w.weight.to(dev)
+    y = ops.shift_labels(w.labels.to(dev)).reshape(-1)
+    g = torch.randn(T, generator=torch.Generator().manual_seed(6)).to(dev) / T
+    for a, b in ((0, 300), (1000, 2600), (T - 700, T - 3)):
+        g[a:b] = 0
+    lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
+    res = {}
+    for skip in (1, 0):
+        _lib.set_tuning(keep_skip_dead=skip)
+        try:
+            res[skip] = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
+        finally:
+            _lib.set_tuning(keep_skip_dead=1)
+    assert torch.equal(res[1][0], res[0][0]) and torch.equal(res[1][1], res[0][1])
+    dH0, dW0, _ = ops.lmhead_bwd(hs, W, None, y, lse, g, None, 1.0, True, True, False, 0)
+    assert cos(res[1][0], dH0) >= 0.9999 and cos(res[1][1], dW0) >= 0.9999
+
+
 def test_keep_refuses_what_it_cannot_do(dev):
     from fgrpo import ops
     hs = torch.randn(512, 192, device=dev).bfloat16()
