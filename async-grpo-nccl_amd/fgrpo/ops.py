@@ -206,8 +206,9 @@ def lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torc
 
 
 def keep_overflowed(kept: torch.Tensor, T: int, V: int) -> bool:
-    """True when the forward flagged that the kept values may have overflowed (a scored token whose log-probability
-    is below -128): the caller must then take the recomputing backward.  Waits for the current stream."""
+    """True when the forward flagged that the kept values may have overflowed (a logit more than 123 log-probability
+    units above both the target logit and the largest logit of the first 512 vocabulary rows): the caller must then
+    take the recomputing backward.  Waits for the current stream."""
     with torch.cuda.device(kept.device):
         rc = _lib.load().fgrpo_keep_overflowed(_ptr(kept), int(T), int(V), _stream())
     if rc < 0:

@@ -112,9 +112,10 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
  * the factor in the epilogue, dW = E'^T (diag(a) hidden)): 6 instead of 8 T*H*V products per step.  The buffer
  * survives the backward (a second backward may reuse it).  lp / entropy / lse are computed as in
  * fgrpo_logprob_fwd and are bit-identical to its results.
- * Range: E holds p_v / p_y * exp(-40) in bf16, finite as long as log p_y > -128 for every scored token; the
- * forward raises a flag in the buffer otherwise, fgrpo_keep_overflowed() reads it (it waits for `stream`), and the
- * caller must then use fgrpo_lmhead_bwd.  Rows of ignored tokens are stored as exact zeros.
+ * Range: E[t][v] = exp(x_tv / temperature - ref_t) in bf16 with ref_t = max(target logit, largest logit among the
+ * first 512 vocabulary rows) / temperature + 40: finite as long as no logit of a scored token lies more than 123
+ * (in units of log probability) above that maximum; the forward raises a flag in the buffer otherwise,
+ * fgrpo_keep_overflowed() reads it (it waits for `stream`), and the caller must then use fgrpo_lmhead_bwd.  Rows of ignored tokens are stored as exact zeros.
  * logits_keep: fgrpo_logits_keep_bytes(T, V) bytes, 16-byte aligned: [ceil(V/256)][round_up(T,256)][256] bf16,
  * then the references and the flag.  workspace of the backward: fgrpo_lmhead_bwd_kept_workspace bytes (the token
  * factors, the scaled transposed copy of hidden, and an fp32 dH accumulator used only when the tuning key keep_panels splits
