@@ -292,6 +292,23 @@ def test_output_indices_are_the_scored_positions():
     assert scored.tolist() == oi.tolist()
 
 
+def test_projection_and_segment_ids_by_hand():
+    """The two helpers every other oracle function goes through: the projection (grpo_loss.py:227-230) against a
+    hand-expanded sum, with bias and temperature; segment ids of a cu_seqlens vector with an empty segment."""
+    W = torch.tensor([[1.0, 2.0], [0.5, -1.0], [3.0, 0.0]], dtype=torch.float64)       # [V=3, H=2]
+    b = torch.tensor([0.1, -0.2, 0.3], dtype=torch.float64)
+    hs = torch.tensor([[[2.0, -1.0], [0.0, 4.0]]], dtype=torch.float64)                # [1, 2, 2]
+    got = O.project(W, b, hs, 0.5)
+    want = torch.tensor([[[(2 * 1 - 1 * 2 + 0.1) / 0.5, (2 * 0.5 + 1 * 1 - 0.2) / 0.5, (2 * 3 + 0 + 0.3) / 0.5],
+                          [(0 + 4 * 2 + 0.1) / 0.5, (0 - 4 - 0.2) / 0.5, (0 + 0 + 0.3) / 0.5]]], dtype=torch.float64)
+    assert torch.allclose(got, want, rtol=0, atol=1e-12)
+    assert torch.equal(O.project(W, None, hs, 1.0), torch.einsum("blh,vh->blv", hs, W))
+    # hidden states arrive in another dtype than the weights: cast to the weights' first (grpo_loss.py:227)
+    assert O.project(W.float(), None, hs, 1.0).dtype == torch.float32
+    seg = O.segment_ids_from_cu_seqlens(torch.tensor([0, 2, 2, 5], dtype=torch.int32), 5)
+    assert seg.tolist() == [0, 0, 2, 2, 2]
+
+
 def test_cu_seqlens_from_position_ids():
     pos = torch.tensor([[0, 1, 2, 0, 1, 0, 1, 2, 3]])
     cu = O.cu_seqlens_from_position_ids(pos)
