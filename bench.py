@@ -493,7 +493,10 @@ def main():
 
     yardstick = None
     if not args.no_library_yardstick:
-        yardstick = library_yardstick(w.hidden.reshape(T, H).detach(), w.weight.detach(), fwd_only)
+        try:        # a comparison beside the measurement: its failure must not cost the line
+            yardstick = library_yardstick(w.hidden.reshape(T, H).detach(), w.weight.detach(), fwd_only)
+        except Exception as e:      # noqa: BLE001
+            yardstick = {"error": f"{type(e).__name__}: {e}"[:300]}
 
     if args.copy_probe:
         # a plain device copy of known size, so that one counter run holds the scale of FETCH_SIZE / WRITE_SIZE
