@@ -107,6 +107,35 @@ __device__ __forceinline__ int acc_col(int wn, int j, int lane) {
   return wn * C::WTN + j * 32 + (lane & 31);
 }
 
+// The 256x256x64 two-buffer direct-to-LDS loops of the 8-wavefront tile can run on v_mfma_f32_16x16x32_bf16 instead
+// of 32x32x16 (kMi16): same flops per cycle, half the fp32 accumulator registers read and written per flop - on this
+// power-limited part the same kernels run 6-10 % faster with it.  A 32x32 block (i, j) of a wavefront is then four
+// 16x16 blocks (rh, ch), each one MFMA per 32-wide K slice, and the block's sixteen accumulator registers are
+//   element e = 4*(2*rh + ch) + r :  row = wm*WTM + i*32 + 16*rh + 4*(lane/16) + r
+//                                   col = wn*WTN + j*32 + 16*ch + (lane%16)
+// relative to the tile origin.
+template <class C>
+constexpr bool kMi16 = C::DMA && C::NSTAGE == 2 && C::NW == 8 && C::BK == 64 && C::TM == 4 && C::TN == 2;
+template <class C>
+__device__ __forceinline__ int acc16_row(int wm, int i, int e, int lane) {
+  return wm * C::WTM + i * 32 + 16 * (e >> 3) + 4 * (lane >> 4) + (e & 3);
+}
+template <class C>
+__device__ __forceinline__ int acc16_col(int wn, int j, int e, int lane) {
+  return wn * C::WTN + j * 32 + 16 * ((e >> 2) & 1) + (lane & 15);
+}
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+// acc<registers 4Q .. 4Q+3> += a (16 rows x 32 k) * b (16 columns x 32 k)
+template <int Q>
+__device__ __forceinline__ void mfma16_slice(bf16x8_t a, bf16x8_t b, f32x16_t& c) {
+  f32x4_t t = __builtin_shufflevector(c, c, 4 * Q, 4 * Q + 1, 4 * Q + 2, 4 * Q + 3);
+  t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, t, 0, 0, 0);
+  c[4 * Q] = t[0];
+  c[4 * Q + 1] = t[1];
+  c[4 * Q + 2] = t[2];
+  c[4 * Q + 3] = t[3];
+}
+
 template <class C>
 __device__ __forceinline__ void zero_acc(f32x16_t (&acc)[C::TM][C::TN]) {
 #pragma unroll
@@ -431,6 +460,127 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
   wg_barrier();                                       // LDS may be reused by the caller
 }
 
+// The same schedule on 16x16x32 MFMAs (kMi16 tiles: TM = 4, TN = 2, BK = 64).  A K step is still four sub-steps of
+// equal length: sub-step kk works on the 32-wide K slice k2 = kk/2 and on the row half rh = kk%2 of every 32x32
+// block - 16 MFMAs: for each block row i the fragment a(i, rh) (16 rows x 32 k) against the four fragments
+// b(j, ch) (16 columns x 32 k) of the slice.  The b fragments of a slice are fetched once, before its first
+// sub-step, and serve both; so the fragment requests alternate between 4 (a only, before an odd sub-step) and
+// 8 (a0, the four b, a1 .. a3, before an even one).
+//   load_a(stage_ptr, I, KK): fragment a(I, KK % 2) of slice KK / 2;  load_b(stage_ptr, JC, K2): fragment b(JC/2, JC%2).
+template <class C, int LPT, int RA, int RB, class IssueOne, class LoadA, class LoadB>
+__device__ __forceinline__ void early_barrier_pipeline16(int nk_total, char* smem, f32x16_t (&acc)[C::TM][C::TN],
+                                                         IssueOne&& issue_one, LoadA&& load_a, LoadB&& load_b) {
+  constexpr int KK = 4;
+  constexpr int TM = C::TM, NB = 2 * C::TN;           // a fragments per sub-step, b fragments per K slice
+  static_assert(kMi16<C> && C::BK == 64, "16x16x32 schedule: 8-wavefront 256x256x64 tile");
+  constexpr int NSLOT = kLoadPhases * TM;
+  // request list of a sub-step by its parity P (0: a0, b0 .. b(NB-1), a1 ..; 1: a0 .. a(TM-1)), all compile time
+  struct Ord {
+    static constexpr int nr(int P) { return P == 0 ? TM + NB : TM; }
+    static constexpr int cost(int P, int e) { return P == 0 ? ((e == 0 || e > NB) ? RA : RB) : RA; }
+    static constexpr int instrs(int P, int n) {
+      int c = 0;
+      for (int e = 0; e < n; ++e) c += cost(P, e);
+      return c;
+    }
+    static constexpr int cum(int P, int i) { return (i * nr(P) + TM - 1) / TM; }     // entries requested before row group i starts
+    static constexpr int need(int P, int i) { return P == 0 ? (i == 0 ? NB : NB + i) : i; }   // last entry row group i waits for
+    // LDS instructions that may still be outstanding when row group i of a sub-step of parity P starts
+    static constexpr int allowed(int P, int i, bool issuing) {
+      return instrs(P, nr(P)) - instrs(P, need(P, i) + 1) + (issuing ? instrs(1 - P, cum(1 - P, i)) : 0);
+    }
+  };
+  FGRPO_WAIT_VMCNT(0);
+  wg_barrier();                                       // step 0 is in buffer 0
+  int steps_issued = nk_total > 0 ? 1 : 0;
+  bool active = steps_issued < nk_total;              // a step is being loaded
+  int tgt = 1;                                        // ... into this buffer
+  if (active) {
+    ++steps_issued;
+    static_for<LPT>([&](auto q) {
+      if constexpr (decltype(q)::value * NSLOT / LPT < TM) issue_one(1, decltype(q)::value);  // phase 0's share
+    });
+  }
+  bf16x8_t af[2][TM], bfr[2][NB];
+  // entry e of the request list of sub-step KN, read from the buffer at `base`
+  auto request = [&](const char* base, auto ec, auto knc) {
+    constexpr int e = decltype(ec)::value, kn = decltype(knc)::value;
+    if constexpr ((kn & 1) == 1) {
+      af[1][e] = load_a(base, ec, knc);
+    } else if constexpr (e == 0) {
+      af[0][0] = load_a(base, std::integral_constant<int, 0>{}, knc);
+    } else if constexpr (e <= NB) {
+      bfr[(kn >> 1) & 1][e - 1] = load_b(base, std::integral_constant<int, e - 1>{}, std::integral_constant<int, (kn >> 1)>{});
+    } else {
+      af[0][e - NB] = load_a(base, std::integral_constant<int, e - NB>{}, knc);
+    }
+  };
+  static_for<Ord::nr(0)>([&](auto e) { request(smem, e, std::integral_constant<int, 0>{}); });
+  int cur = 0;
+  auto step = [&](int kt, auto steady_c) {
+    constexpr bool STEADY = decltype(steady_c)::value;
+    const char* st = smem + cur * C::STAGE;
+    const char* sn = smem + (cur ^ 1) * C::STAGE;
+    const bool next = STEADY || kt + 1 < nk_total;
+    static_for<KK>([&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value;
+      constexpr bool last = (kk == KK - 1);
+      constexpr int kn = last ? 0 : kk + 1;
+      constexpr int P = kk & 1, k2 = kk >> 1;
+      const char* src = last ? sn : st;
+      const bool issuing = STEADY || !last || next;
+      if constexpr (last) {
+        if (next) {
+          FGRPO_WAIT_VMCNT_LGKM0(0);                  // my loads of step kt+1 landed; my reads of `cur` returned
+          wg_barrier();
+          active = STEADY || steps_issued < nk_total; // loads of step kt+2 go into the buffer just freed
+          tgt = cur;
+          if (active) ++steps_issued;
+        }
+      }
+      constexpr int phase = last ? 0 : kk + 1;
+      const bool loads_here = STEADY || (active && phase < kLoadPhases && (phase > 0 || next));
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (!last) {
+          wait_lgkm<Ord::allowed(P, i, true)>();
+        } else {
+          if (next) wait_lgkm<Ord::allowed(P, i, true)>(); else wait_lgkm<Ord::allowed(P, i, false)>();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        {
+          constexpr int R = Ord::cum(1 - P, i + 1) - Ord::cum(1 - P, i);
+          constexpr int slot = phase * TM + i;
+          constexpr int q_lo = (phase < kLoadPhases) ? (slot * LPT + NSLOT - 1) / NSLOT : 0;
+          constexpr int q_hi = (phase < kLoadPhases) ? ((slot + 1) * LPT + NSLOT - 1) / NSLOT : 0;   // loads q_lo .. q_hi-1
+          constexpr int X = R + (q_hi - q_lo);
+          static_for<NB>([&](auto jcc) {
+            constexpr int jc = decltype(jcc)::value;       // b fragment (j, ch) = (jc / 2, jc % 2)
+            mfma16_slice<2 * P + (jc & 1)>(af[P][i], bfr[k2 & 1][jc], acc[i][jc >> 1]);
+            static_for<X>([&](auto xc) {
+              constexpr int x = decltype(xc)::value;
+              if constexpr (x * NB / (X > 0 ? X : 1) == jc) {
+                if constexpr (x < R) {
+                  if (issuing) request(src, std::integral_constant<int, Ord::cum(1 - P, i) + x>{}, std::integral_constant<int, kn>{});
+                } else {
+                  if (loads_here) issue_one(tgt, q_lo + (x - R));
+                }
+              }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+          });
+        }
+      });
+    });
+    cur ^= 1;
+  };
+  int kt = 0;
+  for (; kt + 2 < nk_total; ++kt) step(kt, std::true_type{});
+  for (; kt < nk_total; ++kt) step(kt, std::false_type{});
+  wg_barrier();                                       // LDS may be reused by the caller
+}
+
 // MODE 0: the whole contraction.  MODE 2: only issue the loads of K step 0 into buffer 0 and return (the caller
 // does something else, e.g. the epilogue of the previous tile, while they fly); MODE 1: the contraction, given that
 // a MODE 2 call for the same tile has been made since the last MODE 0/1 call returned.  Modes 1 and 2 exist for
@@ -438,10 +588,11 @@ __device__ __forceinline__ void early_barrier_pipeline(int nk_total, char* smem,
 template <class C>
 constexpr bool kSplitPrologue = C::DMA && C::NSTAGE == 2 && (C::BK / 16) % 2 == 0;
 
-template <class C, int MODE = 0>
+template <class C, int MODE = 0, bool MI16 = false>
 __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row0, int col0, char* smem,
                                                   f32x16_t (&acc)[C::TM][C::TN]) {
   static_assert(MODE == 0 || kSplitPrologue<C>, "split prologue needs the two-buffer schedule");
+  static_assert(!MI16 || kMi16<C>, "16x16x32 MFMAs: 8-wavefront 256x256x64 two-buffer tile only");
   constexpr int D = C::NSTAGE - 1;              // K steps of loads in flight
   constexpr int LPT = C::PA + C::PB;            // loads per thread per K step
   static_assert(D >= 1 && D <= 4 && LPT * (D - 1) < 64, "pipeline depth");
@@ -547,6 +698,26 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
     if constexpr (MODE == 2) return;
   }
 
+  if constexpr (MI16) {
+    // 16x16x32 fragments: lane l reads row (l % 16) of a 16-row block and the 16-byte chunk 4*k2 + l/16 of its
+    // 64-wide K slice (16 consecutive rows at one chunk index: conflict-free under the same swizzle)
+    const int sw16 = lds_swizzle<C>(lane & 15);
+    const int fa16 = (wm * C::WTM + (lane & 15)) * C::ROWB, fb16 = C::BM * C::ROWB + (wn * C::WTN + (lane & 15)) * C::ROWB;
+    int fc16[2];
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2) fc16[k2] = ((4 * k2 + (lane >> 4)) ^ sw16) * 16;
+    early_barrier_pipeline16<C, LPT, 1, 1>(
+        nk_total, smem, acc, issue_one,
+        [&](const char* st, auto i, auto kk) {
+          constexpr int kkv = decltype(kk)::value;
+          return lds_read_b128_asm<(decltype(i)::value * 32 + 16 * (kkv & 1)) * C::ROWB>(lds_addr(st) + fa16 + fc16[kkv >> 1]);
+        },
+        [&](const char* st, auto jc, auto k2) {
+          constexpr int jcv = decltype(jc)::value;
+          return lds_read_b128_asm<((jcv >> 1) * 32 + 16 * (jcv & 1)) * C::ROWB>(lds_addr(st) + fb16 + fc16[decltype(k2)::value]);
+        });
+    return;
+  }
   if constexpr (C::NSTAGE == 2 && (C::BK / 16) % 2 == 0) {
     early_barrier_pipeline<C, LPT, 1, 1>(
         nk_total, smem, acc, issue_one,
@@ -800,10 +971,19 @@ __device__ __forceinline__ void gemm_mainloop_la(const GemmOperands& g, int row0
 // Either operand may instead be K-contiguous (X[m][k]) and is then handled as in
 // gemm_mainloop_dma.  One segment, BM = BN = 256, BK = 64, two LDS buffers.
 // ---------------------------------------------------------------------------
-template <class C, bool AKM, bool BKM>
+// Chunk-index XOR of k row `kr` of a K-major LDS tile (512-byte rows).  The transposing reads of a 32x32x16 operand
+// take rows k .. k+3 per 16-lane group with the two groups of a pass 32 bytes apart in the row: 4*(k%4) spreads the
+// four rows.  A 16x16x32 operand's groups of a pass read the same columns of rows k and k + 8: bit 3 of k moves
+// them another 32 bytes apart.
+template <bool MI16>
+__device__ __forceinline__ int km_swizzle(int kr) {
+  return MI16 ? (((kr & 3) << 2) | (((kr >> 3) & 1) << 1)) : ((kr & 3) << 2);
+}
+template <class C, bool AKM, bool BKM, bool MI16 = false>
 __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0, int col0, char* smem,
                                                  f32x16_t (&acc)[C::TM][C::TN]) {
   static_assert(C::DMA && C::NSTAGE == 2 && C::BM == 256 && C::BN == 256 && C::BK == 64, "K-major loop: 256x256x64, 2 buffers");
+  static_assert(!MI16 || kMi16<C>, "16x16x32 MFMAs: 8-wavefront tile only");
   constexpr int LPT = C::PA + C::PB;
   constexpr int KK = C::BK / 16;
   constexpr int KROWB = 512;                    // bytes of one k row of a K-major tile (256 columns)
@@ -823,7 +1003,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
     for (int i = 0; i < C::PA; ++i) {
       if constexpr (AKM) {
         const int kr = (i * C::NW + wave) * 2 + (lane >> 5);
-        aoff[i] = (uint32_t)((long long)kr * g.lda * 2) + (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
+        aoff[i] = (uint32_t)((long long)kr * g.lda * 2) + (uint32_t)((((lane & 31) ^ km_swizzle<MI16>(kr))) * 16);
       } else {
         const int rt = (i * C::NW + wave) * C::RPI + lrow;
         const int r = rt < amax ? rt : amax;
@@ -834,7 +1014,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
     for (int i = 0; i < C::PB; ++i) {
       if constexpr (BKM) {
         const int kr = (i * C::NW + wave) * 2 + (lane >> 5);
-        boff[i] = (uint32_t)((long long)kr * g.ldb * 2) + (uint32_t)((((lane & 31) ^ ((kr & 3) << 2))) * 16);
+        boff[i] = (uint32_t)((long long)kr * g.ldb * 2) + (uint32_t)((((lane & 31) ^ km_swizzle<MI16>(kr))) * 16);
       } else {
         const int rt = (i * C::NW + wave) * C::RPI + lrow;
         const int r = rt < bmax ? rt : bmax;
@@ -978,6 +1158,45 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
   if (nk_total > 0) {
 #pragma unroll
     for (int idx = 0; idx < LPT; ++idx) issue_one(0, idx);
+  }
+  if constexpr (MI16) {
+    // 16x16x32 fragments.  K-contiguous operand: row l % 16 of a 16-row block, chunk 4*k2 + l/16.  K-major operand:
+    // lane l = 16*g + j supplies row k = 32*k2 + 8*g + 4*r + j/4 (r = 0, 1: the two transposing reads) and the 8 bytes
+    // at column 4*(j%4) of the 16-column block; every 16-lane group gets its own eight k values of the slice.
+    const int sw16 = lds_swizzle<C>(lane & 15);
+    const int fa16 = (wm * C::WTM + (lane & 15)) * C::ROWB, fb16 = REG + (wn * C::WTN + (lane & 15)) * C::ROWB;
+    int fc16[2];
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2) fc16[k2] = ((4 * k2 + (lane >> 4)) ^ sw16) * 16;
+    const int g16 = lane >> 4;
+    const int k16_row = (8 * g16 + j4) * KROWB;                      // + (32*k2 + 4*r) * KROWB
+    const int k16_sw = (j4 << 2) | ((g16 & 1) << 1);                 // km_swizzle of the lane's rows
+    const int k16_cl = (lane & 3) >> 1;                              // chunk of the lane's column inside a 16-column block
+    auto km16_off = [&](int block_col0) { return ((((block_col0 >> 3) + k16_cl) ^ k16_sw) << 4) + frk_half; };
+    int fka16[C::TM][2], fkb16[2 * C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int rh = 0; rh < 2; ++rh) fka16[i][rh] = k16_row + km16_off(wm * C::WTM + i * 32 + 16 * rh);
+#pragma unroll
+    for (int jc = 0; jc < 2 * C::TN; ++jc) fkb16[jc] = REG + k16_row + km16_off(wn * C::WTN + (jc >> 1) * 32 + 16 * (jc & 1));
+    early_barrier_pipeline16<C, LPT, AKM ? 2 : 1, BKM ? 2 : 1>(
+        nk_total, smem, acc, issue_one,
+        [&](const char* st, auto ic, auto kc) -> bf16x8_t {
+          constexpr int i = decltype(ic)::value, kk = decltype(kc)::value, k2 = kk >> 1, rh = kk & 1;
+          if constexpr (AKM)
+            return lds_read_tr_pair<(32 * k2) * KROWB, (32 * k2 + 4) * KROWB>(lds_addr(st) + fka16[i][rh]);
+          else
+            return lds_read_b128_asm<(i * 32 + 16 * rh) * C::ROWB>(lds_addr(st) + fa16 + fc16[k2]);
+        },
+        [&](const char* st, auto jcc, auto k2c) -> bf16x8_t {
+          constexpr int jc = decltype(jcc)::value, k2 = decltype(k2c)::value;
+          if constexpr (BKM)
+            return lds_read_tr_pair<(32 * k2) * KROWB, (32 * k2 + 4) * KROWB>(lds_addr(st) + fkb16[jc]);
+          else
+            return lds_read_b128_asm<((jc >> 1) * 32 + 16 * (jc & 1)) * C::ROWB>(lds_addr(st) + fb16 + fc16[k2]);
+        });
+    return;
   }
   early_barrier_pipeline<C, LPT, AKM ? 2 : 1, BKM ? 2 : 1>(nk_total, smem, acc, issue_one, load_a, load_b);
 }

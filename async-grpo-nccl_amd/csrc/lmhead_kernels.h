@@ -530,9 +530,30 @@ struct StoreParams {
 };
 
 // Output is either fp32 or bf16 (never both); rows/cols past M/N are skipped.
-template <class C, bool HAS_IN, bool OUT_BF16>
+template <class C, bool HAS_IN, bool OUT_BF16, bool MI16 = false>
 __device__ __forceinline__ void store_tile(const StoreParams& p, f32x16_t (&acc)[C::TM][C::TN], float alpha, int row0,
                                            int col0, int wm, int wn, int lane) {
+  if constexpr (MI16) {           // 16x16 blocks: element e of block (i, j) at (acc16_row, acc16_col)
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = row0 + acc16_row<C>(wm, i, e, lane), n = col0 + acc16_col<C>(wn, j, e, lane);
+          if (m < p.g.M && n < p.g.N) {
+            const long long o = (long long)m * p.ldc + n;
+            float v = acc[i][j][e] * alpha;
+            if (p.row_scale) v *= p.row_scale[m];
+            if (HAS_IN) v += p.c_in[o];
+            if (OUT_BF16)
+              p.c_out_bf16[o] = f32_to_bf16_rn(v);
+            else
+              p.c_out_f32[o] = v;
+          }
+        }
+    return;
+  }
   const int mrem = p.g.M - (row0 + wm * C::WTM + 4 * (lane >> 5));  // rr < mrem <=> row valid
 #pragma unroll
   for (int j = 0; j < C::TN; ++j) {
@@ -572,7 +593,7 @@ template <class C>
 constexpr bool kStoreViaLds = C::NW * 32 * C::WTN * 4 <= C::LDS_BYTES && C::WTN % 8 == 0 && 64 % (C::WTN / 8) == 0 &&
                               C::TM * C::TN <= 8;
 
-template <class C, bool HAS_IN, bool OUT_BF16>
+template <class C, bool HAS_IN, bool OUT_BF16, bool MI16 = false>
 __device__ __forceinline__ void store_tile_lds(const StoreParams& p, f32x16_t (&acc)[C::TM][C::TN], float alpha, int row0,
                                                int col0, int wm, int wn, int lane, int wave, char* smem) {
   constexpr int WTN = C::WTN;
@@ -589,8 +610,12 @@ __device__ __forceinline__ void store_tile_lds(const StoreParams& p, f32x16_t (&
 #pragma unroll
     for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * WTN + j * 32 + (lane & 31)] = acc[i][j][r] * alpha;
+      for (int r = 0; r < 16; ++r) {
+        if constexpr (MI16)
+          patch[(16 * (r >> 3) + 4 * (lane >> 4) + (r & 3)) * WTN + j * 32 + 16 * ((r >> 2) & 1) + (lane & 15)] = acc[i][j][r] * alpha;
+        else
+          patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * WTN + j * 32 + (lane & 31)] = acc[i][j][r] * alpha;
+      }
 #pragma unroll
     for (int q = 0; q < 32 / RPP; ++q) {
       const int rr = q * RPP + prow;
@@ -675,12 +700,15 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
   }
   const int row0 = tm * C::BM, col0 = tn * C::BN;
 
+  constexpr bool MI16 = kMi16<C>;             // 16x16x32 MFMAs (and their accumulator layout) on the 8-wavefront tile
   f32x16_t acc[C::TM][C::TN];
   zero_acc<C>(acc);
   const bool dead = p.m_tile_live != nullptr && p.m_tile_live[tm] == 0;     // work-group uniform
   if (!dead) {
     if constexpr (AKM || BKM)
-      gemm_mainloop_km<C, AKM, BKM>(p.g, row0, col0, smem, acc);
+      gemm_mainloop_km<C, AKM, BKM, MI16>(p.g, row0, col0, smem, acc);
+    else if constexpr (MI16)
+      gemm_mainloop_dma<C, 0, true>(p.g, row0, col0, smem, acc);
     else
       run_mainloop<C>(p.g, row0, col0, smem, acc);
   }
@@ -690,19 +718,19 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
   if constexpr (kStoreViaLds<C>) {
     if (p.wide_stores) {
       switch (mode) {
-        case 0: store_tile_lds<C, false, false>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
-        case 1: store_tile_lds<C, true, false>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
-        case 2: store_tile_lds<C, false, true>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
-        default: store_tile_lds<C, true, true>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+        case 0: store_tile_lds<C, false, false, MI16>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+        case 1: store_tile_lds<C, true, false, MI16>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+        case 2: store_tile_lds<C, false, true, MI16>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
+        default: store_tile_lds<C, true, true, MI16>(p, acc, alpha, row0, col0, wm, wn, lane, wave, smem); break;
       }
       return;
     }
   }
   switch (mode) {
-    case 0: store_tile<C, false, false>(p, acc, alpha, row0, col0, wm, wn, lane); break;
-    case 1: store_tile<C, true, false>(p, acc, alpha, row0, col0, wm, wn, lane); break;
-    case 2: store_tile<C, false, true>(p, acc, alpha, row0, col0, wm, wn, lane); break;
-    default: store_tile<C, true, true>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+    case 0: store_tile<C, false, false, MI16>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+    case 1: store_tile<C, true, false, MI16>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+    case 2: store_tile<C, false, true, MI16>(p, acc, alpha, row0, col0, wm, wn, lane); break;
+    default: store_tile<C, true, true, MI16>(p, acc, alpha, row0, col0, wm, wn, lane); break;
   }
 }
 
