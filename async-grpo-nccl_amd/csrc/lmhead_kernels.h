@@ -81,6 +81,16 @@ __device__ __forceinline__ void patch_write_quad(char* patch, int lane_v, int i,
   const int slot = ((i * 32 + 8 * q) >> 2) + (lane_v >> 5);
   lds_write_b64_asm(lds_addr(patch) + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3), v.x, v.y);
 }
+// the same for the 16x16x32 accumulator layout: the lane's token is row 16*ch + lane%16 of the slab and the quad holds
+// its entries i*32 + 16*rh + 4*(lane/16) + 0..3
+template <class C>
+__device__ __forceinline__ void patch_write_quad16(char* patch, int lane_v, int ch, int i, int rh, uint2 v) {
+  constexpr int ROWP = C::WTM * 2;
+  constexpr int NSLOT = ROWP / 8;
+  const int tok = 16 * ch + (lane_v & 15);
+  const int slot = ((i * 32 + 16 * rh) >> 2) + (lane_v >> 4);
+  lds_write_b64_asm(lds_addr(patch) + tok * ROWP + ((slot ^ (tok & (NSLOT - 1) & 31)) << 3), v.x, v.y);
+}
 template <class C>
 __device__ __forceinline__ void patch_flush(char* patch, bf16_t* out, int lane_v) {
   constexpr int ROWP = C::WTM * 2;
@@ -128,18 +138,25 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
   const int vt_end = (int)((long long)(split + 1) * p.tiles_v / p.nsplit);
   const int col0 = tt * C::BN;
 
-  float m_run[C::TN], s_run[C::TN], sx_run[C::TN];
-  float ref2[C::TN];         // KEEP only
-  int y[C::TN];
+  // 16x16x32 MFMAs (kMi16): a lane holds two token columns (ch = 0, 1) of every 32-column block j, 32 vocabulary
+  // values of each per tile; otherwise one column and 64 values.  Slot jc = j * NCL + ch.
+  constexpr bool MI16 = kMi16<C>;
+  constexpr int NCL = MI16 ? 2 : 1, NS = C::TN * NCL;
+  auto slot_col = [&](int jc) {      // column of slot jc inside the tile
+    return MI16 ? wn * C::WTN + (jc >> 1) * 32 + 16 * (jc & 1) + (lane & 15) : acc_col<C>(wn, jc, lane);
+  };
+  float m_run[NS], s_run[NS], sx_run[NS];
+  float ref2[NS];            // KEEP only
+  int y[NS];
 #pragma unroll
-  for (int j = 0; j < C::TN; ++j) {
-    m_run[j] = kNegBig;
-    s_run[j] = 0.f;
-    sx_run[j] = 0.f;
-    const int n = col0 + acc_col<C>(wn, j, lane);
+  for (int jc = 0; jc < NS; ++jc) {
+    m_run[jc] = kNegBig;
+    s_run[jc] = 0.f;
+    sx_run[jc] = 0.f;
+    const int n = col0 + slot_col(jc);
     long long lab = (n < T) ? p.labels[n] : -1;
-    y[j] = (lab >= 0 && lab < V) ? (int)lab : -1;
-    if constexpr (KEEP) ref2[j] = (n < T) ? p.keep_ref2[n] : -kNegBig;
+    y[jc] = (lab >= 0 && lab < V) ? (int)lab : -1;
+    if constexpr (KEEP) ref2[jc] = (n < T) ? p.keep_ref2[n] : -kNegBig;
   }
 
   // KEEP: the wavefront's patch lives behind LDS buffer 0, which the prefetch of the next tile may already be filling
@@ -153,7 +170,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
   if constexpr (kSplitPrologue<C>) {
     if (vt_begin < vt_end) {
       f32x16_t none[C::TM][C::TN];
-      gemm_mainloop_dma<C, 2>(p.g, vt_begin * C::BM, col0, smem, none);
+      gemm_mainloop_dma<C, 2, MI16>(p.g, vt_begin * C::BM, col0, smem, none);
     }
   }
   for (int vt = vt_begin; vt < vt_end; ++vt) {
@@ -161,8 +178,8 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
     f32x16_t acc[C::TM][C::TN];
     zero_acc<C>(acc);
     if constexpr (kSplitPrologue<C>) {
-      gemm_mainloop_dma<C, 1>(p.g, row0, col0, smem, acc);
-      if (vt + 1 < vt_end) gemm_mainloop_dma<C, 2>(p.g, row0 + C::BM, col0, smem, acc);
+      gemm_mainloop_dma<C, 1, MI16>(p.g, row0, col0, smem, acc);
+      if (vt + 1 < vt_end) gemm_mainloop_dma<C, 2, MI16>(p.g, row0 + C::BM, col0, smem, acc);
     } else {
       run_mainloop<C>(p.g, row0, col0, smem, acc);
     }
@@ -175,107 +192,132 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
       for (int i = 0; i < C::TM; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int v = row0 + acc_row<C>(wm, i, r, lane);
-          const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
+          if constexpr (MI16) {
+            if ((r & 4) != 0) continue;                 // the row of element r does not depend on its column half
+            const int v = row0 + acc16_row<C>(wm, i, r, lane);
+            const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
 #pragma unroll
-          for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
+            for (int j = 0; j < C::TN; ++j) {
+              acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
+              acc[i][j][r + 4] = (v < V) ? acc[i][j][r + 4] + b : kNegBig;
+            }
+          } else {
+            const int v = row0 + acc_row<C>(wm, i, r, lane);
+            const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
+          }
         }
     }
 
     const float xs = p.inv_temp * kLog2e;
+    // Elements of slot jc: NQ quads of four consecutive vocabulary rows each.  Quad qq of slot jc is the registers
+    // qreg(jc, qq) .. + 3 of block (qq / QPB, jc / NCL); its first row, relative to the lane's first row, is qrow(qq).
+    constexpr int QPB = MI16 ? 2 : 4, NQ = C::TM * QPB;
+    auto qreg = [&](int jc, int qq) { return MI16 ? 4 * (2 * (qq % QPB) + (jc & 1)) : 4 * (qq % QPB); };
+    auto qrow = [&](int qq) { return MI16 ? (qq / QPB) * 32 + 16 * (qq % QPB) : (qq / QPB) * 32 + 8 * (qq % QPB); };
+    const int lane_row0 = wm * C::WTM + 4 * (MI16 ? (lane >> 4) : (lane >> 5));
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
+    for (int jc = 0; jc < NS; ++jc) {
+      const int j = jc / NCL;
       float mt = kNegBig;
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i)
+      for (int qq = 0; qq < NQ; ++qq)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mt = fmaxf(mt, acc[i][j][r]);
-      const float mn = fmaxf(m_run[j], mt);
-      const float alpha = fast_exp2((m_run[j] - mn) * xs);
+        for (int c = 0; c < 4; ++c) mt = fmaxf(mt, acc[qq / QPB][j][qreg(jc, qq) + c]);
+      const float mn = fmaxf(m_run[jc], mt);
+      const float alpha = fast_exp2((m_run[jc] - mn) * xs);
       // a slot that has seen only masked rows keeps (m, s, sx) = (kNegBig, 0, 0):
       // x*xs - mb would otherwise be the rounding residue of two huge terms
       const float mb = (mn > 0.5f * kNegBig) ? mn * xs : 0.f;
-      // target logit: rows of this lane are lane_row0 + i*32 + 8*(r/4) + (r%4)
-      const int yrel = y[j] - row0 - wm * C::WTM - 4 * (lane >> 5);
-      if (y[j] >= 0 && yrel >= 0 && yrel < C::WTM) {
+      // target logit, if one of this lane's rows holds it
+      const int yrel = y[jc] - row0 - lane_row0;
+      if (y[jc] >= 0 && yrel >= 0 && yrel < C::WTM) {
         float xv = 0.f;
         bool hit = false;
 #pragma unroll
-        for (int i = 0; i < C::TM; ++i)
+        for (int qq = 0; qq < NQ; ++qq)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const bool h = (yrel == i * 32 + 8 * (r >> 2) + (r & 3));
-            xv = h ? acc[i][j][r] : xv;
+          for (int c = 0; c < 4; ++c) {
+            const bool h = (yrel == qrow(qq) + c);
+            xv = h ? acc[qq / QPB][j][qreg(jc, qq) + c] : xv;
             hit = hit || h;
           }
-        if (hit) p.xt[col0 + acc_col<C>(wn, j, lane)] = xv * p.inv_temp;
+        if (hit) p.xt[col0 + slot_col(jc)] = xv * p.inv_temp;
       }
       // KEEP: the exponential computed for the statistics (relative to the running maximum) times one factor per
       // token and tile re-bases it on the token's fixed reference; it replaces the accumulator it came from
       float kf = 0.f;
       if constexpr (KEEP) {
-        const float d2 = mb - ref2[j];
+        const float d2 = mb - ref2[jc];
         kf = fast_exp2(d2);
-        if (d2 > kKeepHeadroom2 && ref2[j] < 0.5f * -kNegBig) *p.keep_flag = 1;
+        if (d2 > kKeepHeadroom2 && ref2[jc] < 0.5f * -kNegBig) *p.keep_flag = 1;
       }
-      float s = s_run[j] * alpha, sx = sx_run[j] * alpha;
+      float s = s_run[jc] * alpha, sx = sx_run[jc] * alpha;
       // KEEP: the patch addresses are recomputed per tile on purpose (hoisted they would sit in registers across the
       // main loop); every quad goes to the patch as soon as its statistics are folded in
       int lane_v = lane;
       if constexpr (KEEP) asm volatile("" : "+v"(lane_v));
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i)
+      for (int qq = 0; qq < NQ; ++qq) {
+        float ek[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float ek[4];
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const float x = acc[i][j][q * 4 + c];
-            const float e = fast_exp2(__builtin_fmaf(x, xs, -mb));
-            s += e;
-            sx = __builtin_fmaf(e, x, sx);
-            ek[c] = e * kf;
-          }
-          if constexpr (KEEP) {
-            uint2 pk;
-            pk.x = pack_bf16x2(ek[0], ek[1]);
-            pk.y = pack_bf16x2(ek[2], ek[3]);
-            patch_write_quad<C>(patch, lane_v, i, q, pk);
-            // pin the running sums here: left alone the compiler first computes all 64 exponentials of the column
-            // (to feed the patch writes) and folds them into the sums afterwards, which keeps all of them in registers
-            asm volatile("" : "+v"(s), "+v"(sx));
-          }
+        for (int c = 0; c < 4; ++c) {
+          const float x = acc[qq / QPB][j][qreg(jc, qq) + c];
+          const float e = fast_exp2(__builtin_fmaf(x, xs, -mb));
+          s += e;
+          sx = __builtin_fmaf(e, x, sx);
+          ek[c] = e * kf;
         }
-      m_run[j] = mn;
-      s_run[j] = s;
-      sx_run[j] = sx;
-      if constexpr (KEEP)
-        patch_flush<C>(patch, p.keep + (long long)vt * p.keep_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM,
-                       lane_v);
+        if constexpr (KEEP) {
+          uint2 pk;
+          pk.x = pack_bf16x2(ek[0], ek[1]);
+          pk.y = pack_bf16x2(ek[2], ek[3]);
+          if constexpr (MI16)
+            patch_write_quad16<C>(patch, lane_v, jc & 1, qq / QPB, qq % QPB, pk);
+          else
+            patch_write_quad<C>(patch, lane_v, qq / QPB, qq % QPB, pk);
+          // pin the running sums here: left alone the compiler first computes all the exponentials of the column
+          // (to feed the patch writes) and folds them into the sums afterwards, which keeps all of them in registers
+          asm volatile("" : "+v"(s), "+v"(sx));
+        }
+      }
+      m_run[jc] = mn;
+      s_run[jc] = s;
+      sx_run[jc] = sx;
+      if constexpr (KEEP) {
+        if (jc % NCL == NCL - 1)          // the 32-token slab of block column j is complete
+          patch_flush<C>(patch, p.keep + (long long)vt * p.keep_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM,
+                         lane_v);
+      }
     }
   }
 
   // back to logit units (a masked-only slot keeps a huge negative maximum and zero sums)
 #pragma unroll
-  for (int j = 0; j < C::TN; ++j) {
-    m_run[j] *= p.inv_temp;
-    sx_run[j] *= p.inv_temp;
+  for (int jc = 0; jc < NS; ++jc) {
+    m_run[jc] *= p.inv_temp;
+    sx_run[jc] *= p.inv_temp;
   }
-  // lanes l and l^32 hold the same tokens (different vocabulary rows)
+  // lanes that hold the same tokens (different vocabulary rows): l ^ 32, and with 16x16 blocks also l ^ 16
 #pragma unroll
-  for (int j = 0; j < C::TN; ++j) {
-    const float m2 = __shfl_xor(m_run[j], 32), s2 = __shfl_xor(s_run[j], 32), x2 = __shfl_xor(sx_run[j], 32);
-    lse_merge(m_run[j], s_run[j], sx_run[j], m2, s2, x2);
+  for (int jc = 0; jc < NS; ++jc) {
+    if constexpr (MI16) {
+      const float m1 = __shfl_xor(m_run[jc], 16), s1 = __shfl_xor(s_run[jc], 16), x1 = __shfl_xor(sx_run[jc], 16);
+      lse_merge(m_run[jc], s_run[jc], sx_run[jc], m1, s1, x1);
+    }
+    const float m2 = __shfl_xor(m_run[jc], 32), s2 = __shfl_xor(s_run[jc], 32), x2 = __shfl_xor(sx_run[jc], 32);
+    lse_merge(m_run[jc], s_run[jc], sx_run[jc], m2, s2, x2);
   }
   // wavefronts stacked along the vocabulary (same wn, different wm) meet in LDS
   float* red = (float*)smem;  // [WM][BN][3]
-  if (lane < 32) {
+  if (lane < (MI16 ? 16 : 32)) {
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      float* d = red + ((wm * C::BN) + wn * C::WTN + j * 32 + lane) * 3;
-      d[0] = m_run[j];
-      d[1] = s_run[j];
-      d[2] = sx_run[j];
+    for (int jc = 0; jc < NS; ++jc) {
+      float* d = red + ((wm * C::BN) + slot_col(jc)) * 3;
+      d[0] = m_run[jc];
+      d[1] = s_run[jc];
+      d[2] = sx_run[jc];
     }
   }
   __syncthreads();
