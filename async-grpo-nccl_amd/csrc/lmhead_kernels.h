@@ -385,17 +385,26 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
 
   const float go = (p.gout ? *p.gout : 1.f) * p.inv_temp;
   const float xs = p.inv_temp * kLog2e;
-  const int lane_row0 = wm * C::WTM + 4 * (lane >> 5);   // first row of this lane inside the tile
-  float lse2[C::TN], cj[C::TN];
-  int ylab[C::TN];
+  // 16x16x32 MFMAs (kMi16, not with SPLIT): two token columns per lane and 32-column block, see lmhead_fwd_kernel
+  constexpr bool MI16 = kMi16<C> && !SPLIT;
+  constexpr int NCL = MI16 ? 2 : 1, NS = C::TN * NCL;
+  constexpr int QPB = MI16 ? 2 : 4, NQ = C::TM * QPB;
+  auto slot_col = [&](int jc) {
+    return MI16 ? wn * C::WTN + (jc >> 1) * 32 + 16 * (jc & 1) + (lane & 15) : acc_col<C>(wn, jc, lane);
+  };
+  auto qreg = [&](int jc, int qq) { return MI16 ? 4 * (2 * (qq % QPB) + (jc & 1)) : 4 * (qq % QPB); };
+  auto qrow = [&](int qq) { return MI16 ? (qq / QPB) * 32 + 16 * (qq % QPB) : (qq / QPB) * 32 + 8 * (qq % QPB); };
+  const int lane_row0 = wm * C::WTM + 4 * (MI16 ? (lane >> 4) : (lane >> 5));   // first row of this lane inside the tile
+  float lse2[NS], cj[NS];
+  int ylab[NS];
 #pragma unroll
-  for (int j = 0; j < C::TN; ++j) {
-    const int n = col0 + acc_col<C>(wn, j, lane);
+  for (int jc = 0; jc < NS; ++jc) {
+    const int n = col0 + slot_col(jc);
     const bool tok_ok = n < T;
-    lse2[j] = tok_ok ? p.lse[n] * kLog2e : -kNegBig;          // padding columns: probability exactly 0
+    lse2[jc] = tok_ok ? p.lse[n] * kLog2e : -kNegBig;         // padding columns: probability exactly 0
     const long long lab = tok_ok ? p.labels[n] : -100;
-    cj[j] = (lab != -100) ? p.gtok[n] * go : 0.f;             // ignored tokens carry no gradient
-    ylab[j] = (lab >= 0 && lab < V) ? (int)lab : (int)0xC0000000;   // far below any row: never matches
+    cj[jc] = (lab != -100) ? p.gtok[n] * go : 0.f;            // ignored tokens carry no gradient
+    ylab[jc] = (lab >= 0 && lab < V) ? (int)lab : (int)0xC0000000;  // far below any row: never matches
   }
 
   // Column-blocked panel: a lane's 8 bytes (4 vocabulary entries of one token) would be a 64-line scatter per
@@ -417,7 +426,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
   if constexpr (kPrefetch) {
     if (vt_begin < vt_end) {
       f32x16_t none[C::TM][C::TN];
-      gemm_mainloop_dma<C, 2>(p.g, p.v0 + vt_begin * C::BM, col0, smem, none);
+      gemm_mainloop_dma<C, 2, MI16>(p.g, p.v0 + vt_begin * C::BM, col0, smem, none);
     }
   }
   for (int vt = vt_begin; vt < vt_end; ++vt) {
@@ -426,8 +435,8 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
     f32x16_t acc[C::TM][C::TN];
     zero_acc<C>(acc);
     if constexpr (kPrefetch) {
-      gemm_mainloop_dma<C, 1>(p.g, row0, col0, smem, acc);
-      if (vt + 1 < vt_end) gemm_mainloop_dma<C, 2>(p.g, row0 + C::BM, col0, smem, acc);
+      gemm_mainloop_dma<C, 1, MI16>(p.g, row0, col0, smem, acc);
+      if (vt + 1 < vt_end) gemm_mainloop_dma<C, 2, MI16>(p.g, row0 + C::BM, col0, smem, acc);
     } else {
       run_mainloop<C>(p.g, row0, col0, smem, acc);
     }
@@ -438,26 +447,38 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
       for (int i = 0; i < C::TM; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int v = row0 + acc_row<C>(wm, i, r, lane);
-          const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
+          if constexpr (MI16) {
+            if ((r & 4) != 0) continue;                 // the row of element r does not depend on its column half
+            const int v = row0 + acc16_row<C>(wm, i, r, lane);
+            const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
 #pragma unroll
-          for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
+            for (int j = 0; j < C::TN; ++j) {
+              acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
+              acc[i][j][r + 4] = (v < V) ? acc[i][j][r + 4] + b : kNegBig;
+            }
+          } else {
+            const int v = row0 + acc_row<C>(wm, i, r, lane);
+            const float b = (p.bias != nullptr && v < V) ? p.bias[v] : 0.f;
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j) acc[i][j][r] = (v < V) ? acc[i][j][r] + b : kNegBig;
+          }
         }
     }
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const int n = col0 + acc_col<C>(wn, j, lane);
-      const float c = cj[j], nc = -c, l2 = lse2[j];
+    for (int jc = 0; jc < NS; ++jc) {
+      const int j = jc / NCL;
+      const int n = col0 + slot_col(jc);
+      const float c = cj[jc], nc = -c, l2 = lse2[jc];
       // target row relative to this lane's first row; out of range when not in this sub-tile
-      const int yrel = ylab[j] - row0 - lane_row0;
+      const int yrel = ylab[jc] - row0 - lane_row0;
       // Few wavefronts hold a target row at all (64 tokens x WTM of V rows): the common case runs without
       // the per-element comparison.
       const bool any_y = __builtin_amdgcn_ballot_w64(yrel >= 0 && yrel < C::WTM) != 0;
+      // The swizzled patch addresses are recomputed per tile on purpose: hoisted out of the vocabulary loop they
+      // would occupy two dozen registers across the main loop.  The empty asm makes them loop-variant.
+      int lane_v = lane;
+      asm volatile("" : "+v"(lane_v));
       auto emit = [&](auto with_y, auto via_lds) {
-        // The swizzled patch addresses are recomputed per tile on purpose: hoisted out of the vocabulary loop they
-        // would occupy two dozen registers across the main loop.  The empty asm makes them loop-variant.
-        int lane_v = lane;
-        asm volatile("" : "+v"(lane_v));
         bf16_t *tv_hi = nullptr, *tv_lo = nullptr, *vt_hi = nullptr, *vt_lo = nullptr;
         if constexpr (!decltype(via_lds)::value) {      // direct stores: plain or blocked rows, optional [vocab][token] copy
           const long long tv_off = p.tv_blk ? (long long)vt * p.tv_blk + (long long)n * 256 + lane_row0
@@ -468,14 +489,13 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
           vt_lo = (SPLIT && p.vt_lo) ? p.vt_lo + (long long)(prow0 + lane_row0) * p.ld_vt + n : nullptr;
         }
 #pragma unroll
-        for (int i = 0; i < C::TM; ++i) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int rr0 = i * 32 + 8 * q;  // row relative to the lane's first row
+        for (int qq = 0; qq < NQ; ++qq) {
+          {
+            const int rr0 = qrow(qq);        // row relative to the lane's first row
             float ds[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              const float pr = fast_exp2(__builtin_fmaf(acc[i][j][q * 4 + e], xs, -l2));
+              const float pr = fast_exp2(__builtin_fmaf(acc[qq / QPB][j][qreg(jc, qq) + e], xs, -l2));
               if constexpr (decltype(with_y)::value)
                 ds[e] = __builtin_fmaf(nc, pr, (rr0 + e == yrel) ? c : 0.f);
               else
@@ -486,8 +506,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
             pk.x = pack_bf16x2(ds[0], ds[1]);
             pk.y = pack_bf16x2(ds[2], ds[3]);
             if constexpr (decltype(via_lds)::value) {
-              const int slot = (rr0 >> 2) + (lane_v >> 5);             // 8-byte slot of (rr0 + 4*(lane/32)) in the row
-              lds_write_b64_asm(lds_addr(patch) + (lane_v & 31) * ROWP + ((slot ^ (lane_v & (NSLOT - 1) & 31)) << 3), pk.x, pk.y);
+              // 8-byte slot of the quad's first row in the token's patch row
+              const int tok = MI16 ? 16 * (jc & 1) + (lane_v & 15) : (lane_v & 31);
+              const int slot = (rr0 >> 2) + (MI16 ? (lane_v >> 4) : (lane_v >> 5));
+              lds_write_b64_asm(lds_addr(patch) + tok * ROWP + ((slot ^ (tok & (NSLOT - 1) & 31)) << 3), pk.x, pk.y);
               continue;
             }
             *(uint2*)(tv_hi + rr0) = pk;
@@ -512,28 +534,6 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
             }
           }
         }
-        if constexpr (decltype(via_lds)::value) {
-          bf16_t* out = p.tv_hi + (long long)vt * p.tv_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
-          // inline-assembly LDS traffic (see lds_write_b64_asm): one wait for all reads, LDS operations of a
-          // wavefront complete in order, so the reads see this wavefront's writes
-          u32x4_t pv[32 / TPP];
-#pragma unroll
-          for (int r = 0; r < 32 / TPP; ++r) {
-            const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
-            const int m = tok & (NSLOT - 1);
-            pv[r] = __builtin_bit_cast(u32x4_t, lds_read_b128_asm<0>(lds_addr(patch) + tok * ROWP + ((piece ^ (m >> 1)) << 4)));
-          }
-          wait_lgkm<0>();
-          __builtin_amdgcn_sched_barrier(0);     // nothing that consumes pv may move above the wait
-#pragma unroll
-          for (int r = 0; r < 32 / TPP; ++r) {
-            const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
-            const int m = tok & (NSLOT - 1);
-            u32x4_t v = pv[r];
-            if (m & 1) v = u32x4_t{v[2], v[3], v[0], v[1]};       // odd rows hold the two slots of a piece swapped
-            __builtin_nontemporal_store(v, (u32x4_t*)(out + (long long)tok * 256 + piece * 8));   // see patch_flush
-          }
-        }
       };
       if (through_lds) {
         if (any_y)
@@ -545,6 +545,28 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
           emit(std::true_type{}, std::false_type{});
         else
           emit(std::false_type{}, std::false_type{});
+      }
+      if (through_lds && jc % NCL == NCL - 1) {      // the 32-token slab of block column j is complete
+        bf16_t* out = p.tv_hi + (long long)vt * p.tv_blk + (long long)(col0 + wn * C::WTN + j * 32) * 256 + wm * C::WTM;
+        // inline-assembly LDS traffic (see lds_write_b64_asm): one wait for all reads, LDS operations of a
+        // wavefront complete in order, so the reads see this wavefront's writes
+        u32x4_t pv[32 / TPP];
+#pragma unroll
+        for (int r = 0; r < 32 / TPP; ++r) {
+          const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
+          const int m = tok & (NSLOT - 1);
+          pv[r] = __builtin_bit_cast(u32x4_t, lds_read_b128_asm<0>(lds_addr(patch) + tok * ROWP + ((piece ^ (m >> 1)) << 4)));
+        }
+        wait_lgkm<0>();
+        __builtin_amdgcn_sched_barrier(0);     // nothing that consumes pv may move above the wait
+#pragma unroll
+        for (int r = 0; r < 32 / TPP; ++r) {
+          const int tok = r * TPP + lane_v / PPT, piece = lane_v % PPT;
+          const int m = tok & (NSLOT - 1);
+          u32x4_t v = pv[r];
+          if (m & 1) v = u32x4_t{v[2], v[3], v[0], v[1]};       // odd rows hold the two slots of a piece swapped
+          __builtin_nontemporal_store(v, (u32x4_t*)(out + (long long)tok * 256 + piece * 8));   // see patch_flush
+        }
       }
     }
     if constexpr (!kPrefetch) __syncthreads();   // the patch (or the direct stores) are done before the buffers refill
