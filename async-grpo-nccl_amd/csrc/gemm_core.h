@@ -257,14 +257,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 // same, and also wait for every outstanding LDS read (lgkmcnt = 0)
 #define FGRPO_WAIT_VMCNT_LGKM0(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (0 << 8) | (((n) >> 4) << 14))
 
-template <class C>
+template <class C, bool MI16 = false>
 __device__ __forceinline__ int lds_swizzle(int row) {
-  // Chosen with SQ_LDS_BANK_CONFLICT on the real kernels (fragment read: lane l -> row l%32,
-  // chunk l/32 + 2*kk; the LDS serves 16 consecutive lanes per pass over 64 banks).
+  // Chosen with SQ_LDS_BANK_CONFLICT on the real kernels and a read-rate microbenchmark.  32x32x16 fragment read:
+  // lane l -> row l%32, chunk l/32 + 2*kk.  16x16x32 fragment read: lane l -> row l%16, chunk l/16 + 4*k2; under the
+  // 32-row swizzle these reads run at half rate (two-way conflicts), under row%8 at the full rate.
   if constexpr (C::CPR == 4)
     return (row >> 2) & 3;                       // 64-byte rows
+  else if constexpr (MI16)
+    return row & 7;                              // 128-byte rows, 16-row fragments
   else
-    return (row + ((row >> 3) & 1)) & 7;                       // 128-byte rows
+    return (row + ((row >> 3) & 1)) & 7;         // 128-byte rows, 32-row fragments
 }
 
 __device__ __forceinline__ void wg_barrier() {
@@ -613,13 +616,13 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   for (int i = 0; i < C::PA; ++i) {
     const int rt = (i * C::NW + wave) * C::RPI + lrow;            // row inside the tile (decides the swizzle)
     const int r = rt < amax ? rt : amax;                          // row actually read
-    aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+    aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C, MI16>(rt)) * 16));
   }
 #pragma unroll
   for (int i = 0; i < C::PB; ++i) {
     const int rt = (i * C::NW + wave) * C::RPI + lrow;
     const int r = rt < bmax ? rt : bmax;
-    boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+    boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C, MI16>(rt)) * 16));
   }
   const int dst_a = wave * C::RPI * C::ROWB;                      // + i * NW*RPI*ROWB, wave-uniform
   const int dst_b = C::BM * C::ROWB + dst_a;
@@ -701,7 +704,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmOperands& g, int row
   if constexpr (MI16) {
     // 16x16x32 fragments: lane l reads row (l % 16) of a 16-row block and the 16-byte chunk 4*k2 + l/16 of its
     // 64-wide K slice (16 consecutive rows at one chunk index: conflict-free under the same swizzle)
-    const int sw16 = lds_swizzle<C>(lane & 15);
+    const int sw16 = lds_swizzle<C, MI16>(lane & 15);
     const int fa16 = (wm * C::WTM + (lane & 15)) * C::ROWB, fb16 = C::BM * C::ROWB + (wn * C::WTN + (lane & 15)) * C::ROWB;
     int fc16[2];
 #pragma unroll
@@ -1007,7 +1010,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
       } else {
         const int rt = (i * C::NW + wave) * C::RPI + lrow;
         const int r = rt < amax ? rt : amax;
-        aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+        aoff[i] = (uint32_t)((long long)r * g.lda * 2 + ((lpc ^ lds_swizzle<C, MI16>(rt)) * 16));
       }
     }
 #pragma unroll
@@ -1018,7 +1021,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
       } else {
         const int rt = (i * C::NW + wave) * C::RPI + lrow;
         const int r = rt < bmax ? rt : bmax;
-        boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C>(rt)) * 16));
+        boff[i] = (uint32_t)((long long)r * g.ldb * 2 + ((lpc ^ lds_swizzle<C, MI16>(rt)) * 16));
       }
     }
   }
@@ -1163,7 +1166,7 @@ __device__ __forceinline__ void gemm_mainloop_km(const GemmOperands& g, int row0
     // 16x16x32 fragments.  K-contiguous operand: row l % 16 of a 16-row block, chunk 4*k2 + l/16.  K-major operand:
     // lane l = 16*g + j supplies row k = 32*k2 + 8*g + 4*r + j/4 (r = 0, 1: the two transposing reads) and the 8 bytes
     // at column 4*(j%4) of the 16-column block; every 16-lane group gets its own eight k values of the slice.
-    const int sw16 = lds_swizzle<C>(lane & 15);
+    const int sw16 = lds_swizzle<C, MI16>(lane & 15);
     const int fa16 = (wm * C::WTM + (lane & 15)) * C::ROWB, fb16 = REG + (wn * C::WTN + (lane & 15)) * C::ROWB;
     int fc16[2];
 #pragma unroll
