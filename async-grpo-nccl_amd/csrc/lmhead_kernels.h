@@ -230,20 +230,17 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
       // a slot that has seen only masked rows keeps (m, s, sx) = (kNegBig, 0, 0):
       // x*xs - mb would otherwise be the rounding residue of two huge terms
       const float mb = (mn > 0.5f * kNegBig) ? mn * xs : 0.f;
-      // target logit, if one of this lane's rows holds it
+      // target logit, if one of this lane's rows holds it: the lane's rows are quads 16 (8 with 32x32 blocks) apart,
+      // so relative to its first row a row of its own has bits 2..3 (bit 2) clear; y = -1 gives a negative yrel
       const int yrel = y[jc] - row0 - lane_row0;
-      if (y[jc] >= 0 && yrel >= 0 && yrel < C::WTM) {
+      constexpr int kRowGap = MI16 ? 12 : 4;
+      if ((unsigned)yrel < (unsigned)C::WTM && (yrel & kRowGap) == 0) {
         float xv = 0.f;
-        bool hit = false;
 #pragma unroll
         for (int qq = 0; qq < NQ; ++qq)
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const bool h = (yrel == qrow(qq) + c);
-            xv = h ? acc[qq / QPB][j][qreg(jc, qq) + c] : xv;
-            hit = hit || h;
-          }
-        if (hit) p.xt[col0 + slot_col(jc)] = xv * p.inv_temp;
+          for (int c = 0; c < 4; ++c) xv = (yrel == qrow(qq) + c) ? acc[qq / QPB][j][qreg(jc, qq) + c] : xv;
+        p.xt[col0 + slot_col(jc)] = xv * p.inv_temp;
       }
       // KEEP: the exponential computed for the statistics (relative to the running maximum) times one factor per
       // token and tile re-bases it on the token's fixed reference; it replaces the accumulator it came from
