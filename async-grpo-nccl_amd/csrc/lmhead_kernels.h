@@ -26,7 +26,11 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rn(float f) { return __builtin_b
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
 
 // (m1,s1,x1) (+) (m2,s2,x2) for sums of exp(v - m) and exp(v - m) * v.
+// No contraction in here: a caller's m is often a product (raw maximum * 1/temperature), and fused into m - mn with
+// mn == m that product's rounding residue would replace the exact zero - for the huge stand-in maximum of a slot
+// that saw only masked rows a residue of ~1e22, whose exponential is 0 or +inf, and 0 * inf = NaN.
 __device__ __forceinline__ void lse_merge(float& m, float& s, float& sx, float m2, float s2, float sx2) {
+#pragma clang fp contract(off)
   const float mn = m > m2 ? m : m2;
   const float a1 = fast_exp2((m - mn) * kLog2e), a2 = fast_exp2((m2 - mn) * kLog2e);
   s = s * a1 + s2 * a2;
@@ -295,6 +299,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_fwd_kernel(const FwdPara
   for (int jc = 0; jc < NS; ++jc) {
     m_run[jc] *= p.inv_temp;
     sx_run[jc] *= p.inv_temp;
+    asm volatile("" : "+v"(m_run[jc]));      // a value from here on, not a product to fuse into the merges below
   }
   // lanes that hold the same tokens (different vocabulary rows): l ^ 32, and with 16x16 blocks also l ^ 16
 #pragma unroll

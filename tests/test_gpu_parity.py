@@ -175,6 +175,30 @@ def test_bias_and_temperature(dev):
         check(want, got, o, g, f32=(dtype == "fp32"))
 
 
+@pytest.mark.parametrize("keep", [False, True])
+def test_masked_only_lanes_of_the_last_vocabulary_tile_over_temperatures(dev, keep):
+    """The vocabulary ends one row into the upper half of its last 256-row tile, on the large tile (19 token tiles x 9
+    vocabulary tiles): most lanes of that half see masked rows only and carry the huge negative stand-in maximum into
+    the merges.  Scaled by 1 / temperature and merged with itself it must still give weight exp(0) = 1 (a fused
+    multiply-subtract there leaves the product's rounding residue, +-1e22, whose exponential is 0 or inf, depending
+    on the temperature).  Checked against the oracle on sampled rows for temperatures of both rounding directions."""
+    from fgrpo import ops
+    T, H, V = 4864, (4096 if keep else 1024), 2048 + 129       # the kernel that keeps the numerators wants V/256 * H/256 >= 128
+    g = torch.Generator().manual_seed(5)
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    weight = (torch.randn(V, H, generator=g) * 0.02).to(torch.bfloat16)
+    y = torch.randint(0, V, (T,), generator=g)
+    assert (not keep) or ops.keep_supported(T, H, V, torch.bfloat16)
+    rows = torch.arange(0, T, 37)
+    for temp in (1.3, 0.57, 1.0, 2.005, 0.745):
+        res = ops.lmhead_logprob_fwd(hidden.to(dev), weight.to(dev), None, y.to(dev), temp, keep=keep)
+        lp, ent, lse = (t.cpu() for t in res[:3])
+        assert torch.isfinite(lp).all() and torch.isfinite(ent).all() and torch.isfinite(lse).all(), temp
+        logits = O.project(weight.float(), None, hidden.float()[rows], temp)
+        assert (lp[rows] - O.logprobs_from_logits(logits, y[rows])).abs().max().item() <= LP_TOL_BF16, temp
+        assert (ent[rows] - O.entropy_from_logits(logits)).abs().max().item() <= 5e-3, temp
+
+
 # ------------------------------------------------------------------ gradient GEMMs on operands read in place
 @pytest.mark.parametrize("layout,M,N,K,k_valid", [
     ("b", 512, 256, 128, 0),
