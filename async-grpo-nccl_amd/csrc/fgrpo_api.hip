@@ -833,12 +833,18 @@ struct KeptBwdPlan {
   float* dh_acc;          // [T x H] fp32, panels > 1 only
   size_t bytes;
 };
+// Row length of the scaled, transposed copy of hidden: the padded token count plus 192 elements.  Rows 2 * Tpad bytes
+// apart (a multiple of 512, at T = 32768 exactly 64 KiB) all start in the same memory channel, and a tile of the dW
+// product reads 256 of them side by side.  Measured on that product at T = 32768, H = 1536: no padding 11.03 ms,
+// 64 bytes 11.86 (rows then straddle 128-byte lines), 128 bytes 10.69, 256 / 384 / 640 / 2176 bytes 10.55-10.59.
+long long kept_hs_ld(int T) { return round_up(T, 256) + 192; }
+
 void plan_kept_bwd(KeptBwdPlan& pl, void* ws, int T, int H) {
   Carver cv(ws);
   pl.row_scale = cv.take<float>((size_t)T);
   pl.k_runs = cv.take<int>((size_t)(2 + 2 * kRunCap));
   pl.m_tile_live = cv.take<int>((size_t)((T + 255) / 256));
-  pl.hidden_scaled = cv.take<bf16_t>((size_t)H * round_up(T, 256));
+  pl.hidden_scaled = cv.take<bf16_t>((size_t)H * kept_hs_ld(T));
   pl.dh_acc = cv.take<float>((size_t)T * H);     // always sized: a concurrent set_tuning must not make it short
   pl.bytes = cv.total();
 }
@@ -896,7 +902,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
     HIP_TRY(hipGetLastError());
     if (dW_out)
       hipLaunchKernelGGL(keep_scaled_transpose_kernel, dim3(Tpad / 64, H / 64), dim3(256), 0, st, (const bf16_t*)hidden,
-                         (const float*)pl.row_scale, T, H, Tpad, pl.hidden_scaled);
+                         (const float*)pl.row_scale, T, H, Tpad, kept_hs_ld(T), pl.hidden_scaled);
     if (skip_dead) {
       KeepLiveParams lv{pl.row_scale, T, (T + 63) / 64, Tpad / 64, pl.k_runs, pl.m_tile_live};
       hipLaunchKernelGGL(keep_live_runs_kernel, dim3(1), dim3(1024), 0, st, lv);
@@ -948,7 +954,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       s.g.N = H;
       s.g.lda = 256;
       s.g.a_blk = blk;
-      s.g.ldb = Tpad;
+      s.g.ldb = kept_hs_ld(T);
       s.g.nseg = 1;
       s.g.seg[0] = GemmSeg{ek_p, pl.hidden_scaled, Tpad};
       s.g.ka_valid = T;

@@ -251,9 +251,10 @@ __global__ __launch_bounds__(256) void keep_backward_prep_kernel(const KeepPrepP
 
 // B operand of the dW product, contraction-contiguous: out[h][t] = a_t * hidden[t][h] for t < T, zero up to Tpad
 // (the contraction runs over whole 64-token steps; the kept buffer's rows past T read as zero, and zero times a
-// stale value must not be a NaN).  64 x 64 tiles through LDS; H % 64 == 0, Tpad % 64 == 0.
+// stale value must not be a NaN); rows of `out` are ld elements apart.  64 x 64 tiles through LDS; H % 64 == 0,
+// Tpad % 64 == 0, ld >= Tpad, ld % 8 == 0.
 __global__ __launch_bounds__(256) void keep_scaled_transpose_kernel(const bf16_t* hidden, const float* row_scale, int T,
-                                                                    int H, int Tpad, bf16_t* out) {
+                                                                    int H, int Tpad, long long ld, bf16_t* out) {
   __shared__ uint16_t tile[64][66];
   const int t0 = blockIdx.x * 64, h0 = blockIdx.y * 64;
   const int r = threadIdx.x >> 3, cidx = threadIdx.x & 7;
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(256) void keep_scaled_transpose_kernel(const bf16_t
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       o[e] = (uint32_t)tile[8 * cidx + 2 * e][hl] | ((uint32_t)tile[8 * cidx + 2 * e + 1][hl] << 16);
-    *(u32x4_t*)(out + (long long)(h0 + hl) * Tpad + t0 + 8 * cidx) = o;
+    *(u32x4_t*)(out + (long long)(h0 + hl) * ld + t0 + 8 * cidx) = o;
   }
 }
 
