@@ -1,5 +1,7 @@
 // bf16 GEMM main loops for gfx950 (CDNA4): D[m,n] = sum_k A[m,k] * B[n,k] on v_mfma_f32_32x32x16_bf16
-// (lane l supplies row l % 32 and the eight k values 8*(l/32) .. 8*(l/32)+7 of each operand).
+// (lane l supplies row l % 32 and the eight k values 8*(l/32) .. 8*(l/32)+7 of each operand) or, on the
+// 8-wavefront 256x256x64 tile every large problem takes (kMi16 below), on v_mfma_f32_16x16x32_bf16
+// (lane l supplies row l % 16 and the eight k values 8*(l/16) .. 8*(l/16)+7).
 //
 // Work-group tile BM x BN, K step BK, WM x WN wavefronts (64 lanes each), every wavefront owning a
 // (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA blocks kept in fp32 accumulators.  Four loops, chosen by the
@@ -109,7 +111,7 @@ __device__ __forceinline__ int acc_col(int wn, int j, int lane) {
 
 // The 256x256x64 two-buffer direct-to-LDS loops of the 8-wavefront tile can run on v_mfma_f32_16x16x32_bf16 instead
 // of 32x32x16 (kMi16): same flops per cycle, half the fp32 accumulator registers read and written per flop - on this
-// power-limited part the same kernels run 6-10 % faster with it.  A 32x32 block (i, j) of a wavefront is then four
+// power-limited part the same kernels run 5 % faster with it.  A 32x32 block (i, j) of a wavefront is then four
 // 16x16 blocks (rh, ch), each one MFMA per 32-wide K slice, and the block's sixteen accumulator registers are
 //   element e = 4*(2*rh + ch) + r :  row = wm*WTM + i*32 + 16*rh + 4*(lane/16) + r
 //                                   col = wn*WTN + j*32 + 16*ch + (lane%16)
