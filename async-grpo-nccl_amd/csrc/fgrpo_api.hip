@@ -107,6 +107,7 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "wide_stores")) return &g_tune.wide_stores;
   if (!strcmp(key, "keep_panels")) return &g_tune.keep_panels;
   if (!strcmp(key, "keep_skip_dead")) return &g_tune.keep_skip_dead;
+  if (!strcmp(key, "dh_split")) return &g_tune.dh_split;
   return nullptr;
 }
 
@@ -166,6 +167,10 @@ int pick_variant(const Tuning& tn, int requested, long long M, long long N) {
 // ---- forward plan -------------------------------------------------------------------
 struct FwdPlan {
   int variant, tiles_v, tiles_t, nsplit;
+  // Token regions: the first t_main tokens (whole device rounds of token tiles at `nsplit` vocabulary splits) and, when
+  // t_main < T, the rest with a split count of their own (`nsplit_rem`), launched right behind them.
+  int t_main, nsplit_rem;
+  float4* part_rem;
   int Hp;            // padded contraction length
   bool copy_ops;     // operands are staged (fp32 split or padding) instead of used in place
   bf16_t *w_hi, *w_lo, *h_hi, *h_lo;
@@ -175,17 +180,20 @@ struct FwdPlan {
   size_t bytes;
 };
 
-int choose_nsplit(int tiles_t, int tiles_v, int slots, int forced, int prefer = 4) {
+// Device rounds x vocabulary tiles per work-group: the time of a launch in tile units.
+long long split_cost(int tiles_t, int tiles_v, int slots, int s) {
+  const long long blocks = (long long)tiles_t * s;
+  const long long rounds = (blocks + slots - 1) / slots;
+  const long long per = (tiles_v + s - 1) / s;
+  return rounds * per;
+}
+
+int choose_nsplit(int tiles_t, int tiles_v, int slots, int forced, int prefer = 4, int max_split = 64) {
   if (forced > 0) return forced < tiles_v ? forced : tiles_v;
   int best = 1;
   long long best_cost = -1;
-  const int cap = tiles_v < 64 ? tiles_v : 64;
-  auto cost_of = [&](int s) {
-    const long long blocks = (long long)tiles_t * s;
-    const long long rounds = (blocks + slots - 1) / slots;
-    const long long per = (tiles_v + s - 1) / s;
-    return rounds * per;
-  };
+  const int cap = tiles_v < max_split ? tiles_v : max_split;
+  auto cost_of = [&](int s) { return split_cost(tiles_t, tiles_v, slots, s); };
   for (int s = 1; s <= cap; ++s) {
     const long long cost = cost_of(s);
     if (best_cost < 0 || cost < best_cost) {
@@ -217,7 +225,31 @@ void plan_fwd(const Tuning& tn, FwdPlan& pl, void* ws, int T, int H, int V, int 
   // (4 token tiles per XCD) halve it (T=16384, H=8192, V=128256: 28.9 -> 24.9 ms; H=5120 and 3584 measure equal
   // or better with four).
   const int prefer = (16384LL * H * 2 > (192LL << 20)) ? 8 : 4;
-  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, num_cus() * c.wgs_per_cu, tn.fwd_nsplit, prefer);
+  const int slots = num_cus() * c.wgs_per_cu;
+  pl.nsplit = choose_nsplit(pl.tiles_t, pl.tiles_v, slots, tn.fwd_nsplit, prefer);
+  pl.t_main = T;
+  pl.nsplit_rem = 0;
+  // A token count that is not a whole number of device rounds (slots / prefer token tiles each) leaves the choice
+  // above between a last round that is nearly empty and a split count that fits the rounds but breaks up the 32
+  // work-group patches an XCD shares its operands in (T = 33000 instead of 32768: 14.7 instead of 12.8 ms).  Give the
+  // whole rounds the preferred split and the remaining token tiles a launch of their own, split as finely as it
+  // takes to spread them over the device, unless the tile count says that is more than 10 % dearer (the count knows
+  // nothing of the patches: by it alone 33 splits of 129 token tiles cost 306 tile times against 303 for the two
+  // regions, measured they are 15 % apart).
+  if (tn.fwd_nsplit <= 0 && tn.dh_split != 0 && pl.tiles_v >= prefer && slots % prefer == 0) {
+    const int per_round = slots / prefer;                       // token tiles of one full round
+    const int main_tiles = pl.tiles_t / per_round * per_round;
+    if (main_tiles > 0 && main_tiles < pl.tiles_t) {
+      const int rem_tiles = pl.tiles_t - main_tiles;
+      const int ns_rem = choose_nsplit(rem_tiles, pl.tiles_v, slots, 0, prefer, 128);
+      const long long two = split_cost(main_tiles, pl.tiles_v, slots, prefer) + split_cost(rem_tiles, pl.tiles_v, slots, ns_rem);
+      if (two * 100 <= split_cost(pl.tiles_t, pl.tiles_v, slots, pl.nsplit) * 110) {
+        pl.nsplit = prefer;
+        pl.t_main = main_tiles * c.bn;
+        pl.nsplit_rem = ns_rem;
+      }
+    }
+  }
   pl.Hp = (int)round_up(H, 64);
   pl.copy_ops = (dtype == FGRPO_F32) || (H % 64 != 0);
   Carver cv(ws);
@@ -232,6 +264,7 @@ void plan_fwd(const Tuning& tn, FwdPlan& pl, void* ws, int T, int H, int V, int 
   }
   pl.bias32 = has_bias ? cv.take<float>((size_t)V) : nullptr;
   pl.part = cv.take<float4>((size_t)pl.nsplit * T);
+  pl.part_rem = pl.t_main < T ? cv.take<float4>((size_t)pl.nsplit_rem * (T - pl.t_main)) : nullptr;
   pl.xt = cv.take<float>((size_t)T);
   pl.bytes = cv.total();
 }
@@ -505,6 +538,7 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   p.nsplit = pl.nsplit;
   p.group_t = tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
   if (pl.nsplit >= 8 && p.group_t * pl.nsplit > 32) p.group_t = 32 / pl.nsplit > 0 ? 32 / pl.nsplit : 1;   // one XCD's 32 work-groups per patch
+  const int c_bn = kCfg[pl.variant].bn;
   p.part = pl.part;
   p.xt = pl.xt;
   if (keep) {
@@ -527,16 +561,35 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
     HIP_TRY(hipGetLastError());
     p.keep_ref2 = ref2;
     p.keep_flag = flag;
-    rc = launch_fwd_keep(p, st);
-  } else {
-    rc = launch_fwd_variant(pl.variant, p, st);
   }
+  // One launch per token region: tokens [t0, t0 + count) with `nsplit` vocabulary splits, then their merge.
+  auto run_region = [&](int t0, int count, int nsplit, float4* part) -> int {
+    FwdParams q = p;
+    q.g.N = count;
+    for (int sg = 0; sg < q.g.nseg; ++sg) q.g.seg[sg].B += (long long)t0 * q.g.ldb;
+    q.labels += t0;
+    q.tiles_t = (count + c_bn - 1) / c_bn;
+    q.nsplit = nsplit;
+    q.group_t = tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
+    if (nsplit >= 8 && q.group_t * nsplit > 32) q.group_t = 32 / nsplit > 0 ? 32 / nsplit : 1;   // one XCD's 32 work-groups per patch
+    q.part = part;
+    q.xt += t0;
+    if (keep) {
+      q.keep += (long long)t0 * 256;           // token t0 of every 256-column block
+      q.keep_ref2 += t0;
+    }
+    const int rc2 = keep ? launch_fwd_keep(q, st) : launch_fwd_variant(pl.variant, q, st);
+    if (rc2) return rc2;
+    CombineParams c{part, pl.xt + t0, (const long long*)labels + t0, count, V, nsplit, lp_out + t0,
+                    ent_out ? ent_out + t0 : nullptr, lse_out ? lse_out + t0 : nullptr};
+    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((count + 255) / 256), dim3(256), 0, st, c);
+    HIP_TRY(hipGetLastError());
+    return 0;
+  };
+  rc = run_region(0, pl.t_main, pl.nsplit, pl.part);
   if (rc) return rc;
-
-  CombineParams c{pl.part, pl.xt, (const long long*)labels, T, V, pl.nsplit, lp_out, ent_out, lse_out};
-  hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((T + 255) / 256), dim3(256), 0, st, c);
-  HIP_TRY(hipGetLastError());
-  return 0;
+  if (pl.t_main < T) rc = run_region(pl.t_main, T - pl.t_main, pl.nsplit_rem, pl.part_rem);
+  return rc;
 }
 
 // Per-device address of `scratch`, resolved once per device with that device current.
@@ -831,8 +884,51 @@ struct KeptBwdPlan {
   int* m_tile_live;       // live 256-row tiles for the dH product
   bf16_t* hidden_scaled;  // [H x Tpad]: diag(a) hidden, transposed (the token contiguous), zero from T to Tpad
   float* dh_acc;          // [T x H] fp32, panels > 1 only
+  float* dh_part;         // fp32 tiles of the split contraction of dHidden's last row tiles (one per CU at most)
   size_t bytes;
 };
+// dHidden's tiles come in device rounds (one 256 x 256 tile per CU, each walking the whole vocabulary: 3.4 ms at
+// V = 151936, H = 1536); a token count just past a whole number of rounds (T = 33000: 129 x 6 tiles = 3.02 rounds)
+// would spend a fourth round on a handful of CUs (measured 14.1 ms against 10.3 at T = 32768).  Plan: row tiles
+// [0, main_tiles) as whole tiles in whole rounds; the others' contraction in ksplit pieces of kchunk columns, a
+// work-group each (at most kDhPartRounds per CU, which bounds the fp32 tiles they write); then a fixed-order sum of
+// the pieces.  The plan is taken when its rounds are at least 5 % fewer (T = 33000: 11.2 ms, 24000: 8.3 against
+// 10.4, 12000: 4.1 against 6.9; a last round that is half full gains little, the device is power-limited and
+// gives the CUs that do run more clock).
+struct DhSplitPlan {
+  int main_tiles;   // == tiles_m: no split
+  int ksplit, kchunk;
+};
+constexpr int kDhPartRounds = 3;      // fp32 tiles the split contraction may write: this many per CU
+DhSplitPlan plan_dh_split(int T, int H, int kv) {
+  const int tiles_m = (T + 255) / 256, tiles_n = (H + 255) / 256, slots = num_cus(), per_xcd = slots / 8;
+  DhSplitPlan d{tiles_m, 1, 0};
+  if (H % 4 != 0 || tiles_n > per_xcd) return d;
+  // time in device rounds of whole tiles.  Whole-tile launches deal row tiles round-robin to the 8 XCDs (or hand
+  // each a contiguous range): an XCD runs its share x tiles_n work-groups on slots / 8 CUs.
+  auto whole_rounds = [&](int row_tiles) { return ((row_tiles + 7) / 8 * tiles_n + per_xcd - 1) / per_xcd; };
+  const int blocks = (kv + 255) / 256;                         // 256-column blocks of the contraction
+  double best = (double)whole_rounds(tiles_m);
+  const int full = tiles_m * tiles_n / slots;
+  for (int f = full; f >= 0 && f >= full - 1; --f) {
+    const int main_tiles = 8 * (f * per_xcd / tiles_n);        // whole rounds on every XCD under either raster
+    const int tail = (tiles_m - main_tiles) * tiles_n;
+    if (tail <= 0) continue;
+    for (int ks = 2; ks <= 16 && tail * ks <= kDhPartRounds * slots; ++ks) {
+      const int per = (blocks + ks - 1) / ks;
+      if (per < 8) break;                                      // pieces under 32 K steps are not worth their tile store
+      const int pieces = (blocks + per - 1) / per;
+      const double cost = whole_rounds(main_tiles) + (double)((tail * pieces + slots - 1) / slots) * per / blocks + 0.03;
+      if (cost < best * 0.95) {
+        best = cost;
+        d.main_tiles = main_tiles;
+        d.ksplit = pieces;
+        d.kchunk = per * 256;
+      }
+    }
+  }
+  return d;
+}
 // Row length of the scaled, transposed copy of hidden: the padded token count plus 192 elements.  Rows 2 * Tpad bytes
 // apart (a multiple of 512, at T = 32768 exactly 64 KiB) all start in the same memory channel, and a tile of the dW
 // product reads 256 of them side by side.  Measured on that product at T = 32768, H = 1536: no padding 11.03 ms,
@@ -846,6 +942,7 @@ void plan_kept_bwd(KeptBwdPlan& pl, void* ws, int T, int H) {
   pl.m_tile_live = cv.take<int>((size_t)((T + 255) / 256));
   pl.hidden_scaled = cv.take<bf16_t>((size_t)H * kept_hs_ld(T));
   pl.dh_acc = cv.take<float>((size_t)T * H);     // always sized: a concurrent set_tuning must not make it short
+  pl.dh_part = cv.take<float>((size_t)kDhPartRounds * num_cus() * 256 * 256);
   pl.bytes = cv.total();
 }
 }  // namespace
@@ -942,7 +1039,40 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
         // so each XCD streams its rows of the buffer once (measured against groups of 4: dH 11.3 vs 11.5 ms,
         // dW 11.7 vs 12.1 at T=32768, H=1536, V=151936)
         PhaseScope ph(kPhaseDh, st);
-        rc = run_store_gemm_kmajor(tn, s, false, true, st, skip_dead ? -1 : 1);
+        const DhSplitPlan sp = (npanels == 1 && tn.dh_split != 0) ? plan_dh_split(T, H, kv) : DhSplitPlan{(T + 255) / 256, 1, 0};
+        if (sp.ksplit <= 1) {
+          rc = run_store_gemm_kmajor(tn, s, false, true, st, skip_dead ? -1 : 1);
+        } else {
+          // whole rounds of whole tiles, then the last row tiles with their contraction in pieces, then the sum
+          const int r0 = sp.main_tiles * 256, tr = T - r0;
+          if (r0 > 0) {
+            StoreParams m = s;
+            m.g.M = r0;
+            rc = run_store_gemm_kmajor(tn, m, false, true, st, skip_dead ? -1 : 1);
+            if (rc) return rc;
+          }
+          StoreParams t = s;
+          t.g.M = tr;
+          t.g.seg[0].A = ek_p + (long long)r0 * 256;               // row r0 of every 256-column block
+          t.c_out_bf16 = nullptr;
+          t.c_out_f32 = pl.dh_part;
+          t.row_scale = nullptr;                                    // applied once, to the sum
+          t.m_tile_live = skip_dead ? pl.m_tile_live + sp.main_tiles : nullptr;
+          t.ksplit = sp.ksplit;
+          t.kchunk = sp.kchunk;
+          t.part_slice = (long long)tr * H;
+          t.tiles_m = (tr + 255) / 256;
+          t.tiles_n = (H + 255) / 256;
+          t.nblocks = t.tiles_m * t.tiles_n * sp.ksplit;
+          t.wide_stores = can_store_wide(tn, t);
+          rc = launch_store_splitk(t, st);
+          if (rc) return rc;
+          const long long quads = (long long)tr * (H / 4);
+          hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st,
+                             (const float*)pl.dh_part, sp.ksplit, t.part_slice, tr, H, (long long)H,
+                             (const float*)pl.row_scale + r0, (bf16_t*)dH_out + (size_t)r0 * H);
+          HIP_TRY(hipGetLastError());
+        }
       }
       if (rc) return rc;
     }

@@ -17,6 +17,10 @@ int launch_store_variant(int variant, const StoreParams& p, hipStream_t st) {
   return rc;
 }
 
+int launch_store_splitk(const StoreParams& p, hipStream_t st) {
+  return launch_tile_kernel<gemm_store_kernel<Cfg8, false, true, true>, Cfg8>(p, p.nblocks, st);
+}
+
 int launch_store_kmajor(bool akm, bool bkm, const StoreParams& p, hipStream_t st) {
   const int nb = p.nblocks;
   if (akm && bkm) return launch_tile_kernel<gemm_store_kernel<Cfg8, true, true>, Cfg8>(p, nb, st);

@@ -593,6 +593,11 @@ struct StoreParams {
   const float* row_scale;  // optional [M]: output row m is multiplied by row_scale[m] (after alpha, before c_in)
   const int* m_tile_live;  // optional [tiles_m] (BM = 256 rows per tile): 0 = every row of the tile has row_scale 0,
                            // the contraction is skipped and the tile is written as zeros (or as c_in)
+  // Contraction split (gemm_store_kernel<..., SPLITK = true> only): work-group (tile, ks) contracts the K range
+  // [ks * kchunk, (ks + 1) * kchunk) and writes its fp32 tile into slice ks of c_out_f32 (slices part_slice
+  // elements apart); splitk_reduce_kernel adds the slices up in a fixed order.
+  int ksplit, kchunk;      // kchunk: a multiple of 256
+  long long part_slice;
 };
 
 // Output is either fp32 or bf16 (never both); rows/cols past M/N are skipped.
@@ -728,11 +733,43 @@ __device__ __forceinline__ void store_tile_lds(const StoreParams& p, f32x16_t (&
   }
 }
 
-template <class C, bool AKM = false, bool BKM = false>
-__global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StoreParams p) {
+// SPLITK (a K-contiguous, column-blocked A and a contraction-major B only): the tiles of a device round that would
+// otherwise run nearly empty are contracted in ksplit pieces by ksplit work-groups each.
+template <class C, bool AKM = false, bool BKM = false, bool SPLITK = false>
+__global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StoreParams p0) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
+
+  if constexpr (SPLITK) {
+    static_assert(!AKM && BKM && kMi16<C>, "split contraction: dHidden's layouts on the 16x16x32 tile");
+    StoreParams p = p0;
+    const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int ks = lid / tiles, w = lid - ks * tiles;     // pieces of one K range side by side: they share both operands' slices
+    const int tm = w % p.tiles_m, tn = w / p.tiles_m;
+    const int row0 = tm * C::BM, col0 = tn * C::BN;
+    const int k0 = ks * p.kchunk;
+    const int klen = (p.g.seg[0].K - k0) < p.kchunk ? (p.g.seg[0].K - k0) : p.kchunk;
+    const int b_rows = (p.g.kb_valid > 0 ? p.g.kb_valid : p.g.seg[0].K) - k0;        // rows of B that exist from k0 on
+    f32x16_t acc[C::TM][C::TN];
+    zero_acc<C>(acc);
+    const bool dead = (p.m_tile_live != nullptr && p.m_tile_live[tm] == 0) || klen <= 0 || b_rows <= 0;
+    if (!dead) {
+      p.g.seg[0].A += (long long)(k0 / 256) * p.g.a_blk;
+      p.g.seg[0].B += (long long)k0 * p.g.ldb;
+      p.g.seg[0].K = klen;
+      p.g.kb_valid = b_rows;
+      gemm_mainloop_km<C, false, true, true>(p.g, row0, col0, smem, acc);
+    }
+    p.c_out_f32 += (long long)ks * p.part_slice;
+    if (p.wide_stores)
+      store_tile_lds<C, false, false, true>(p, acc, 1.f, row0, col0, wm, wn, lane, wave, smem);
+    else
+      store_tile<C, false, false, true>(p, acc, 1.f, row0, col0, wm, wn, lane);
+    return;
+  }
+  const StoreParams& p = p0;
 
   int tm, tn;
   if (p.group_m > 0) {

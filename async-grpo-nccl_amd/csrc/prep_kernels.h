@@ -286,6 +286,30 @@ __global__ __launch_bounds__(256) void keep_scaled_transpose_kernel(const bf16_t
   }
 }
 
+// Sum of the ksplit fp32 slices a split contraction wrote (fixed order: bit-reproducible), times the row factor,
+// as bf16: out[m][n] = row_scale[m] * sum_ks part[ks][m][n].  Four columns per thread; ld % 4 == 0.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* part, int ksplit, long long slice, int M, int N,
+                                                            long long ld, const float* row_scale, bf16_t* out) {
+  const long long q = (long long)blockIdx.x * 256 + threadIdx.x;      // quad index
+  const int nq = N / 4;
+  if (q >= (long long)M * nq) return;
+  const int m = (int)(q / nq), n = (int)(q - (long long)m * nq) * 4;
+  const float* src = part + (long long)m * ld + n;
+  float4 s = *(const float4*)src;
+  for (int k = 1; k < ksplit; ++k) {
+    const float4 v = *(const float4*)(src + (long long)k * slice);
+    s.x += v.x;
+    s.y += v.y;
+    s.z += v.z;
+    s.w += v.w;
+  }
+  const float a = row_scale ? row_scale[m] : 1.f;
+  uint2 o;
+  o.x = pack_bf16x2(s.x * a, s.y * a);
+  o.y = pack_bf16x2(s.z * a, s.w * a);
+  *(uint2*)(out + (long long)m * ld + n) = o;
+}
+
 // dbias from the kept numerators: out[v] = sum_t a_t * E'[t][v].  One block owns 64 columns; its four row groups
 // are combined in a fixed order.
 __global__ void keep_col_sum_kernel(const bf16_t* e, long long blk, const float* row_scale, int T, int V,

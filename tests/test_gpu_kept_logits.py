@@ -190,6 +190,41 @@ def test_rows_without_gradient_are_skipped_exactly(dev, pattern):
         assert cos(res[1][0], dH0) >= 0.9999 and cos(res[1][1], dW0) >= 0.9999
 
 
+@pytest.mark.parametrize("tokens,H", [(64 * 256 + 700, 2048), (9000, 1024), (33 * 256 + 1, 1536)])
+def test_split_contraction_of_the_last_row_tiles(dev, tokens, H):
+    """dHidden's row tiles beyond whole device rounds (or all of them, when there are few) have their contraction
+    over the vocabulary split among several work-groups, whose fp32 tiles are then added in a fixed order: against
+    the same backward with the split switched off (equal up to the rounding of bf16 outputs summed in another
+    order), bit-identical between two runs, rows without gradient exact zeros, and dW untouched by the switch."""
+    from fgrpo import _lib, ops
+    V = 4000 if H == 2048 else 8492
+    g0 = torch.Generator().manual_seed(tokens)
+    hs = torch.randn(tokens, H, generator=g0).to(torch.bfloat16).to(dev)
+    W = (torch.randn(V, H, generator=g0) * 0.03).to(torch.bfloat16).to(dev)
+    y = torch.randint(0, V, (tokens,), generator=g0).to(dev)
+    g = (torch.randn(tokens, generator=g0) / tokens).to(dev)
+    g[tokens - 300: tokens - 40] = 0             # a dead stretch inside the last row tiles
+    g[100:700] = 0                               # and a whole dead tile (rows 256..511) in the first ones
+    assert ops.keep_supported(tokens, H, V, torch.bfloat16)
+    lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
+    res = {}
+    for split in (1, 0, 1):
+        _lib.set_tuning(dh_split=split)
+        try:
+            out = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
+        finally:
+            _lib.set_tuning(dh_split=1)
+        if split in res:
+            assert torch.equal(out[0], res[split][0]) and torch.equal(out[1], res[split][1])
+        res[split] = out
+    a, b = res[1][0].float(), res[0][0].float()
+    assert ((a - b).norm() / b.norm()).item() <= 3e-3 and cos(a, b) >= 0.99999
+    assert (res[1][0][g == 0] == 0).all()
+    assert torch.equal(res[1][1], res[0][1])
+    dH0, _, _ = ops.lmhead_bwd(hs, W, None, y, lse, g, None, 1.0, True, False, False, 0)
+    assert cos(res[1][0], dH0) >= 0.9999
+
+
 @pytest.mark.parametrize("tokens", [4321, 13 * 256 + 17])
 def test_wide_hidden_takes_the_patch_rasters(dev, tokens):
     """More than 8 column tiles (H = 2560: 10): the gradient GEMMs walk 4 x 8 tile patches per XCD - the grouped

@@ -199,6 +199,47 @@ def test_masked_only_lanes_of_the_last_vocabulary_tile_over_temperatures(dev, ke
         assert (ent[rows] - O.entropy_from_logits(logits)).abs().max().item() <= 5e-3, temp
 
 
+@pytest.mark.parametrize("keep", [False, True])
+def test_token_count_just_past_whole_device_rounds(dev, keep):
+    """67 token tiles = one whole device round of 64 (at four vocabulary splits) and three more: the forward runs the
+    round and the rest as two launches with split counts of their own.  Every output against the oracle on rows
+    sampled from both regions and around their border; the backward on the kept numerators against the recomputing
+    one (both read what the forward wrote for all tokens)."""
+    from fgrpo import ops
+    T, H, V = 64 * 256 + 700, 2048, 4000
+    g = torch.Generator().manual_seed(11)
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    weight = (torch.randn(V, H, generator=g) * 0.02).to(torch.bfloat16)
+    y = torch.randint(0, V, (T,), generator=g)
+    y[torch.rand(T, generator=g) < 0.05] = -100
+    assert ops.keep_supported(T, H, V, torch.bfloat16)
+    hd, wd, yd = hidden.to(dev), weight.to(dev), y.to(dev)
+    res = ops.lmhead_logprob_fwd(hd, wd, None, yd, 0.9, keep=keep)
+    lp, ent, lse = (t.cpu() for t in res[:3])
+    rows = torch.cat([torch.arange(0, T, 211), torch.arange(64 * 256 - 3, 64 * 256 + 3), torch.arange(T - 5, T)])
+    logits = O.project(weight.float(), None, hidden.float()[rows], 0.9)
+    valid = y[rows] != -100
+    want_lp = O.logprobs_from_logits(logits, y[rows])
+    assert (lp[rows] - want_lp).abs().max().item() <= LP_TOL_BF16
+    assert ((ent[rows] - O.entropy_from_logits(logits)) * valid).abs().max().item() <= 5e-3
+    assert (lse[rows] - torch.logsumexp(logits, -1)).abs().max().item() <= LP_TOL_BF16
+    gt = torch.randn(T, generator=g)
+    gt[y == -100] = 0
+    gd = gt.to(dev)
+    ref = ops.lmhead_bwd(hd, wd, None, yd, res[2], gd, None, 0.9, True, True, False)
+    if keep:
+        assert not ops.keep_overflowed(res[3], T, V)
+        got = ops.lmhead_bwd_kept(hd, wd, None, yd, res[2], gd, None, 0.9, res[3], True, True, False)
+        for a, b in zip(got[:2], ref[:2]):
+            assert cos(a, b) >= 0.9999
+            assert ((a.float() - b.float()).norm() / b.float().norm()).item() <= 1e-2
+    # the recomputing backward against autograd through the oracle's projection on the sampled rows
+    hs = hidden.float()[rows].clone().requires_grad_(True)
+    lpo = O.logprobs_from_logits(O.project(weight.float(), None, hs, 0.9), y[rows])
+    (lpo * gt[rows]).sum().backward()
+    assert cos(ref[0].cpu()[rows], hs.grad) >= COS_MIN
+
+
 # ------------------------------------------------------------------ gradient GEMMs on operands read in place
 @pytest.mark.parametrize("layout,M,N,K,k_valid", [
     ("b", 512, 256, 128, 0),
