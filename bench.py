@@ -387,6 +387,9 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed steps, run one 1 GiB device copy (reference point for traffic counters)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--tokens", type=int, default=None,
+                    help="pack this many tokens instead of the configuration's own count (the reference fills a "
+                         "micro-batch up to a budget, 36000 by default: token counts off the 256-token tile grid)")
     ap.add_argument("--attention", action="store_true",
                     help="time the packed attention kernels instead (prints their own JSON line)")
     ap.add_argument("--attention-shape", choices=["cfg1", "long"], default="cfg1")
@@ -410,8 +413,12 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = make_workload(args.config, seed=args.seed, device=dev,
-                      overrides=None if args.reward_p is None else dict(reward_p=args.reward_p))
+    over = {}
+    if args.reward_p is not None:
+        over["reward_p"] = args.reward_p
+    if args.tokens is not None:
+        over["tokens"] = args.tokens
+    w = make_workload(args.config, seed=args.seed, device=dev, overrides=over or None)
     p = w.params
     T, H, V = w.T, w.H, w.V
     fwd_only = p["forward_only"]
