@@ -204,7 +204,9 @@ def test_split_contraction_of_the_last_row_tiles(dev, tokens, H):
     y = torch.randint(0, V, (tokens,), generator=g0).to(dev)
     g = (torch.randn(tokens, generator=g0) / tokens).to(dev)
     g[tokens - 300: tokens - 40] = 0             # a dead stretch inside the last row tiles
-    g[100:700] = 0                               # and a whole dead tile (rows 256..511) in the first ones
+    g[100:700] = 0                               # a whole dead tile (rows 256..511) in the first ones
+    nt = (tokens + 255) // 256
+    g[(nt - 3) * 256: (nt - 2) * 256] = 0        # and one among the last ones
     assert ops.keep_supported(tokens, H, V, torch.bfloat16)
     lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
     res = {}
