@@ -107,7 +107,7 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "wide_stores")) return &g_tune.wide_stores;
   if (!strcmp(key, "keep_panels")) return &g_tune.keep_panels;
   if (!strcmp(key, "keep_skip_dead")) return &g_tune.keep_skip_dead;
-  if (!strcmp(key, "dh_split")) return &g_tune.dh_split;
+  if (!strcmp(key, "tail_split")) return &g_tune.tail_split;
   return nullptr;
 }
 
@@ -236,7 +236,7 @@ void plan_fwd(const Tuning& tn, FwdPlan& pl, void* ws, int T, int H, int V, int 
   // takes to spread them over the device, unless the tile count says that is more than 10 % dearer (the count knows
   // nothing of the patches: by it alone 33 splits of 129 token tiles cost 306 tile times against 303 for the two
   // regions, measured they are 15 % apart).
-  if (tn.fwd_nsplit <= 0 && tn.dh_split != 0 && pl.tiles_v >= prefer && slots % prefer == 0) {
+  if (tn.fwd_nsplit <= 0 && tn.tail_split != 0 && pl.tiles_v >= prefer && slots % prefer == 0) {
     const int per_round = slots / prefer;                       // token tiles of one full round
     const int main_tiles = pl.tiles_t / per_round * per_round;
     if (main_tiles > 0 && main_tiles < pl.tiles_t) {
@@ -900,7 +900,7 @@ struct DhSplitPlan {
   int ksplit, kchunk;
 };
 constexpr int kDhPartRounds = 3;      // fp32 tiles the split contraction may write: this many per CU
-DhSplitPlan plan_dh_split(int T, int H, int kv) {
+DhSplitPlan plan_tail_split(int T, int H, int kv) {
   const int tiles_m = (T + 255) / 256, tiles_n = (H + 255) / 256, slots = num_cus(), per_xcd = slots / 8;
   DhSplitPlan d{tiles_m, 1, 0};
   if (H % 4 != 0 || tiles_n > per_xcd) return d;
@@ -1039,7 +1039,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
         // so each XCD streams its rows of the buffer once (measured against groups of 4: dH 11.3 vs 11.5 ms,
         // dW 11.7 vs 12.1 at T=32768, H=1536, V=151936)
         PhaseScope ph(kPhaseDh, st);
-        const DhSplitPlan sp = (npanels == 1 && tn.dh_split != 0) ? plan_dh_split(T, H, kv) : DhSplitPlan{(T + 255) / 256, 1, 0};
+        const DhSplitPlan sp = (npanels == 1 && tn.tail_split != 0) ? plan_tail_split(T, H, kv) : DhSplitPlan{(T + 255) / 256, 1, 0};
         if (sp.ksplit <= 1) {
           rc = run_store_gemm_kmajor(tn, s, false, true, st, skip_dead ? -1 : 1);
         } else {

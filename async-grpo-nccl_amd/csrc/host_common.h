@@ -89,7 +89,7 @@ struct Tuning {
   int attn_heads = 0;      // query heads per work-group of the attention forward / dQ kernels (1, 2, 4); 0 = heuristic
   int wide_stores = 1;     // GEMM epilogues write 16-byte pieces through an LDS patch where alignment allows
   int keep_skip_dead = 1;  // kept-path backward skips stretches of tokens that carry no gradient
-  int dh_split = 1;        // kept-path dHidden: last partial device round as a split contraction; forward: token regions
+  int tail_split = 1;        // kept-path dHidden: last partial device round as a split contraction; forward: token regions
   int keep_panels = 0;     // kept-logits backward: vocabulary panels of the gradient GEMMs; 0 = one
 };
 extern Tuning g_tune;

@@ -211,11 +211,11 @@ def test_split_contraction_of_the_last_row_tiles(dev, tokens, H):
     lp, ent, lse, kept = ops.lmhead_logprob_fwd(hs, W, None, y, 1.0, keep=True)
     res = {}
     for split in (1, 0, 1):
-        _lib.set_tuning(dh_split=split)
+        _lib.set_tuning(tail_split=split)
         try:
             out = ops.lmhead_bwd_kept(hs, W, None, y, lse, g, None, 1.0, kept, True, True, False)
         finally:
-            _lib.set_tuning(dh_split=1)
+            _lib.set_tuning(tail_split=1)
         if split in res:
             assert torch.equal(out[0], res[split][0]) and torch.equal(out[1], res[split][1])
         res[split] = out
