@@ -746,8 +746,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void gemm_store_kernel(const StorePa
     StoreParams p = p0;
     const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int tiles = p.tiles_m * p.tiles_n;
-    const int ks = lid / tiles, w = lid - ks * tiles;     // pieces of one K range side by side: they share both operands' slices
-    const int tm = w % p.tiles_m, tn = w / p.tiles_m;
+    // pieces of one K range side by side, and of them the column tiles of a row tile: they stream the same slice of
+    // A, the big operand (rows fastest instead: 6.7 against 5.6 ms at T = 16384, H = 1536, V = 151936)
+    const int ks = lid / tiles, w = lid - ks * tiles;
+    const int tm = w / p.tiles_n, tn = w - tm * p.tiles_n;
     const int row0 = tm * C::BM, col0 = tn * C::BN;
     const int k0 = ks * p.kchunk;
     const int klen = (p.g.seg[0].K - k0) < p.kchunk ? (p.g.seg[0].K - k0) : p.kchunk;
