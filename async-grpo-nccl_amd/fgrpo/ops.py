@@ -84,7 +84,8 @@ def set_fwd_event_sink(sink) -> None:
 
 
 def keep_supported(T: int, H: int, V: int, dtype: torch.dtype) -> bool:
-    """Whether the kept-logits forward/backward pair handles this problem (bf16, H % 256 == 0, device-filling)."""
+    """Whether the kept-logits forward/backward pair handles this problem: bf16, H % 64 == 0 and a vocabulary side
+    that fills the device (V/256 x H/256 tiles for at least half the CUs; any token count)."""
     if dtype != torch.bfloat16 or T <= 0:
         return False
     return bool(_lib.load().fgrpo_keep_supported(int(T), int(H), int(V), _lib.BF16))

@@ -120,7 +120,8 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
  * then the references and the flag.  workspace of the backward: fgrpo_lmhead_bwd_kept_workspace bytes (the token
  * factors, the scaled transposed copy of hidden, and an fp32 dH accumulator used only when the tuning key keep_panels splits
  * the products into vocabulary panels).
- * Supported (fgrpo_keep_supported() != 0): bf16, H a multiple of 64, enough tiles to fill the device; anything
+ * Supported (fgrpo_keep_supported() != 0): bf16, H a multiple of 64, V/256 x H/256 tiles for at least half the
+ * CUs (any token count); anything
  * else returns FGRPO_ERR_UNSUPPORTED - use the recomputing pair.  dH_out / dW_out / dbias_out as in
  * fgrpo_lmhead_bwd. */
 int fgrpo_keep_supported(int T, int H, int V, int dtype);

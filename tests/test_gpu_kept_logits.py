@@ -190,6 +190,40 @@ def test_rows_without_gradient_are_skipped_exactly(dev, pattern):
         assert cos(res[1][0], dH0) >= 0.9999 and cos(res[1][1], dW0) >= 0.9999
 
 
+@pytest.mark.parametrize("tokens", [1, 77, 300, 1000])
+def test_few_tokens_take_the_kept_path_too(dev, tokens):
+    """The kept numerators need the vocabulary side to fill the device, not the token side: with one or a few token
+    tiles the forward splits the vocabulary finely and dHidden its contraction.  Forward against the oracle row by
+    row, the backward against the oracle's autograd, for token counts down to a single token."""
+    from fgrpo import ops
+    H, V = 512, 33000              # 129 vocabulary tiles: the large tile for any token count
+    assert ops.keep_supported(tokens, H, V, torch.bfloat16)
+    g0 = torch.Generator().manual_seed(100 + tokens)
+    hidden = torch.randn(tokens, H, generator=g0).to(torch.bfloat16)
+    weight = (torch.randn(V, H, generator=g0) * 0.05).to(torch.bfloat16)
+    bias = (torch.randn(V, generator=g0) * 0.3).to(torch.bfloat16)
+    y = torch.randint(0, V, (tokens,), generator=g0)
+    if tokens > 10:
+        y[3] = -100
+    gt = torch.randn(tokens, generator=g0)
+    gt[y == -100] = 0
+    hd, wd, bd, yd, gd = (t.to(dev) for t in (hidden, weight, bias, y, gt))
+    lp, ent, lse, kept = ops.lmhead_logprob_fwd(hd, wd, bd, yd, 0.8, keep=True)
+    assert not ops.keep_overflowed(kept, tokens, V)
+    dH, dW, db = ops.lmhead_bwd_kept(hd, wd, bd, yd, lse, gd, None, 0.8, kept, True, True, True)
+    hs = hidden.float().requires_grad_(True)
+    Wo = weight.float().requires_grad_(True)
+    bo = bias.float().requires_grad_(True)
+    logits = O.project(Wo, bo, hs, 0.8)
+    want_lp = O.logprobs_from_logits(logits, y)
+    valid = y != -100
+    assert (lp.cpu() - want_lp.detach()).abs().max().item() <= LP_TOL_BF16
+    assert ((ent.cpu() - O.entropy_from_logits(logits.detach())) * valid).abs().max().item() <= 5e-3
+    (want_lp * gt).sum().backward()
+    assert cos(dH, hs.grad) >= COS_MIN and cos(dW, Wo.grad) >= COS_MIN and cos(db, bo.grad) >= COS_MIN
+    assert (dH.cpu()[~valid] == 0).all()
+
+
 @pytest.mark.parametrize("tokens,H", [(64 * 256 + 700, 2048), (9000, 1024), (33 * 256 + 1, 1536)])
 def test_split_contraction_of_the_last_row_tiles(dev, tokens, H):
     """dHidden's row tiles beyond whole device rounds (or all of them, when there are few) have their contraction
