@@ -307,9 +307,10 @@ def test_keep_refuses_what_it_cannot_do(dev):
 
 
 # ------------------------------------------------------------------ full benchmark sizes through the drop-in
-@pytest.mark.parametrize("name,keep", [("cfg1", True), ("cfg1", False), ("cfg2", True), ("cfg2", False),
-                                       ("cfg4", True), ("cfg4", False)])
-def test_full_size_through_the_drop_in(dev, name, keep):
+@pytest.mark.parametrize("name,keep,tokens", [("cfg1", True, None), ("cfg1", False, None), ("cfg2", True, None),
+                                              ("cfg2", False, None), ("cfg4", True, None), ("cfg4", False, None),
+                                              ("cfg1", True, 33000)])
+def test_full_size_through_the_drop_in(dev, name, keep, tokens):
     """grpo_loss_and_entropy_ce_fn exactly as bench.py calls it (KL to the reference policy, mean over samples of
     per-sample token means, cu_seqlens, the configuration's chunk hint), then backward with a non-unit upstream
     scale.  Checked: loss and the four per-token diagnostics against the oracle's objective evaluated on the
@@ -318,10 +319,12 @@ def test_full_size_through_the_drop_in(dev, name, keep):
     import grpo_loss as G
     from fgrpo import ops
     from fgrpo.synthetic import make_workload
-    w = make_workload(name, seed=0, device=dev)
+    # tokens: a count off the 256-token tile grid (129 token tiles at 33000: the forward's two token regions and the
+    # split contraction of dHidden's last row tile, at the benchmark's H and V)
+    w = make_workload(name, seed=0, device=dev, overrides=None if tokens is None else dict(tokens=tokens))
     p = w.params
     T, H, V = w.T, w.H, w.V
-    assert ops.keep_supported(T, H, V, torch.bfloat16)
+    assert ops.keep_supported(T, H, V, torch.bfloat16) and (tokens is None or T == tokens)
     shifted = ops.shift_labels(w.labels).reshape(-1)
     hs2 = w.hidden.reshape(T, H)
     adv = group_adv(w, p["adv_eps"]).to(dev)
