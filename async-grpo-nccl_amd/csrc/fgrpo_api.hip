@@ -85,7 +85,7 @@ struct PhaseScope {
     if (slot >= 0) (void)hipEventRecord(g_phase.ev[2 * slot + 1], st);
   }
 };
-enum { kPhaseDlogits = 0, kPhaseDh = 1, kPhaseDw = 2, kPhaseOther = 3 };
+enum { kPhaseDlogits = 0, kPhaseDh = 1, kPhaseDw = 2, kPhaseOther = 3, kPhaseFwd = 4 };
 
 
 int* tuning_slot(const char* key) {
@@ -507,7 +507,7 @@ int* keep_flag_of(void* keep, int T, int V) {
 
 int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
                       int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
-                      size_t ws_bytes, void* stream, void* keep = nullptr) {
+                      size_t ws_bytes, void* stream, void* keep = nullptr, const Tuning* snapshot = nullptr) {
   hipStream_t st = (hipStream_t)stream;
   if (!hidden || !weight || !labels || !lp_out) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: null argument");
   if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: T=%d H=%d V=%d", T, H, V);
@@ -515,7 +515,7 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: inv_temperature must be positive");
   if (!ws || !aligned16(ws)) return fail(FGRPO_ERR_WORKSPACE, "logprob_fwd: workspace null or misaligned");
   if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "logprob_fwd: hidden/weight must be 16-byte aligned");
-  Tuning tn = g_tune;   // one reading of the tuning state per call
+  Tuning tn = snapshot ? *snapshot : g_tune;   // one reading of the tuning state per call
   if (keep) tn.fwd_variant = 8;
   FwdPlan pl;
   plan_fwd(tn, pl, ws, T, H, V, dtype, bias != nullptr);
@@ -881,15 +881,6 @@ void kept_panels(const Tuning& tn, int T, int H, int V, int& panel, int& npanels
 }  // namespace
 
 namespace {
-struct KeptBwdPlan {
-  float* row_scale;       // [T]
-  int* k_runs;            // live runs of the token axis for the dW product
-  int* m_tile_live;       // live 256-row tiles for the dH product
-  bf16_t* hidden_scaled;  // [H x Tpad]: diag(a) hidden, transposed (the token contiguous), zero from T to Tpad
-  float* dh_acc;          // [T x H] fp32, panels > 1 only
-  float* dh_part;         // fp32 tiles of the split contraction of dHidden's last row tiles (one per CU at most)
-  size_t bytes;
-};
 // dHidden's tiles come in device rounds (one 256 x 256 tile per CU, each walking the whole vocabulary: 3.4 ms at
 // V = 151936, H = 1536); a token count just past a whole number of rounds (T = 33000: 129 x 6 tiles = 3.02 rounds)
 // would spend a fourth round on a handful of CUs (measured 14.1 ms against 10.3 at T = 32768).  Plan: row tiles
@@ -938,69 +929,103 @@ DhSplitPlan plan_tail_split(int T, int H, int kv) {
 // 64 bytes 11.86 (rows then straddle 128-byte lines), 128 bytes 10.69, 256 / 384 / 640 / 2176 bytes 10.55-10.59.
 long long kept_hs_ld(int T) { return round_up(T, 256) + 192; }
 
-void plan_kept_bwd(KeptBwdPlan& pl, void* ws, int T, int H) {
+// Workspace of the kept-numerators backward, laid out from the tuning state the call itself will use: the fp32 dH
+// accumulator exists only when the products are split into vocabulary panels, the fp32 tiles of the split
+// contraction only when the plan takes it.
+struct KeptBwdPlan {
+  int panel, npanels;     // vocabulary panels of the two products
+  DhSplitPlan split;      // of dHidden's last row tiles (one panel only)
+  float* row_scale;       // [T]
+  int* k_runs;            // live runs of the token axis for the dW product
+  int* m_tile_live;       // live 256-row tiles for the dH product
+  bf16_t* hidden_scaled;  // [H x (Tpad + 192)]: diag(a) hidden, transposed (the token contiguous), zero from T to Tpad
+  float* dh_acc;          // [T x H] fp32, panels > 1 only
+  float* dh_part;         // fp32 tiles of the split contraction of dHidden's last row tiles
+  float* bias32;          // [V] fp32 copy of the bias for the recomputing fall-back
+  size_t bytes;
+};
+void plan_kept_bwd(const Tuning& tn, KeptBwdPlan& pl, void* ws, int T, int H, int V, bool has_bias, bool want_dh,
+                   bool want_dw) {
+  kept_panels(tn, T, H, V, pl.panel, pl.npanels);
+  const int tiles_m = (T + 255) / 256;
+  pl.split = (want_dh && pl.npanels == 1 && tn.tail_split != 0) ? plan_tail_split(T, H, (int)round_up(V, 256))
+                                                                : DhSplitPlan{tiles_m, 1, 0};
   Carver cv(ws);
   pl.row_scale = cv.take<float>((size_t)T);
   pl.k_runs = cv.take<int>((size_t)(2 + 2 * kRunCap));
-  pl.m_tile_live = cv.take<int>((size_t)((T + 255) / 256));
-  pl.hidden_scaled = cv.take<bf16_t>((size_t)H * kept_hs_ld(T));
-  pl.dh_acc = cv.take<float>((size_t)T * H);     // always sized: a concurrent set_tuning must not make it short
-  pl.dh_part = cv.take<float>((size_t)kDhPartRounds * num_cus() * 256 * 256);
+  pl.m_tile_live = cv.take<int>((size_t)tiles_m);
+  pl.hidden_scaled = want_dw ? cv.take<bf16_t>((size_t)H * kept_hs_ld(T)) : nullptr;
+  pl.dh_acc = (want_dh && pl.npanels > 1) ? cv.take<float>((size_t)T * H) : nullptr;
+  pl.dh_part = pl.split.ksplit > 1 ? cv.take<float>((size_t)pl.split.ksplit * (T - pl.split.main_tiles * 256) * H) : nullptr;
+  pl.bias32 = has_bias ? cv.take<float>((size_t)V) : nullptr;
   pl.bytes = cv.total();
 }
-}  // namespace
 
-size_t fgrpo_lmhead_bwd_kept_workspace(int T, int H, int V, int dtype) {
-  if (T <= 0 || H <= 0 || V <= 0 || dtype != FGRPO_BF16) return 0;
+// Where the products of one call go when the caller walks the tokens in chunks: dW (and dbias) are sums over all
+// tokens, carried in fp32 from chunk to chunk.
+struct KeptBwdSums {
+  const float* dw_in = nullptr;     // [V x H] fp32 sum of the earlier chunks, or null
+  float* dw_out_f32 = nullptr;      // where the sum goes on (null: this is the last chunk, dW_out takes it in `dtype`)
+  const float* db_in = nullptr;     // the same for dbias [V]
+  float* db_out_f32 = nullptr;
+};
+
+int kept_bwd_impl(const Tuning& tn, const void* hidden, const void* weight, const void* bias, const int64_t* labels,
+                  const float* lse, const float* g, const float* gout_dev, float inv_temp, int T, int H, int V,
+                  void* logits_keep, void* dH_out, void* dW_out, void* dbias_out, const KeptBwdSums& sums, void* ws,
+                  size_t ws_bytes, hipStream_t st) {
+  const bool want_dh = dH_out != nullptr, want_dw = dW_out != nullptr || sums.dw_out_f32 != nullptr;
+  const bool want_db = dbias_out != nullptr || sums.db_out_f32 != nullptr;
   KeptBwdPlan pl;
-  plan_kept_bwd(pl, nullptr, T, H);
-  return pl.bytes;
-}
-
-int fgrpo_keep_overflowed(const void* logits_keep, int T, int V, void* stream) {
-  if (!logits_keep || T <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "keep_overflowed: bad argument");
-  int flag = 0;
-  HIP_TRY(hipMemcpyAsync(&flag, keep_flag_of(const_cast<void*>(logits_keep), T, V), sizeof(int), hipMemcpyDeviceToHost,
-                         (hipStream_t)stream));
-  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-  return flag != 0 ? 1 : 0;
-}
-
-int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bias, const int64_t* labels,
-                          const float* lse, const float* g, const float* gout_dev, float inv_temp, int T, int H, int V,
-                          int dtype, void* logits_keep, size_t logits_keep_bytes, void* dH_out, void* dW_out,
-                          void* dbias_out, void* ws, size_t ws_bytes, void* stream) {
-  hipStream_t st = (hipStream_t)stream;
-  if (!hidden || !weight || !labels || !lse || !g) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: null argument");
-  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: T=%d H=%d V=%d", T, H, V);
-  if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: inv_temperature must be positive");
-  const Tuning tn = g_tune;
-  if (!keep_supported(tn, T, H, V, dtype))
-    return fail(FGRPO_ERR_UNSUPPORTED, "lmhead_bwd_kept: needs bf16, H %% 64 == 0 and V/256 x H/256 tiles for half the CUs (T=%d H=%d V=%d)", T, H, V);
-  if (!logits_keep || !aligned16(logits_keep) || logits_keep_bytes < keep_bytes(T, V))
-    return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: kept buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
-  if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: dbias requested without a bias");
-  if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "lmhead_bwd_kept: hidden/weight must be 16-byte aligned");
-  if (!dH_out && !dW_out && !dbias_out) return 0;
-  KeptBwdPlan pl;
-  plan_kept_bwd(pl, ws, T, H);
+  plan_kept_bwd(tn, pl, ws, T, H, V, bias != nullptr, want_dh, want_dw);
   if (!ws || !aligned16(ws) || ws_bytes < pl.bytes)
     return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: workspace null, misaligned or smaller than %zu bytes", pl.bytes);
   const int Tpad = (int)round_up(T, 256);
   const long long blk = (long long)Tpad * 256;
   bf16_t* ek = (bf16_t*)logits_keep;
-  int panel = 0, npanels = 0;
-  kept_panels(tn, T, H, V, panel, npanels);
+  const int panel = pl.panel, npanels = pl.npanels;
+  int* flag = keep_flag_of(logits_keep, T, V);
   // rows without a gradient (zero advantage, ignored label) are skipped by 256-row tile (dH) and 64-row K step (dW)
   const bool skip_dead = tn.keep_skip_dead != 0 && (T + 63) / 64 <= kLiveMaxChunks;
 
   {
     PhaseScope ph(kPhaseDlogits, st);
     KeepPrepParams k{ek, blk, keep_ref2_of(logits_keep, T, V), keep_xy_of(logits_keep, T, V), (const long long*)labels, lse, g, gout_dev, inv_temp,
-                     (const bf16_t*)hidden, T, H, V, pl.row_scale};
+                     (const bf16_t*)hidden, T, H, V, pl.row_scale, flag};
     hipLaunchKernelGGL(keep_backward_prep_kernel, dim3((T + 3) / 4), dim3(256), 0, st, k);
     HIP_TRY(hipGetLastError());
-    if (dW_out)
+    {
+      // Out-of-range batches (the forward raised the buffer's flag): the decision is taken on the device.  This launch
+      // returns at once unless the flag is set; when it is, it overwrites the whole buffer with dLogits recomputed
+      // from the operands (the kernel of the recomputing backward, one panel over the whole vocabulary, same
+      // layout), and the prep kernel above has set the row factors to 1: the products below then are that backward.
+      DsParams d;
+      memset(&d, 0, sizeof(d));
+      int rc = stage_logit_operands(d.g, hidden, weight, T, H, V, FGRPO_BF16, false, H, nullptr, nullptr, nullptr, nullptr, st);
+      if (rc) return rc;
+      if (bias) {
+        hipLaunchKernelGGL(to_f32_kernel, dim3((V + 255) / 256), dim3(256), 0, st, bias, 0, pl.bias32, V);
+        HIP_TRY(hipGetLastError());
+      }
+      d.bias = bias ? pl.bias32 : nullptr;
+      d.labels = (const long long*)labels;
+      d.lse = lse;
+      d.gtok = g;
+      d.gout = gout_dev;
+      d.inv_temp = inv_temp;
+      d.v0 = 0;
+      d.tiles_t = Tpad / 256;
+      d.tiles_v = (V + 255) / 256;
+      d.nsplit = choose_nsplit(d.tiles_t, d.tiles_v, num_cus(), tn.ds_nsplit > 0 ? tn.ds_nsplit : tn.fwd_nsplit, 8);
+      d.group_t = tn.ds_group_t > 0 ? tn.ds_group_t : d.nsplit == 8 ? 2 : tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
+      d.tv_hi = ek;
+      d.ld_tv = round_up(V, 256);
+      d.tv_blk = blk;
+      d.gate = flag;
+      rc = launch_ds_variant(8, false, d, st);
+      if (rc) return rc;
+    }
+    if (want_dw)
       hipLaunchKernelGGL(keep_scaled_transpose_kernel, dim3(Tpad / 64, H / 64), dim3(256), 0, st, (const bf16_t*)hidden,
                          (const float*)pl.row_scale, T, H, Tpad, kept_hs_ld(T), pl.hidden_scaled);
     if (skip_dead) {
@@ -1016,7 +1041,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
     const int rows = (V - v0) < panel ? (V - v0) : panel;      // vocabulary rows of W / dW in this panel
     const int kv = (int)round_up(rows, 256);                   // columns of the panel (zero past V)
     bf16_t* ek_p = ek + (long long)(v0 / 256) * blk;
-    if (dH_out) {   // dH[T x H] (+)= diag(a) E'[T x kv] W[v0 : v0+rows, H]: A column-blocked K-contiguous, B = W read in place
+    if (want_dh) {   // dH[T x H] (+)= diag(a) E'[T x kv] W[v0 : v0+rows, H]: A column-blocked K-contiguous, B = W read in place
       StoreParams s;
       memset(&s, 0, sizeof(s));
       s.g.M = T;
@@ -1042,7 +1067,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
         // so each XCD streams its rows of the buffer once (measured against groups of 4: dH 11.3 vs 11.5 ms,
         // dW 11.7 vs 12.1 at T=32768, H=1536, V=151936)
         PhaseScope ph(kPhaseDh, st);
-        const DhSplitPlan sp = (npanels == 1 && tn.tail_split != 0) ? plan_tail_split(T, H, kv) : DhSplitPlan{(T + 255) / 256, 1, 0};
+        const DhSplitPlan sp = pl.split;
         if (sp.ksplit <= 1) {
           rc = run_store_gemm_kmajor(tn, s, false, true, st, skip_dead ? -1 : 1);
         } else {
@@ -1079,7 +1104,7 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       }
       if (rc) return rc;
     }
-    if (dW_out) {   // dW[v0 : v0+rows, H] = E'^T[rows x Tpad] (diag(a) hidden)^T[H x Tpad]^T: A read where the forward left it
+    if (want_dw) {  // dW[v0 : v0+rows, H] = E'^T[rows x Tpad] (diag(a) hidden)^T[H x Tpad]^T: A read where the forward left it
                     // (the token is its row), B a token-contiguous copy, so that only A needs transposing LDS reads
       StoreParams s;
       memset(&s, 0, sizeof(s));
@@ -1094,7 +1119,11 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       s.g.k_runs = skip_dead ? pl.k_runs : nullptr;
       s.ldc = H;
       s.alpha = 1.f;
-      s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
+      s.c_in = sums.dw_in ? sums.dw_in + (size_t)v0 * H : nullptr;
+      if (sums.dw_out_f32)
+        s.c_out_f32 = sums.dw_out_f32 + (size_t)v0 * H;
+      else
+        s.c_out_bf16 = (bf16_t*)dW_out + (size_t)v0 * H;
       {
         PhaseScope ph(kPhaseDw, st);
         rc = run_store_gemm_kmajor(tn, s, true, false, st, 1);
@@ -1102,13 +1131,49 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
       if (rc) return rc;
     }
   }
-  if (dbias_out) {
+  if (want_db) {
     PhaseScope ph(kPhaseOther, st);
     hipLaunchKernelGGL(keep_col_sum_kernel, dim3((V + 63) / 64), dim3(256), 0, st, ek, blk, pl.row_scale, T, V,
-                       (bf16_t*)dbias_out);
+                       sums.db_in, sums.db_out_f32, sums.db_out_f32 ? nullptr : (bf16_t*)dbias_out);
     HIP_TRY(hipGetLastError());
   }
   return 0;
+}
+}  // namespace
+
+size_t fgrpo_lmhead_bwd_kept_workspace(int T, int H, int V, int dtype) {
+  if (T <= 0 || H <= 0 || V <= 0 || dtype != FGRPO_BF16) return 0;
+  KeptBwdPlan pl;
+  plan_kept_bwd(g_tune, pl, nullptr, T, H, V, true, true, true);
+  return pl.bytes;
+}
+
+int fgrpo_keep_overflowed(const void* logits_keep, int T, int V, void* stream) {
+  if (!logits_keep || T <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "keep_overflowed: bad argument");
+  int flag = 0;
+  HIP_TRY(hipMemcpyAsync(&flag, keep_flag_of(const_cast<void*>(logits_keep), T, V), sizeof(int), hipMemcpyDeviceToHost,
+                         (hipStream_t)stream));
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return flag != 0 ? 1 : 0;
+}
+
+int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bias, const int64_t* labels,
+                          const float* lse, const float* g, const float* gout_dev, float inv_temp, int T, int H, int V,
+                          int dtype, void* logits_keep, size_t logits_keep_bytes, void* dH_out, void* dW_out,
+                          void* dbias_out, void* ws, size_t ws_bytes, void* stream) {
+  if (!hidden || !weight || !labels || !lse || !g) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: null argument");
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: T=%d H=%d V=%d", T, H, V);
+  if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: inv_temperature must be positive");
+  const Tuning tn = g_tune;
+  if (!keep_supported(tn, T, H, V, dtype))
+    return fail(FGRPO_ERR_UNSUPPORTED, "lmhead_bwd_kept: needs bf16, H %% 64 == 0 and V/256 x H/256 tiles for half the CUs (T=%d H=%d V=%d)", T, H, V);
+  if (!logits_keep || !aligned16(logits_keep) || logits_keep_bytes < keep_bytes(T, V))
+    return fail(FGRPO_ERR_WORKSPACE, "lmhead_bwd_kept: kept buffer null, misaligned or smaller than %zu bytes", keep_bytes(T, V));
+  if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "lmhead_bwd_kept: dbias requested without a bias");
+  if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "lmhead_bwd_kept: hidden/weight must be 16-byte aligned");
+  if (!dH_out && !dW_out && !dbias_out) return 0;
+  return kept_bwd_impl(tn, hidden, weight, bias, labels, lse, g, gout_dev, inv_temp, T, H, V, logits_keep, dH_out, dW_out,
+                       dbias_out, KeptBwdSums{}, ws, ws_bytes, (hipStream_t)stream);
 }
 
 int fgrpo_phase_timing_begin(void) {
@@ -1134,7 +1199,7 @@ int fgrpo_phase_timing_end(float* ms_by_phase, int* brackets_by_phase) {
   for (int i = 0; i < t.n; ++i) {
     float ms = 0.f;
     HIP_TRY(hipEventElapsedTime(&ms, t.ev[2 * i], t.ev[2 * i + 1]));
-    const int k = (t.kind[i] >= 0 && t.kind[i] < FGRPO_NUM_PHASES) ? t.kind[i] : FGRPO_NUM_PHASES - 1;
+    const int k = (t.kind[i] >= 0 && t.kind[i] < FGRPO_NUM_PHASES) ? t.kind[i] : kPhaseOther;
     ms_by_phase[k] += ms;
     ++brackets_by_phase[k];
   }
@@ -1203,6 +1268,215 @@ int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, co
   hipLaunchKernelGGL(grpo_loss_tokens_kernel, dim3(nblocks), dim3(kLossThreads), 0, st, p);
   HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(grpo_loss_finalize_kernel, dim3(std::min(nblocks, kFinalizeBlocks)), dim3(kLossThreads), 0, st, p, nblocks);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int fgrpo_loss_prepare(const int64_t* labels, const int32_t* cu, int nseq, int T, int agg_mode, double denom_override,
+                       float* tokw_out, int32_t* seg_cnt_out, double* pre_out, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!labels || !pre_out || T <= 0) return fail(FGRPO_ERR_BAD_ARG, "loss_prepare: bad argument");
+  if (agg_mode != FGRPO_AGG_TOKEN_MEAN && agg_mode != FGRPO_AGG_SAMPLE_MEAN)
+    return fail(FGRPO_ERR_BAD_ARG, "loss_prepare: agg_mode=%d", agg_mode);
+  const bool by_sample = agg_mode == FGRPO_AGG_SAMPLE_MEAN;
+  if (by_sample && (!cu || nseq <= 0 || !tokw_out || !seg_cnt_out))
+    return fail(FGRPO_ERR_BAD_ARG, "loss_prepare: sample_mean needs cu_seqlens, tokw_out and seg_cnt_out");
+  if (by_sample) {
+    // tokens outside every segment keep weight 0
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((T + 255) / 256), dim3(256), 0, st, tokw_out, 0.f, T);
+    HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(segment_valid_weight_kernel, dim3((nseq + 3) / 4), dim3(256), 0, st, (const long long*)labels, cu,
+                       nseq, T, seg_cnt_out, tokw_out);
+    HIP_TRY(hipGetLastError());
+  }
+  hipLaunchKernelGGL(grpo_loss_prepare_kernel, dim3(1), dim3(1024), 0, st, (const long long*)labels, T,
+                     by_sample ? (const int*)seg_cnt_out : nullptr, by_sample ? nseq : 0, agg_mode, denom_override, pre_out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+namespace {
+// Token chunk of the chunked step: the caller's bound rounded to whole 256-token tiles, then the tokens dealt evenly
+// over the chunks that bound needs (a last chunk of a few hundred tokens would pay whole passes over the dW sum).
+int fused_chunk_tokens(int T, int chunk_tokens) {
+  long long c = chunk_tokens > 0 ? chunk_tokens : 8192;
+  c = c / 256 * 256;
+  if (c < 256) c = 256;
+  if (c >= T) return (int)round_up(T, 256);
+  const long long n = (T + c - 1) / c;
+  return (int)round_up((T + n - 1) / n, 256);
+}
+
+struct ChunkedPlan {
+  int chunk, nchunks;
+  void* keep;
+  size_t keep_bytes;
+  void* fwd_ws;
+  size_t fwd_bytes;
+  void* bwd_ws;
+  size_t bwd_bytes;
+  float* dw_acc;
+  float* db_acc;
+  double* partial;
+  size_t bytes;
+};
+void plan_chunked(const Tuning& tn, ChunkedPlan& pl, void* ws, int T, int H, int V, int chunk_tokens, bool has_bias,
+                  bool want_dh, bool want_dw, bool want_db) {
+  pl.chunk = fused_chunk_tokens(T, chunk_tokens);
+  pl.nchunks = (T + pl.chunk - 1) / pl.chunk;
+  const int last = T - (pl.nchunks - 1) * pl.chunk;
+  pl.keep_bytes = keep_bytes(pl.chunk < T ? pl.chunk : T, V);
+  pl.fwd_bytes = pl.bwd_bytes = 0;
+  for (int cnt : {pl.chunk < T ? pl.chunk : T, last}) {
+    Tuning tf = tn;
+    tf.fwd_variant = 8;
+    FwdPlan fp;
+    plan_fwd(tf, fp, nullptr, cnt, H, V, FGRPO_BF16, has_bias);
+    if (fp.bytes > pl.fwd_bytes) pl.fwd_bytes = fp.bytes;
+    KeptBwdPlan bp;
+    plan_kept_bwd(tn, bp, nullptr, cnt, H, V, has_bias, want_dh, want_dw);
+    if (bp.bytes > pl.bwd_bytes) pl.bwd_bytes = bp.bytes;
+  }
+  Carver cv(ws);
+  pl.keep = cv.take<char>(pl.keep_bytes);
+  pl.fwd_ws = cv.take<char>(pl.fwd_bytes);
+  pl.bwd_ws = cv.take<char>(pl.bwd_bytes);
+  pl.dw_acc = (want_dw && pl.nchunks > 1) ? cv.take<float>((size_t)V * H) : nullptr;
+  pl.db_acc = (want_db && pl.nchunks > 1) ? cv.take<float>((size_t)V) : nullptr;
+  pl.partial = cv.take<double>(2 * (size_t)((T + kLossThreads - 1) / kLossThreads));
+  pl.bytes = cv.total();
+}
+}  // namespace
+
+namespace {
+// every chunk - the full ones and the shorter last one - must be a problem the kept-numerators pair handles
+bool chunked_supported(const Tuning& tn, int T, int H, int V, int dtype, int chunk_tokens) {
+  if (T <= 0 || H <= 0 || V <= 0) return false;
+  const int chunk = fused_chunk_tokens(T, chunk_tokens);
+  const int nchunks = (T + chunk - 1) / chunk;
+  const int last = T - (nchunks - 1) * chunk;
+  return keep_supported(tn, chunk < T ? chunk : T, H, V, dtype) && keep_supported(tn, last, H, V, dtype);
+}
+}  // namespace
+
+int fgrpo_grpo_step_chunked_supported(int T, int H, int V, int dtype, int chunk_tokens) {
+  return chunked_supported(g_tune, T, H, V, dtype, chunk_tokens) ? 1 : 0;
+}
+
+int fgrpo_grpo_step_chunk_tokens(int T, int chunk_tokens) {
+  if (T <= 0) return fail(FGRPO_ERR_BAD_ARG, "grpo_step_chunk_tokens: T=%d", T);
+  return fused_chunk_tokens(T, chunk_tokens);
+}
+
+size_t fgrpo_grpo_step_chunked_workspace(int T, int H, int V, int dtype, int chunk_tokens) {
+  if (T <= 0 || H <= 0 || V <= 0 || dtype != FGRPO_BF16) return 0;
+  ChunkedPlan pl;
+  plan_chunked(g_tune, pl, nullptr, T, H, V, chunk_tokens, true, true, true, true);
+  return pl.bytes;
+}
+
+int fgrpo_grpo_step_chunked(const void* hidden, const void* weight, const void* bias, const int64_t* labels,
+                            const float* old_lp, const float* ref_lp, const float* adv, const float* tokw,
+                            const double* pre, float inv_temp, int T, int H, int V, int dtype, float clip_low,
+                            float clip_high, float clip_c, float kl_beta, int chunk_tokens, float* lp_out, float* ent_out,
+                            float* lse_out, float* loss_out, float* g_out, float* log_ratio, float* clip1,
+                            float* unclipped, float* clipped, float* scal_out, void* dH_out, void* dW_out,
+                            void* dbias_out, void* ws, size_t ws_bytes, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (!hidden || !weight || !labels || !adv || !pre || !lp_out || !lse_out || !loss_out || !g_out)
+    return fail(FGRPO_ERR_BAD_ARG, "grpo_step_chunked: null argument");
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "grpo_step_chunked: T=%d H=%d V=%d", T, H, V);
+  if (!(inv_temp > 0.f)) return fail(FGRPO_ERR_BAD_ARG, "grpo_step_chunked: inv_temperature must be positive");
+  if (dbias_out && !bias) return fail(FGRPO_ERR_BAD_ARG, "grpo_step_chunked: dbias requested without a bias");
+  if (!aligned16(hidden) || !aligned16(weight)) return fail(FGRPO_ERR_ALIGN, "grpo_step_chunked: hidden/weight must be 16-byte aligned");
+  const Tuning tn = g_tune;   // one reading of the tuning state per call
+  ChunkedPlan pl;
+  plan_chunked(tn, pl, ws, T, H, V, chunk_tokens, bias != nullptr, dH_out != nullptr, dW_out != nullptr, dbias_out != nullptr);
+  if (!chunked_supported(tn, T, H, V, dtype, chunk_tokens))
+    return fail(FGRPO_ERR_UNSUPPORTED, "grpo_step_chunked: every chunk needs bf16, H %% 64 == 0, V/256 x H/256 tiles for half the CUs and V/256 x tokens/256 tiles for half the CUs (T=%d H=%d V=%d, chunks of %d)", T, H, V, pl.chunk);
+  if (!ws || !aligned16(ws) || ws_bytes < pl.bytes)
+    return fail(FGRPO_ERR_WORKSPACE, "grpo_step_chunked: workspace null, misaligned or smaller than %zu bytes", pl.bytes);
+
+  LossParams lp;
+  memset(&lp, 0, sizeof(lp));
+  lp.clip_low = clip_low;
+  lp.clip_high = clip_high;
+  lp.clip_c = clip_c;
+  lp.kl_beta = kl_beta;
+  lp.pre = pre;
+  lp.loss = loss_out;
+  lp.scal = scal_out;
+
+  const size_t esz = sizeof(bf16_t);
+  for (int ci = 0; ci < pl.nchunks; ++ci) {
+    const int t0 = ci * pl.chunk;
+    const int cnt = (T - t0) < pl.chunk ? (T - t0) : pl.chunk;
+    const char* h_c = (const char*)hidden + (size_t)t0 * H * esz;
+    int rc;
+    {
+      PhaseScope ph(kPhaseFwd, st);
+      rc = logprob_fwd_impl(h_c, weight, bias, labels + t0, inv_temp, cnt, H, V, dtype, lp_out + t0,
+                            ent_out ? ent_out + t0 : nullptr, lse_out + t0, pl.fwd_ws, pl.fwd_bytes, stream, pl.keep, &tn);
+    }
+    if (rc) return rc;
+    {
+      // the objective on this chunk's tokens: the normaliser is known (pre), so g is final as it is written
+      PhaseScope ph(kPhaseOther, st);
+      LossParams q = lp;
+      q.lp = lp_out + t0;
+      q.old_lp = old_lp ? old_lp + t0 : nullptr;
+      q.ref_lp = ref_lp ? ref_lp + t0 : nullptr;
+      q.adv = adv + t0;
+      q.labels = (const long long*)labels + t0;
+      q.tokw = tokw ? tokw + t0 : nullptr;
+      q.T = cnt;
+      q.g = g_out + t0;
+      q.log_ratio = log_ratio ? log_ratio + t0 : nullptr;
+      q.clip1 = clip1 ? clip1 + t0 : nullptr;
+      q.unclipped = unclipped ? unclipped + t0 : nullptr;
+      q.clipped = clipped ? clipped + t0 : nullptr;
+      q.partial = pl.partial + 2 * (size_t)(t0 / kLossThreads);     // chunks start on whole blocks of the token kernel
+      hipLaunchKernelGGL(grpo_loss_tokens_kernel, dim3((cnt + kLossThreads - 1) / kLossThreads), dim3(kLossThreads), 0, st, q);
+      HIP_TRY(hipGetLastError());
+    }
+    if (dH_out || dW_out || dbias_out) {
+      const bool first = ci == 0, last = ci == pl.nchunks - 1;
+      KeptBwdSums sums;
+      if (dW_out && pl.nchunks > 1) {
+        sums.dw_in = first ? nullptr : pl.dw_acc;
+        sums.dw_out_f32 = last ? nullptr : pl.dw_acc;
+      }
+      if (dbias_out && pl.nchunks > 1) {
+        sums.db_in = first ? nullptr : pl.db_acc;
+        sums.db_out_f32 = last ? nullptr : pl.db_acc;
+      }
+      rc = kept_bwd_impl(tn, h_c, weight, bias, labels + t0, lse_out + t0, g_out + t0, nullptr, inv_temp, cnt, H, V,
+                         pl.keep, dH_out ? (char*)dH_out + (size_t)t0 * H * esz : nullptr, dW_out, dbias_out, sums,
+                         pl.bwd_ws, pl.bwd_bytes, st);
+      if (rc) return rc;
+    }
+  }
+  {
+    PhaseScope ph(kPhaseOther, st);
+    const int nblocks = (T + kLossThreads - 1) / kLossThreads;
+    lp.T = T;
+    lp.partial = pl.partial;
+    hipLaunchKernelGGL(grpo_loss_finalize_kernel, dim3(1), dim3(kLossThreads), 0, st, lp, nblocks);
+    HIP_TRY(hipGetLastError());
+  }
+  return 0;
+}
+
+int fgrpo_scale_inplace(void* x, long long n, int dtype, const float* scale_dev, void* stream) {
+  if (!x || !scale_dev || n < 0) return fail(FGRPO_ERR_BAD_ARG, "scale_inplace: bad argument");
+  if (dtype != FGRPO_BF16 && dtype != FGRPO_F32) return fail(FGRPO_ERR_BAD_ARG, "scale_inplace: dtype=%d", dtype);
+  if (!aligned16(x)) return fail(FGRPO_ERR_ALIGN, "scale_inplace: the array must be 16-byte aligned");
+  if (n == 0) return 0;
+  const long long nv = n / (dtype == FGRPO_F32 ? 4 : 8);
+  long long nb = (nv + 255) / 256;
+  nb = nb < 1 ? 1 : (nb > 4096 ? 4096 : nb);
+  hipLaunchKernelGGL(scale_inplace_kernel, dim3((unsigned)nb), dim3(256), 0, (hipStream_t)stream, x, n,
+                     dtype == FGRPO_F32, scale_dev);
   HIP_TRY(hipGetLastError());
   return 0;
 }

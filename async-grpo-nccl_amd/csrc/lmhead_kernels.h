@@ -362,6 +362,7 @@ struct DsParams {
   bf16_t* vt_hi;             // [tiles_v*BM][ld_vt]
   bf16_t* vt_lo;
   long long ld_vt;
+  const int* gate;           // optional device flag: the launch does nothing unless *gate != 0 (null: always runs)
 };
 
 template <class C, bool SPLIT>
@@ -370,6 +371,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lmhead_ds_kernel(const DsParams
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
   const int V = p.g.M, T = p.g.N;
+  if (p.gate != nullptr && *p.gate == 0) return;     // work-group uniform: every wavefront leaves before any barrier
 
   // work-group -> (token tile, share of the panel's vocabulary tiles), rastered like the forward kernel: the
   // per-token inputs are read once and the next tile's first K slice is requested under this tile's epilogue

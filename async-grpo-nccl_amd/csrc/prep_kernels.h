@@ -229,18 +229,25 @@ struct KeepPrepParams {
   const bf16_t* hidden;      // [T][H]
   int T, H, V;
   float* row_scale;          // [T] out: a_t
+  // The forward's overflow flag, read here on the device (null = not consulted).  When it is set the kept values
+  // are not to be trusted: the caller's next launch (lmhead_ds_kernel gated on the same flag) overwrites the whole
+  // buffer with dLogits recomputed from the operands, and this kernel leaves the buffer alone and writes the row
+  // factor as 1 for tokens with a gradient, 0 for the others - the gradient products that follow are the same
+  // launches either way.
+  const int* gate;
 };
 
 __global__ __launch_bounds__(256) void keep_backward_prep_kernel(const KeepPrepParams p) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (t >= p.T) return;
   const long long lab = p.labels[t];
+  const bool recompute = p.gate != nullptr && *p.gate != 0;
   float a = 0.f;
   if (lab >= 0 && lab < p.V) {
     const float c = p.gtok[t] * (p.gout ? *p.gout : 1.f) * p.inv_temp;
     const float d2 = p.ref2[t] - p.lse[t] * kLog2e;        // log2 s_t
-    a = -c * fast_exp2(d2);
-    if (lane == 0) {
+    a = recompute ? (c != 0.f ? 1.f : 0.f) : -c * fast_exp2(d2);
+    if (lane == 0 && !recompute) {
       // p_y - 1 from the fp32 quantities: log p_y = x_y/temperature - lse
       const float pm1 = expm1f(p.xy[t] - p.lse[t]);
       p.e[(lab >> 8) * p.blk + (long long)t * 256 + (lab & 255)] = f32_to_bf16_rn(pm1 * fast_exp2(-d2));
@@ -312,8 +319,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* part, i
 
 // dbias from the kept numerators: out[v] = sum_t a_t * E'[t][v].  One block owns 64 columns; its four row groups
 // are combined in a fixed order.
+// acc_in (fp32 [V] or null) is added first; the sum goes to acc_out (fp32) and / or out_bf16, whichever is given:
+// a caller that walks the tokens in chunks carries the sum in fp32 and takes bf16 from the last chunk.
 __global__ void keep_col_sum_kernel(const bf16_t* e, long long blk, const float* row_scale, int T, int V,
-                                    bf16_t* out_bf16) {
+                                    const float* acc_in, float* acc_out, bf16_t* out_bf16) {
   __shared__ float red[4][64];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int c = blockIdx.x * 64 + tx;
@@ -324,7 +333,41 @@ __global__ void keep_col_sum_kernel(const bf16_t* e, long long blk, const float*
   }
   red[ty][tx] = s;
   __syncthreads();
-  if (ty == 0 && c < V) out_bf16[c] = f32_to_bf16_rn((red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]));
+  if (ty == 0 && c < V) {
+    float r = (red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]);
+    if (acc_in) r += acc_in[c];
+    if (acc_out) acc_out[c] = r;
+    if (out_bf16) out_bf16[c] = f32_to_bf16_rn(r);
+  }
+}
+
+// x[i] *= *scale for a bf16 or fp32 array, 16 bytes per thread and step (n: elements; the base is 16-byte aligned).
+// A scale of exactly 1 leaves the array untouched: every work-group returns after reading the scalar.
+__global__ __launch_bounds__(256) void scale_inplace_kernel(void* x, long long n, int is_f32, const float* scale) {
+  const float s = *scale;
+  if (s == 1.f) return;
+  const long long per = is_f32 ? 4 : 8;
+  const long long nv = n / per;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nv; i += (long long)gridDim.x * 256) {
+    if (is_f32) {
+      float4 v = ((float4*)x)[i];
+      v.x *= s, v.y *= s, v.z *= s, v.w *= s;
+      ((float4*)x)[i] = v;
+    } else {
+      u32x4_t v = ((u32x4_t*)x)[i];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        v[e] = pack_bf16x2(s * __uint_as_float(v[e] << 16), s * __uint_as_float(v[e] & 0xffff0000u));
+      ((u32x4_t*)x)[i] = v;
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    for (long long i = nv * per; i < n; ++i) {
+      if (is_f32)
+        ((float*)x)[i] *= s;
+      else
+        ((bf16_t*)x)[i] = f32_to_bf16_rn(s * bf16_to_f32(((bf16_t*)x)[i]));
+    }
 }
 
 // Which parts of the token axis carry a gradient at all (row factor a_t != 0): zero-advantage samples and ignored

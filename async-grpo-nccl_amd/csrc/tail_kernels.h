@@ -235,6 +235,11 @@ struct LossParams {
   double* partial;           // [2 * nblocks] : sum, count
   float* loss;               // scalar
   float* scal;               // [4] : normaliser, valid count, nonempty segments, raw sum
+  // Normaliser known before the tokens are walked (grpo_loss_prepare_kernel): {denominator, valid tokens, non-empty
+  // segments, 1 / denominator rounded to fp32}.  With it the token kernel writes g already normalised - the same
+  // two fp32 products the finalize kernel would have made - so that a caller may walk the tokens in chunks and use
+  // each chunk's g before the last chunk has been seen; the finalize kernel then only forms the loss.
+  const double* pre;
 };
 
 constexpr int kLossThreads = 256;
@@ -267,7 +272,9 @@ __global__ __launch_bounds__(kLossThreads) void grpo_loss_tokens_kernel(const Lo
       dtok += p.kl_beta * (1.0f - ed);
     }
     const float w = valid ? (p.tokw ? p.tokw[t] : 1.0f) : 0.f;
-    p.g[t] = w * dtok;
+    float gv = w * dtok;
+    if (p.pre) gv *= (float)p.pre[3];
+    p.g[t] = gv;
     if (p.log_ratio) p.log_ratio[t] = lr;
     if (p.clip1) p.clip1[t] = c1;
     if (p.unclipped) p.unclipped[t] = l1;
@@ -330,17 +337,58 @@ __global__ __launch_bounds__(kLossThreads) void grpo_loss_finalize_kernel(const 
   double den = (p.agg_mode == 0) ? tot[1] : tot[2];
   if (p.denom_override > 0.0) den = p.denom_override;
   if (den < 1.0) den = 1.0;
+  double valid_n = tot[1], nonempty = tot[2];
+  if (p.pre) {                       // the same numbers, formed from the labels before the tokens were walked
+    den = p.pre[0];
+    valid_n = p.pre[1];
+    nonempty = p.pre[2];
+  }
   const float norm = (float)(1.0 / den);
-  for (long long t = (long long)blockIdx.x * kLossThreads + threadIdx.x; t < p.T; t += (long long)gridDim.x * kLossThreads)
-    p.g[t] *= norm;
+  if (!p.pre)
+    for (long long t = (long long)blockIdx.x * kLossThreads + threadIdx.x; t < p.T; t += (long long)gridDim.x * kLossThreads)
+      p.g[t] *= norm;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *p.loss = (float)(tot[0] / den);
     if (p.scal) {
       p.scal[0] = norm;
-      p.scal[1] = (float)tot[1];
-      p.scal[2] = (float)tot[2];
+      p.scal[1] = (float)valid_n;
+      p.scal[2] = (float)nonempty;
       p.scal[3] = (float)tot[0];
     }
+  }
+}
+
+// The normaliser of the objective depends on the labels and the segments only: valid tokens (token mean), segments
+// with at least one valid token (sample mean), or the caller's override.  One work-group counts them before any
+// logprob exists; pre = {denominator, valid tokens, non-empty segments, (double)(float)(1 / denominator)}.
+__global__ __launch_bounds__(1024) void grpo_loss_prepare_kernel(const long long* labels, int T, const int* seg_cnt,
+                                                                 int nseq, int agg_mode, double denom_override,
+                                                                 double* pre) {
+  __shared__ int sh[2][16];
+  int c = 0, ne = 0;
+  for (int t = threadIdx.x; t < T; t += 1024) c += (labels[t] != -100);
+  if (seg_cnt)
+    for (int i = threadIdx.x; i < nseq; i += 1024) ne += (seg_cnt[i] > 0);
+  c = wave_sum_i(c);
+  ne = wave_sum_i(ne);
+  if ((threadIdx.x & 63) == 0) {
+    sh[0][threadIdx.x >> 6] = c;
+    sh[1][threadIdx.x >> 6] = ne;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    long long cs = 0, ns = 0;
+    for (int w = 0; w < 16; ++w) {
+      cs += sh[0][w];
+      ns += sh[1][w];
+    }
+    double den = (agg_mode == 0) ? (double)cs : (double)ns;
+    if (denom_override > 0.0) den = denom_override;
+    if (den < 1.0) den = 1.0;
+    pre[0] = den;
+    pre[1] = (double)cs;
+    pre[2] = (double)ns;
+    pre[3] = (double)(float)(1.0 / den);
   }
 }
 

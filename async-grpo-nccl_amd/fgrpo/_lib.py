@@ -14,7 +14,7 @@ ERR = {-1: "bad argument", -2: "unsupported", -3: "workspace", -4: "HIP error", 
 BF16, F32 = 0, 1
 AGG_TOKEN_MEAN, AGG_SAMPLE_MEAN = 0, 1
 NUM_STATS = 16
-NUM_PHASES = 4           # FGRPO_NUM_PHASES
+NUM_PHASES = 5           # FGRPO_NUM_PHASES
 STATIC_SCRATCH_BYTES = 8 << 20   # FGRPO_STATIC_SCRATCH_BYTES
 METRIC_BLOCKS = 128      # work-groups of the diagnostics' first stage (FGRPO_METRIC_BLOCKS)
 
@@ -44,6 +44,13 @@ SIGNATURES = {
     "fgrpo_loss_fwd_workspace": (_sz, [_i, _i]),
     "fgrpo_loss_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _f, _f, _i, _d,
                             _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgrpo_loss_prepare": (_i, [_vp, _vp, _i, _i, _i, _d, _vp, _vp, _vp, _vp]),
+    "fgrpo_grpo_step_chunk_tokens": (_i, [_i, _i]),
+    "fgrpo_grpo_step_chunked_supported": (_i, [_i, _i, _i, _i, _i]),
+    "fgrpo_grpo_step_chunked_workspace": (_sz, [_i, _i, _i, _i, _i]),
+    "fgrpo_grpo_step_chunked": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _f, _f, _f, _f, _i,
+                                     _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgrpo_scale_inplace": (_i, [_vp, _ll, _i, _vp, _vp]),
     "fgrpo_metrics": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _vp, _vp]),
     "fgrpo_group_advantages": (_i, [_vp, _i, _vp, _i, _i, _d, _vp, _vp, _vp]),
     "fgrpo_segment_broadcast": (_i, [_vp, _i, _vp, _i, _i, _vp, _vp]),

@@ -135,19 +135,27 @@ def build(verbose: bool = True, only=None) -> str:
     missing = [o for o in objs if not os.path.exists(o)]
     if missing:
         raise RuntimeError(f"objects missing (build everything first): {missing}")
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("link failed:\n" + res.stdout)
+    # The guard decides before anything is linked: a build it refuses leaves no library behind (a stale one from an
+    # earlier build is removed too), so nothing can load the kernels it exists to block.
     usage = {k: v for src in SOURCES for k, v in by_source.get(src, {}).items()}
     problems = check_resource_usage(usage)
     json.dump({"sources": by_source, "kernels": usage, "problems": problems}, open(USAGE_PATH, "w"), indent=1,
               sort_keys=True)
     if problems:
-        raise RuntimeError("kernel resource guard failed:\n  " + "\n  ".join(problems))
+        if os.path.exists(LIB_PATH):
+            os.remove(LIB_PATH)
+        raise RuntimeError("kernel resource guard failed (no library written):\n  " + "\n  ".join(problems))
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    tmp = LIB_PATH + ".linking"
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        raise RuntimeError("link failed:\n" + res.stdout)
+    os.replace(tmp, LIB_PATH)
     return LIB_PATH
 
 

@@ -156,14 +156,15 @@ def phase_timing_begin() -> None:
 
 
 def phase_timing_end():
-    """Stop and read: ({phase: summed ms}, {phase: brackets}, dropped) for the phases dlogits / dh / dw / other."""
+    """Stop and read: ({phase: summed ms}, {phase: brackets}, dropped) for the phases dlogits / dh / dw / other / fwd
+    (fwd: the forward launches of the chunked step; the stand-alone forward is not bracketed by the library)."""
     import ctypes
     ms = (ctypes.c_float * _lib.NUM_PHASES)()
     cnt = (ctypes.c_int * _lib.NUM_PHASES)()
     rc = _lib.load().fgrpo_phase_timing_end(ctypes.cast(ms, ctypes.c_void_p), ctypes.cast(cnt, ctypes.c_void_p))
     if rc < 0:
         _lib.check(rc, "phase_timing_end")
-    names = ("dlogits", "dh", "dw", "other")
+    names = ("dlogits", "dh", "dw", "other", "fwd")
     return {n: float(ms[i]) for i, n in enumerate(names)}, {n: int(cnt[i]) for i, n in enumerate(names)}, int(rc)
 
 
@@ -208,8 +209,8 @@ def lmhead_bwd(hidden, weight, bias, labels_shifted, lse, g, gout: Optional[torc
 
 def keep_overflowed(kept: torch.Tensor, T: int, V: int) -> bool:
     """True when the forward flagged that the kept values may have overflowed (a logit more than 123 log-probability
-    units above both the target logit and the largest logit of the first 512 vocabulary rows): the caller must then
-    take the recomputing backward.  Waits for the current stream."""
+    units above both the target logit and the largest logit of the first 512 vocabulary rows).  Waits for the current
+    stream.  A query for tests and reports: the backward reads the flag on the device and recomputes by itself."""
     with torch.cuda.device(kept.device):
         rc = _lib.load().fgrpo_keep_overflowed(_ptr(kept), int(T), int(V), _stream())
     if rc < 0:
@@ -221,7 +222,8 @@ def lmhead_bwd_kept(hidden, weight, bias, labels_shifted, lse, g, gout: Optional
                     kept: torch.Tensor, need_dh: bool, need_dw: bool, need_db: bool):
     """The backward on the soft-max numerators the forward kept (``lmhead_logprob_fwd(..., keep=True)``): one
     element per row of ``kept`` is patched in place, then dH / dW / dbias come from one GEMM each reading the buffer
-    as it lies.  The caller has checked ``keep_overflowed(kept, T, V)``."""
+    as it lies.  When the forward raised the buffer's overflow flag, the library (reading it on the device)
+    first overwrites the buffer with dLogits recomputed from the operands: same launches, no host synchronisation."""
     dev = _require_cuda(hidden, weight, labels_shifted, lse, g, kept)
     lib = _lib.load()
     T, H = hidden.shape
@@ -556,27 +558,61 @@ def _valid_rows(labels_shifted: torch.Tensor, compact):
     return mask.nonzero(as_tuple=False).squeeze(1)
 
 
-# Keeping the logits for the backward (as the reference's autograd does) instead of recomputing them: "auto" keeps
-# them when the kernels support the shape and the buffer takes at most this share of the memory still obtainable
-# (free on the device + cached by torch's allocator); True insists (raises when unsupported); False recomputes.
+# How a training step gets its gradients (``keep_logits`` of the calls below; None = the module default
+# ``KEEP_LOGITS``).  The choice depends on shapes and on these settings only - never on what else happens to be
+# resident on the device - so the same inputs give bit-identical gradients whatever the allocator's state.
+#   "chunked"   the whole step inside the forward call, token chunk by token chunk (``grpo_step_chunked``): 6 T H V of
+#               matrix work with one chunk of soft-max numerators as the transient; what the reference's chunk loop
+#               is for (grpo_loss.py:280-316).  Needs the objective fused with the projection (``fused_grpo_loss``).
+#   "auto"      "chunked" where the kernels support the shape, else "recompute"; for ``lmhead_logprob`` alone (whose
+#               per-token gradient only arrives with backward()): the whole-batch kept buffer when it takes at most
+#               ``KEEP_WHOLE_MAX_BYTES``, else "recompute".
+#   True / "whole"   soft-max numerators of the whole batch kept for backward() ([T x V] bf16; raises when unsupported).
+#   False / "recompute"   logits recomputed in backward(), one vocabulary panel of dLogits at a time (8 T H V).
 KEEP_LOGITS = "auto"
-KEEP_MAX_MEMORY_FRACTION = 0.5
+KEEP_WHOLE_MAX_BYTES = 4 << 30
+# Token chunk of the chunked step: twice the caller's ``loss_chunksize`` (the reference holds a chunk's logits in bf16
+# plus fp32 temporaries of the same shape; the one buffer here is 2 * loss_chunksize * V bf16), else this many tokens;
+# never more than ``CHUNK_MAX_BYTES`` of kept numerators.
+CHUNK_TOKENS = 8192
+CHUNK_MAX_BYTES = 8 << 30
 
 
-def _want_keep(T: int, H: int, V: int, dtype, dev, needs_grad: bool, keep_logits=None) -> bool:
+def _grad_mode(keep_logits):
     mode = KEEP_LOGITS if keep_logits is None else keep_logits
-    if not needs_grad or mode is False or T == 0:
+    if mode is True or mode == "whole":
+        return "whole"
+    if mode is False or mode == "recompute":
+        return "recompute"
+    if mode in ("auto", "chunked"):
+        return mode
+    raise ValueError(f"fgrpo: keep_logits={mode!r} (expected 'auto', 'chunked', 'whole' / True, 'recompute' / False)")
+
+
+def chunk_bound_for(V: int, loss_chunksize: Optional[int] = None) -> int:
+    """Upper bound on the token chunk of the chunked step (a multiple of 256), from the settings above."""
+    bound = 2 * int(loss_chunksize) if (loss_chunksize is not None and loss_chunksize > 0) else CHUNK_TOKENS
+    by_bytes = CHUNK_MAX_BYTES // (2 * ((V + 255) // 256 * 256))
+    return max(256, min(bound, by_bytes) // 256 * 256)
+
+
+def chunk_tokens_for(T: int, V: int, loss_chunksize: Optional[int] = None) -> int:
+    """Token chunk the chunked step uses for a packed batch of T tokens: the bound, then the tokens dealt evenly over
+    the chunks that bound needs (whole 256-token tiles)."""
+    return int(_lib.load().fgrpo_grpo_step_chunk_tokens(int(T), chunk_bound_for(V, loss_chunksize)))
+
+
+def _want_keep(T: int, H: int, V: int, dtype, needs_grad: bool, keep_logits=None) -> bool:
+    """Whole-batch kept numerators for a forward whose backward comes later (see ``KEEP_LOGITS``)."""
+    mode = _grad_mode(keep_logits)
+    if not needs_grad or mode == "recompute" or T == 0:
         return False
     ok = keep_supported(T, H, V, dtype)
-    if mode is True:
+    if mode == "whole":
         if not ok:
             raise RuntimeError(f"fgrpo: keep_logits=True but T={T} H={H} V={V} {dtype} is not supported")
         return True
-    if not ok:
-        return False
-    free, _total = torch.cuda.mem_get_info(dev)
-    obtainable = free + torch.cuda.memory_reserved(dev) - torch.cuda.memory_allocated(dev)
-    return logits_keep_bytes(T, V) <= KEEP_MAX_MEMORY_FRACTION * obtainable
+    return ok and mode == "auto" and logits_keep_bytes(T, V) <= KEEP_WHOLE_MAX_BYTES
 
 
 def _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx, needs_grad=False, keep_logits=None):
@@ -587,8 +623,7 @@ def _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx, ne
         y = labels_shifted.reshape(-1).index_select(0, idx)
     else:
         y = labels_shifted
-    keep = _want_keep(hidden.shape[0], hidden.shape[1], weight.shape[0], weight.dtype, hidden.device, needs_grad,
-                      keep_logits)
+    keep = _want_keep(hidden.shape[0], hidden.shape[1], weight.shape[0], weight.dtype, needs_grad, keep_logits)
     res = lmhead_logprob_fwd(hidden, weight, bias, y, temperature, keep=keep)
     lp, ent, lse = res[:3]
     kept = res[3] if keep else None
@@ -613,9 +648,8 @@ def panel_elems_bound(T: int, V: int, loss_chunksize: Optional[int]) -> int:
 def _bwd_rows(h_used, weight, bias, y_used, lse, g_full, gout, temperature, need, panel_hint, idx, hidden_shape,
               kept=None):
     g_used = g_full if idx is None else g_full.reshape(-1).index_select(0, idx)
-    if kept is not None and keep_overflowed(kept, h_used.shape[0], weight.shape[0]):
-        kept = None                                # out of the kept values' range: recompute (exact for any input)
     if kept is not None:
+        # an out-of-range batch is recomputed by the library itself (flag read on the device): no host wait here
         dH, dW, db = lmhead_bwd_kept(h_used, weight, bias, y_used, lse, g_used, gout, temperature, kept, need[0],
                                      need[1], need[2])
     else:
@@ -626,6 +660,93 @@ def _bwd_rows(h_used, weight, bias, y_used, lse, g_full, gout, temperature, need
     return dH, dW, db
 
 
+def loss_prepare(labels_shifted, cu_seqlens=None, loss_agg_mode="token_mean", denom_override: float = 0.0):
+    """The objective's normalisers from the labels and segments alone: (tokw [T] fp32 | None, pre [4] float64) -
+    see ``fgrpo_loss_prepare``."""
+    dev = _require_cuda(labels_shifted)
+    lib = _lib.load()
+    y = labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    T = y.numel()
+    pre = torch.empty(4, dtype=torch.float64, device=dev)
+    if loss_agg_mode == "token_mean":
+        agg, tokw, segc, cu, nseq = _lib.AGG_TOKEN_MEAN, None, None, None, 0
+    elif loss_agg_mode == "sample_mean":
+        if cu_seqlens is None:
+            raise RuntimeError("fgrpo: loss_agg_mode='sample_mean' needs cu_seqlens")
+        agg = _lib.AGG_SAMPLE_MEAN
+        cu = cu_seqlens.to(device=dev, dtype=torch.int32).contiguous()
+        nseq = cu.numel() - 1
+        tokw = torch.empty(T, dtype=torch.float32, device=dev)
+        segc = torch.empty(max(nseq, 1), dtype=torch.int32, device=dev)
+    else:
+        raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_loss_prepare(_ptr(y), _ptr(cu), nseq, T, agg, float(denom_override), _ptr(tokw), _ptr(segc),
+                                    _ptr(pre), _stream())
+    _lib.check(rc, "loss_prepare")
+    return tokw, pre
+
+
+def chunked_supported(T: int, H: int, V: int, dtype: torch.dtype, chunk_tokens: int) -> bool:
+    """Whether the chunked step handles this problem under the chunk bound ``chunk_tokens``: the kept-numerators
+    kernels must accept every chunk, the shorter last one included."""
+    if dtype != torch.bfloat16 or T <= 0:
+        return False
+    return bool(_lib.load().fgrpo_grpo_step_chunked_supported(int(T), int(H), int(V), _lib.BF16, int(chunk_tokens)))
+
+
+def grpo_step_chunked(hidden, weight, bias, labels_shifted, old_lp, ref_lp, adv, tokw, pre, temperature, clip_low,
+                      clip_high, clip_ratio_c, kl_beta, chunk_tokens, need_dh=True, need_dw=True, need_db=False,
+                      want_diag=True):
+    """Projection, logprob, objective and gradients of one packed batch, token chunk by token chunk, in one library
+    call (``fgrpo_grpo_step_chunked``): hidden [T,H], weight [V,H] bf16; per-token inputs fp32 [T]; ``tokw`` / ``pre``
+    from ``loss_prepare``.  Returns (loss, lp, ent, lse, g, log_ratio, clip1, unclipped, clipped, scal, dH, dW, db):
+    the gradients are those of the loss itself (upstream gradient 1)."""
+    dev = _require_cuda(hidden, weight, bias, labels_shifted, adv, pre)
+    lib = _lib.load()
+    T, H = hidden.shape
+    V = weight.shape[0]
+    code = _code(weight.dtype)
+    if hidden.dtype != weight.dtype:
+        raise RuntimeError("fgrpo: hidden and weight must share a dtype")
+    hidden, weight = _aligned(hidden), _aligned(weight)
+    if bias is not None:
+        bias = bias.detach().to(weight.dtype).contiguous()
+    y = labels_shifted.reshape(-1).to(torch.int64).contiguous()
+    old_lp, ref_lp, adv, tokw = _f32(old_lp, T, "old_logprobs"), _f32(ref_lp, T, "ref_logprobs"), \
+        _f32(adv, T, "advantages"), _f32(tokw, T, "token weights")
+    mk = lambda: torch.empty(T, dtype=torch.float32, device=dev)
+    lp, ent, lse, g = mk(), mk(), mk(), mk()
+    lr, c1, l1, l2 = (mk(), mk(), mk(), mk()) if want_diag else (None, None, None, None)
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    scal = torch.empty(4, dtype=torch.float32, device=dev)
+    dH = torch.empty_like(hidden) if need_dh else None
+    dW = torch.empty_like(weight) if need_dw else None
+    db = torch.empty(V, dtype=weight.dtype, device=dev) if (need_db and bias is not None) else None
+    ws = _ws(lib.fgrpo_grpo_step_chunked_workspace(T, H, V, code, int(chunk_tokens)), dev)
+    clamp = lambda x: float(max(min(float(x), 3.0e38), -3.0e38))
+    with torch.cuda.device(dev):
+        rc = lib.fgrpo_grpo_step_chunked(_ptr(hidden), _ptr(weight), _ptr(bias), _ptr(y), _ptr(old_lp), _ptr(ref_lp),
+                                         _ptr(adv), _ptr(tokw), _ptr(pre), 1.0 / float(temperature), T, H, V, code,
+                                         clamp(clip_low), clamp(clip_high), clamp(clip_ratio_c), clamp(kl_beta),
+                                         int(chunk_tokens), _ptr(lp), _ptr(ent), _ptr(lse), _ptr(loss), _ptr(g),
+                                         _ptr(lr), _ptr(c1), _ptr(l1), _ptr(l2), _ptr(scal), _ptr(dH), _ptr(dW), _ptr(db),
+                                         _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "grpo_step_chunked")
+    return loss, lp, ent, lse, g, lr, c1, l1, l2, scal, dH, dW, db
+
+
+def scale_inplace(x: Optional[torch.Tensor], scale_dev: torch.Tensor) -> None:
+    """x *= scale (a one-element fp32 device tensor) in place; exactly 1 leaves x untouched."""
+    if x is None or x.numel() == 0:
+        return
+    if not x.is_contiguous():
+        raise RuntimeError("fgrpo: scale_inplace needs a contiguous tensor")
+    with torch.cuda.device(x.device):
+        rc = _lib.load().fgrpo_scale_inplace(_ptr(x), x.numel(), _code(x.dtype), _ptr(scale_dev), _stream())
+    _lib.check(rc, "scale_inplace")
+
+
 class _LMHeadLogprob(torch.autograd.Function):
     """(hidden, weight, bias, labels_shifted) -> (lp, entropy); entropy carries no gradient."""
 
@@ -633,6 +754,8 @@ class _LMHeadLogprob(torch.autograd.Function):
     def forward(ctx, hidden, weight, bias, labels_shifted, temperature, panel_hint, compact, keep_logits=None):
         idx = _valid_rows(labels_shifted, compact)
         needs_grad = any(ctx.needs_input_grad[:3])
+        if _grad_mode(keep_logits) == "chunked":
+            keep_logits = "auto"        # the per-token gradient only arrives with backward(): nothing to chunk here
         lp, ent, lse, h_used, y_used, kept = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx,
                                                                needs_grad, keep_logits)
         ctx.save_for_backward(h_used, weight, bias if bias is not None else hidden.new_empty(0), y_used, lse,
@@ -664,34 +787,80 @@ class _FusedGRPOLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens, temperature,
                 clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode, denom_override, panel_hint, compact,
-                keep_logits=None):
+                keep_logits=None, chunk_tokens=0):
         idx = _valid_rows(labels_shifted, compact)
+        need = (ctx.needs_input_grad[0], ctx.needs_input_grad[1], bias is not None and ctx.needs_input_grad[2])
         needs_grad = any(ctx.needs_input_grad[:3])
-        lp, ent, lse, h_used, y_used, kept = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx,
-                                                               needs_grad, keep_logits)
-        ctx.kept = kept       # released by the first backward (a second backward through this node recomputes)
-        loss, g, lr, c1, l1, l2, scal = grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
-                                                      clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
-                                                      denom_override)
-        ctx.save_for_backward(h_used, weight, bias if bias is not None else hidden.new_empty(0), y_used, lse, g,
-                              idx if idx is not None else hidden.new_empty(0))
+        T_used = hidden.shape[0] if idx is None else idx.numel()
+        H, V = hidden.shape[1], weight.shape[0]
+        mode = _grad_mode(keep_logits)
+        chunk = int(chunk_tokens) if chunk_tokens and chunk_tokens > 0 else chunk_bound_for(V)   # a bound: the library deals the tokens evenly
+        chunked = needs_grad and mode in ("auto", "chunked") and weight.dtype == torch.bfloat16 and \
+            hidden.dtype == weight.dtype and chunked_supported(T_used, H, V, weight.dtype, chunk)
+        if mode == "chunked" and needs_grad and not chunked:
+            raise RuntimeError(f"fgrpo: keep_logits='chunked' but T={T_used} H={H} V={V} {weight.dtype} is not supported")
         ctx.has_bias = bias is not None
         ctx.compacted = idx is not None
         ctx.hidden_shape = tuple(hidden.shape)
         ctx.temperature = temperature
         ctx.panel_hint = panel_hint
+        ctx.kept = None
+        ctx.grads = None
+        if chunked:
+            # every gradient is formed here, chunk by chunk, for an upstream gradient of 1; backward() scales them
+            tokw, pre = loss_prepare(labels_shifted, cu_seqlens, loss_agg_mode, denom_override)
+            y_full = labels_shifted.reshape(-1)
+            if idx is None:
+                h_used, y_used = hidden, y_full
+                sel = lambda t: t
+            else:
+                h_used, y_used = hidden.index_select(0, idx), y_full.index_select(0, idx)
+                sel = lambda t: None if t is None else t.detach().reshape(-1).index_select(0, idx)
+            loss, lp, ent, lse, g, lr, c1, l1, l2, _scal, dH, dW, db = grpo_step_chunked(
+                h_used, weight, bias, y_used, sel(old_lp), sel(ref_lp), sel(adv), sel(tokw), pre, temperature, clip_low,
+                clip_high, clip_ratio_c, kl_beta, chunk, need[0], need[1], need[2], want_diag=idx is None)
+            if idx is not None:
+                # outputs live on all T positions: scatter, and let the objective kernels write the loss and the
+                # diagnostics there (as the other paths do; g, the gradients' source, stays the compacted one)
+                T = y_full.numel()
+                lp = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, lp)
+                ent = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, ent)
+                g = torch.zeros(T, dtype=torch.float32, device=hidden.device).index_copy_(0, idx, g)
+                loss, _g, lr, c1, l1, l2, _scal = grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
+                                                                clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
+                                                                denom_override)
+                if dH is not None:
+                    dH = torch.zeros(ctx.hidden_shape, dtype=dH.dtype, device=dH.device).index_copy_(0, idx, dH)
+            ctx.grads = (dH, dW, db)
+        else:
+            lp, ent, lse, h_used, y_used, kept = _logprob_fwd_rows(hidden, weight, bias, labels_shifted, temperature, idx,
+                                                                   needs_grad, "recompute" if mode == "chunked" else keep_logits)
+            ctx.kept = kept       # released by the first backward (a second backward through this node recomputes)
+            loss, g, lr, c1, l1, l2, scal = grpo_loss_fwd(lp, old_lp, ref_lp, adv, labels_shifted, cu_seqlens,
+                                                          clip_low, clip_high, clip_ratio_c, kl_beta, loss_agg_mode,
+                                                          denom_override)
+        ctx.save_for_backward(h_used, weight, bias if bias is not None else hidden.new_empty(0), y_used, lse, g,
+                              idx if idx is not None else hidden.new_empty(0))
         ctx.mark_non_differentiable(ent, lr, c1, l1, l2, lp)
         return loss, ent, lr, c1, l1, l2, lp
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
+        grads, ctx.grads = ctx.grads, None
+        if grads is not None:
+            # the chunked step left the gradients of the loss itself: multiply by the upstream scalar (on the device;
+            # exactly 1 costs three empty launches).  A second backward through this node recomputes, below.
+            scale = g_loss.detach().reshape(-1)[:1].to(torch.float32).contiguous()
+            for t in grads:
+                scale_inplace(t, scale)
+            return tuple(grads) + (None,) * 16
         h_used, weight, bias, y_used, lse, g, idx = ctx.saved_tensors
         bias = bias if ctx.has_bias else None
         need = (ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.has_bias and ctx.needs_input_grad[2])
         kept, ctx.kept = ctx.kept, None
         dH, dW, db = _bwd_rows(h_used, weight, bias, y_used, lse, g, g_loss, ctx.temperature, need, ctx.panel_hint,
                                idx if ctx.compacted else None, ctx.hidden_shape, kept)
-        return (dH, dW, db) + (None,) * 15
+        return (dH, dW, db) + (None,) * 16
 
 
 class _GRPOLossFromLogprobs(torch.autograd.Function):
@@ -732,13 +901,15 @@ def lmhead_logprob(hidden, weight, bias, labels_shifted, temperature=1.0, panel_
 
 def fused_grpo_loss(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp=None, cu_seqlens=None,
                     temperature=1.0, clip_low=0.2, clip_high=0.4, clip_ratio_c=1e32, kl_beta=0.0,
-                    loss_agg_mode="token_mean", denom_override=0.0, panel_hint=0, compact=False, keep_logits=None):
+                    loss_agg_mode="token_mean", denom_override=0.0, panel_hint=0, compact=False, keep_logits=None,
+                    chunk_tokens=0):
     """(loss, entropy, log_ratio, clip1, unclipped, clipped, lp); only loss carries a gradient.
-    ``keep_logits``: None = the module default (``KEEP_LOGITS``), True / False / "auto"."""
+    ``keep_logits``: how the gradients are formed, see ``KEEP_LOGITS`` (None = that module default);
+    ``chunk_tokens``: token chunk of the chunked step (0 = ``chunk_tokens_for``)."""
     return _FusedGRPOLoss.apply(hidden, weight, bias, labels_shifted, old_lp, adv, ref_lp, cu_seqlens,
                                 float(temperature), float(clip_low), float(clip_high), float(clip_ratio_c),
                                 float(kl_beta), loss_agg_mode, float(denom_override), int(panel_hint),
-                                compact if torch.is_tensor(compact) else bool(compact), keep_logits)
+                                compact if torch.is_tensor(compact) else bool(compact), keep_logits, int(chunk_tokens))
 
 
 # --------------------------------------------------------------------------- packed variable-length attention

@@ -241,14 +241,16 @@ def grpo_loss_and_entropy_ce_fn(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """6-tuple ``(loss, entropy, log_ratio, loss_clip1, loss_unclipped,
     loss_clipped)`` of the dual-clip token-mean objective (reference:
-    grpo_loss.py:256-348).  ``loss_chunksize`` only widens the transient of the
-    backward (one dLogits panel, bf16) beyond the library's own bound of a
-    quarter of ``[T, V]``, at most 2 GiB, when ``loss_chunksize * V`` elements
-    are more than that; the result does not depend on it.  Where the kernels
-    support the shape and memory allows, the bf16 logits are kept for the
-    backward as the reference's autograd keeps them (``keep_logits=False``
-    among the keyword arguments forces the recomputing backward, ``True``
-    insists on keeping)."""
+    grpo_loss.py:256-348).  When an input needs a gradient the whole step -
+    projection, objective and the gradients - runs here, token chunk by token
+    chunk as the reference's loop does (grpo_loss.py:280-316), with one chunk
+    of bf16 soft-max numerators as the only ``[. x V]`` transient
+    (``2 * loss_chunksize`` tokens, 8192 without one; ``backward()`` then only
+    multiplies by the upstream scalar).  The loss, the logprobs and the
+    diagnostics do not depend on the chunk size.  ``keep_logits`` among the
+    keyword arguments picks another way to the same gradients: ``False`` /
+    ``"recompute"`` recomputes the logits in ``backward()``, ``True`` /
+    ``"whole"`` keeps the numerators of the whole batch (``[T, V]`` bf16)."""
     if advantages is None:
         raise ValueError("grpo_loss_and_entropy_ce_fn: advantages are required")
     ref_logprobs = unused_kwargs.get("ref_logprobs", None)
@@ -277,7 +279,8 @@ def grpo_loss_and_entropy_ce_fn(
         advantages.reshape(-1),
         None if ref_logprobs is None else ref_logprobs.reshape(-1),
         cu_seqlens, temperature, clip_low, clip_high, clip_ratio_c, kl_beta,
-        loss_agg_mode, denom, hint, compact, unused_kwargs.get("keep_logits", None))
+        loss_agg_mode, denom, hint, compact, unused_kwargs.get("keep_logits", None),
+        ops.chunk_bound_for(V, loss_chunksize))
     return loss, ent, lr, c1, l1, l2
 
 

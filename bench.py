@@ -26,8 +26,8 @@ PEAK_CLOCK_MHZ = 2400.0
 # --copy-probe.  Not measured in the run that prints it: the figure belongs to the binary and workload named in the
 # profile summary it cites, and is None for workloads that were not profiled.
 PROFILED_TRAFFIC = {
-    # (workload, numerators kept): (bytes per launch, summary under profiles/)
-    ("cfg1", True): (3.2489e+10, "profiles/lmhead_fwd_kernel_cfg1_traffic_pmc.txt"),
+    # (workload, path): (bytes per launch of the forward kernel, summary under profiles/)
+    ("cfg1", "whole"): (3.2489e+10, "profiles/lmhead_fwd_kernel_cfg1_traffic_pmc.txt"),
 }
 
 
@@ -39,7 +39,9 @@ def cpu_baseline(name: str, cfg_chunk, seed: int):
     from oracle import grpo_oracle as O
     from fgrpo.synthetic import CONFIGS
     cfg = CONFIGS[name]
-    cores = min(os.cpu_count() or 1, 16)
+    # every core this process may use: the harness states its share in OMP_NUM_THREADS where the machine has more
+    # cores than that share (torch then starts with that many threads); otherwise all of os.cpu_count()
+    cores = int(os.environ.get("OMP_NUM_THREADS") or 0) or (os.cpu_count() or 1)
     torch.set_num_threads(cores)
     H, V = cfg["H"], cfg["V"]
     g = torch.Generator().manual_seed(seed)
@@ -62,13 +64,17 @@ def cpu_baseline(name: str, cfg_chunk, seed: int):
 
     probe = 128
     t_probe = run(probe)            # also the warm-up
-    # aim at ~5 s per run (three timed runs), at most the configuration's own chunk size
-    n = int(max(probe, min(cfg_chunk or 4096, probe * 5.0 / max(t_probe, 1e-3))))
+    # one chunk of the configuration's own size, unless three runs of it would take more than 45 s on this host
+    # (then the largest multiple of 128 tokens that stays inside; the line says which)
+    want = cfg_chunk or 4096
+    fits = probe * (45.0 / 3.0) / max(t_probe, 1e-3)
+    n = int(max(probe, min(want, fits)))
     n = max(probe, (n // 128) * 128)
     times = sorted(run(n) for _ in range(3))
     t = times[1]
-    return {"value": n / t, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{n} tokens (one chunk) at full H={H}, V={V}, fwd{'' if cfg['forward_only'] else '+bwd'}, "
+    what = "one chunk of the configuration's size" if n == want else f"a slice of the configuration's {want}-token chunk: three runs of the whole chunk would exceed the 45 s bound"
+    return {"value": n / t, "unit": "tokens/s", "cores": cores, "os_cpu_count": os.cpu_count(), "kind": "port",
+            "sample": f"{n} tokens ({what}) at full H={H}, V={V}, fwd{'' if cfg['forward_only'] else '+bwd'}, "
                       f"fp32 math on bf16-rounded inputs, one warm-up, median of 3 ({times[0]:.2f}/{times[1]:.2f}/"
                       f"{times[2]:.2f} s); tokens/s is linear in tokens"}
 
@@ -381,9 +387,14 @@ def main():
     ap.add_argument("--reward-p", type=float, default=None,
                     help="probability of reward 1 per sample (default: the configuration's); with --objective reference "
                          "it sets the share of zero-advantage groups")
-    ap.add_argument("--keep-logits", choices=["auto", "on", "off"], default="auto",
-                    help="keep the [T x V] bf16 soft-max numerators for the backward (auto: when supported and memory allows) "
-                         "or recompute the logits there")
+    ap.add_argument("--keep-logits", choices=["auto", "chunked", "whole", "on", "recompute", "off"], default="auto",
+                    help="the headline path's way to the gradients: chunked (the default where supported: the whole step in "
+                         "token chunks, one chunk of bf16 soft-max numerators as the transient), whole / on (numerators of the "
+                         "whole batch kept, [T x V] bf16), recompute / off (logits recomputed in the backward)")
+    ap.add_argument("--chunk", type=int, default=None,
+                    help="loss_chunksize handed to the drop-in instead of the configuration's (the chunked step walks twice that many tokens at a time)")
+    ap.add_argument("--no-alt-paths", action="store_true",
+                    help="time the headline path only (by default the other ways to the same gradients are timed after it)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed steps, run one 1 GiB device copy (reference point for traffic counters)")
     ap.add_argument("--seed", type=int, default=0)
@@ -424,8 +435,9 @@ def main():
     fwd_only = p["forward_only"]
     labels = w.labels
     shifted = ops.shift_labels(labels).reshape(-1)
-    keep_logits = {"auto": None, "on": True, "off": False}[args.keep_logits]
     north_star = args.objective == "north_star"
+    thv = 2.0 * T * H * V
+    chunk_arg = p["chunk"] if args.chunk is None else args.chunk
 
     # inputs of the objective: advantages from the group kernel, old/ref = current logprob + noise
     adv_s = ops.group_advantages(w.rewards, w.group_offsets, p["adv_eps"])
@@ -444,7 +456,7 @@ def main():
             self.cu = w.cu_seqlens.clone()
     sets = [Inputs(), Inputs()]
 
-    def step(k=0):
+    def step(k=0, keep_logits=None):
         s = sets[k % len(sets)]
         if fwd_only:
             with torch.no_grad():
@@ -453,14 +465,42 @@ def main():
         s.weight.grad = None
         extra = dict(ref_logprobs=s.ref, kl_beta=p["kl_beta"], loss_agg_mode="sample_mean", cu_seqlens=s.cu) if north_star else {}
         out = G.grpo_loss_and_entropy_ce_fn(s.weight, None, s.hidden, s.labels, 1.0, s.old, s.adv, p["clip_low"],
-                                            p["clip_high"], p["clip_ratio_c"], loss_chunksize=p["chunk"],
+                                            p["clip_high"], p["clip_ratio_c"], loss_chunksize=chunk_arg,
                                             keep_logits=keep_logits, **extra)
         out[0].backward()
         return out
 
+    # Which way to the gradients each timed path takes (fgrpo.ops.KEEP_LOGITS); the headline is the default.
+    chunk_tok = ops.chunk_tokens_for(T, V, chunk_arg)
+    chunked_ok = (not fwd_only) and ops.chunked_supported(T, H, V, w.dtype, chunk_tok)
+    whole_ok = (not fwd_only) and ops.keep_supported(T, H, V, w.dtype)
+    headline = {"auto": "chunked" if chunked_ok else "recompute", "chunked": "chunked", "on": "whole", "whole": "whole",
+                "off": "recompute", "recompute": "recompute"}[args.keep_logits]
+    if fwd_only:
+        headline = "forward"
+    n_chunks = (T + chunk_tok - 1) // chunk_tok if chunked_ok else 1
+    lib = ops._lib.load()
+    path_notes = {
+        "chunked": {"never_holds_T_x_V": True, "executed_products": 3,
+                    "what": f"the whole step in {n_chunks} token chunks of {chunk_tok}: forward keeping one chunk of bf16 soft-max "
+                            "numerators, objective, dHidden rows, dW summed in fp32 across chunks; backward() scales by the upstream scalar",
+                    "transient_bytes": int(lib.fgrpo_grpo_step_chunked_workspace(T, H, V, ops._lib.BF16, chunk_tok)) if chunked_ok else None,
+                    "transient_of_which_kept_numerators_bytes": int(ops.logits_keep_bytes(min(T, chunk_tok), V)) if chunked_ok else None,
+                    "transient_of_which_fp32_dW_sum_bytes": (4 * V * H if n_chunks > 1 else 0) if chunked_ok else None},
+        "whole": {"never_holds_T_x_V": False, "executed_products": 3,
+                  "what": "bf16 soft-max numerators of the whole batch kept between forward and backward",
+                  "transient_bytes": int(ops.logits_keep_bytes(T, V)) if whole_ok else None},
+        "recompute": {"never_holds_T_x_V": True, "executed_products": 4,
+                      "what": "logits recomputed in backward(), one vocabulary panel of dLogits at a time",
+                      "transient_bytes": None if fwd_only else int(lib.fgrpo_lmhead_bwd_workspace(T, H, V, ops._lib.BF16 if w.dtype == torch.bfloat16 else ops._lib.F32,
+                                                                                     ops.panel_elems_bound(T, V, chunk_arg)))},
+        "forward": {"never_holds_T_x_V": True, "executed_products": 1, "what": "forward only (logprobs and entropy), no gradient",
+                    "transient_bytes": int(lib.fgrpo_logprob_fwd_workspace(T, H, V, ops._lib.BF16 if w.dtype == torch.bfloat16 else ops._lib.F32))},
+    }
+
     # ---- parity on the same inputs, before timing ----
     def gate_step():
-        out = step(0)
+        out = step(0, None if fwd_only else headline)
         torch.cuda.synchronize()
         if fwd_only:
             return out[0], out[1], None, None
@@ -472,31 +512,90 @@ def main():
             print("bench.py: parity check failed, nothing timed: " + json.dumps(parity), file=sys.stderr)
             sys.exit(1)
 
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    # Per-kernel times inside the timed steps: HIP events recorded on the launch stream around the forward's
-    # library call (the bracket also holds the per-token combine kernel, some tens of microseconds) and, inside the
-    # library, around each launch of the backward.
-    fwd_events = []
-    ops.set_fwd_event_sink(fwd_events)
-    if not fwd_only:
-        ops.phase_timing_begin()
-    step_events = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    with ClockSampler() as clock:
-        t0 = time.perf_counter()
-        step_events[0].record()
-        for i in range(args.steps):
-            step(i)
-            step_events[i + 1].record()
+    def phase(kernel, total_ms, launches, steps, flops, note=None):
+        per = total_ms / steps
+        d = {"kernel": kernel, "ms": per, "launches_per_step": launches // steps if steps else 0, "flops": flops,
+             "frac": (flops / (per * 1e-3) / 1e12 / PEAK_BF16_TFLOPS) if (flops and per > 0) else None}
+        if note:
+            d["note"] = note
+        return d
+
+    def measure(path, steps, warmup, sample_clock=False):
+        """`steps` timed steps of one path after `warmup` untimed ones: wall clock around the loop (bracketed by
+        synchronisations), HIP events per step, and HIP events on the launch stream around the kernels' launches
+        (inside the library for the backward and the chunked step, around the library call for the stand-alone
+        forward)."""
+        keep = None if fwd_only else path
+        for i in range(warmup):
+            step(i, keep)
         torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-    ops.set_fwd_event_sink(None)
-    phase_ms, phase_n, dropped = ops.phase_timing_end() if not fwd_only else ({}, {}, 0)
-    per_step = sorted(step_events[i].elapsed_time(step_events[i + 1]) for i in range(args.steps))
-    ms = dt / args.steps * 1e3
-    tok_s = T / (ms / 1e3)
-    k_ms = sum(a.elapsed_time(b) for a, b in fwd_events) / max(1, len(fwd_events))
+        fwd_events = []
+        ops.set_fwd_event_sink(fwd_events)
+        if not fwd_only:
+            ops.phase_timing_begin()
+        step_events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        clock = ClockSampler()
+        with clock:
+            t0 = time.perf_counter()
+            step_events[0].record()
+            for i in range(steps):
+                step(i, keep)
+                step_events[i + 1].record()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        ops.set_fwd_event_sink(None)
+        phase_ms, phase_n, dropped = ops.phase_timing_end() if not fwd_only else ({}, {}, 0)
+        per_step = sorted(step_events[i].elapsed_time(step_events[i + 1]) for i in range(steps))
+        ms = dt / steps * 1e3
+        if path == "chunked":
+            k_total, k_n = phase_ms["fwd"], phase_n["fwd"]
+            tok_per_launch = T / max(1, k_n // steps)
+        else:
+            k_total, k_n = sum(a.elapsed_time(b) for a, b in fwd_events), len(fwd_events)
+            tok_per_launch = T
+        k_ms = k_total / max(1, k_n)
+        flops_launch = 2.0 * tok_per_launch * H * V
+        kept = path in ("chunked", "whole")
+        fwd_name = "lmhead_fwd_kernel" + (" (keeps the bf16 soft-max numerators" + (" of one token chunk)" if path == "chunked" else ")") if kept else "") + " + combine"
+        phases = [phase(fwd_name, k_total, k_n, steps, thv)]
+        if not fwd_only:
+            if kept:
+                phases.append(phase("keep_backward_prep_kernel (+ the gated recompute launch, scaled transposed copy of hidden, live runs)",
+                                    phase_ms["dlogits"], phase_n["dlogits"], steps, 0.0,
+                                    f"per-token factors, one patched element per row ({4.0 * T * H / 1e6:.0f} MB): no pass over [T x V]"))
+            else:
+                phases.append(phase("lmhead_ds_kernel (recomputes the logits, one vocabulary panel per launch)",
+                                    phase_ms["dlogits"], phase_n["dlogits"], steps, thv, "executed, not algorithmic, work"))
+            phases.append(phase("gemm_store_kernel dHidden", phase_ms["dh"], phase_n["dh"], steps, thv))
+            phases.append(phase("gemm_store_kernel dW" + (" (fp32 sum across chunks)" if path == "chunked" and n_chunks > 1 else ""),
+                                phase_ms["dw"], phase_n["dw"], steps, thv))
+            phases.append(phase("objective, normalisers, upstream scale, bias sums", phase_ms["other"], phase_n["other"], steps, 0.0))
+        alg = (1.0 if fwd_only else 3.0) * thv
+        res = {"path": path, **path_notes[path], "steps": steps, "warmup": warmup, "ms_per_step": ms,
+               "ms_per_step_median": per_step[len(per_step) // 2], "ms_per_step_min": per_step[0],
+               "tokens_per_s": T / (ms / 1e3), "path_mfma_frac": alg / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+               "path_algorithmic_tflops": alg / (ms * 1e-3) / 1e12,
+               "path_executed_tflops": path_notes[path]["executed_products"] * thv / (ms * 1e-3) / 1e12,
+               "forward_kernel_ms_per_launch": k_ms, "forward_launches_timed": k_n,
+               "forward_frac": flops_launch / (k_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS if k_ms > 0 else None,
+               "phases": phases, "phase_brackets_dropped": dropped}
+        return res, clock.summary(), k_ms, flops_launch, k_n
+
+    head, clock_summary, k_ms, flops_launch, k_n = measure(headline, args.steps, args.warmup)
+    ms = head["ms_per_step"]
+    tok_s = head["tokens_per_s"]
+
+    # the other ways to the same gradients, timed after the headline with fewer steps
+    alt = {}
+    if not fwd_only and not args.no_alt_paths:
+        for path in ("whole", "recompute", "chunked"):
+            if path == headline or (path == "whole" and not whole_ok) or (path == "chunked" and not chunked_ok):
+                continue
+            try:
+                alt[{"whole": "whole_batch_kept"}.get(path, path)] = measure(path, max(3, min(args.steps, 8)), 2)[0]
+            except Exception as e:      # noqa: BLE001
+                alt[path] = {"error": f"{type(e).__name__}: {e}"[:300]}
+            torch.cuda.empty_cache()
 
     yardstick = None
     if not args.no_library_yardstick:
@@ -512,32 +611,8 @@ def main():
         torch.cuda.synchronize()
         dst.copy_(src)
         torch.cuda.synchronize()
-    thv = 2.0 * T * H * V
-    achieved = thv / (k_ms * 1e-3) / 1e12
-    alg_flops_step = (1.0 if fwd_only else 3.0) * thv
-    kept = (not fwd_only) and phase_n.get("dlogits", 0) == args.steps and phase_n.get("dh", 0) == args.steps
-    executed = (1.0 if fwd_only else (3.0 if kept else 4.0)) * thv
-
-    def phase(kernel, total_ms, flops, note=None):
-        per = total_ms / args.steps
-        d = {"kernel": kernel, "ms": per, "flops": flops,
-             "frac": (flops / (per * 1e-3) / 1e12 / PEAK_BF16_TFLOPS) if (flops and per > 0) else None}
-        if note:
-            d["note"] = note
-        return d
-    phases = [phase("lmhead_fwd_kernel" + (" (keeps the bf16 soft-max numerators)" if kept else "") + " + combine",
-                    k_ms * args.steps, thv)]
-    if not fwd_only:
-        if kept:
-            phases.append(phase("keep_backward_prep_kernel", phase_ms["dlogits"], 0.0,
-                                "per-token factors, one patched element per row, scaled transposed copy of hidden "
-                                f"({4.0 * T * H / 1e6:.0f} MB): no pass over [T x V]"))
-        else:
-            phases.append(phase(f"lmhead_ds_kernel x {phase_n['dlogits'] // args.steps} panels (recomputes the logits)",
-                                phase_ms["dlogits"], thv, "executed, not algorithmic, work"))
-        phases.append(phase(f"gemm_store_kernel dHidden x {phase_n['dh'] // args.steps}", phase_ms["dh"], thv))
-        phases.append(phase(f"gemm_store_kernel dW x {phase_n['dw'] // args.steps}", phase_ms["dw"], thv))
-    prof = PROFILED_TRAFFIC.get((args.config, bool(kept)))
+    achieved = flops_launch / (k_ms * 1e-3) / 1e12
+    prof = PROFILED_TRAFFIC.get((args.config if args.tokens is None else None, headline))
 
     line = {
         "metric": "packed tokens/sec fused logprob+GRPO fwd/bwd (Qwen2.5-1.5B shape); MFMA % peak",
@@ -546,38 +621,41 @@ def main():
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "fp32", "data": "synthetic",
         "config": {"workload": f"{args.config}: T={T} packed tokens, H={H}, V={V}, "
                                f"{'forward only' if fwd_only else 'forward+backward (dHidden, dW)'}, "
-                               f"{w.n_samples} samples, chunk hint {p['chunk']}",
+                               f"{w.n_samples} samples, loss chunk size {chunk_arg}",
                    "tokens": T, "hidden": H, "vocab": V, "samples": w.n_samples,
                    "objective": None if fwd_only else (
                        "north_star: dual clip + k3 KL to the reference policy, mean over samples of per-sample token means"
                        if north_star else "reference: dual clip, token mean, no KL (grpo_loss.py:318-348)"),
                    "tokens_without_gradient": None if fwd_only else float(((adv == 0) | (shifted == -100)).float().mean()) if not north_star
                    else float((shifted == -100).float().mean()),
-                   "backward": None if fwd_only else ("bf16 soft-max numerators kept for the backward" if kept else "logits recomputed in the backward"),
+                   "backward": None if fwd_only else f"{headline}: {path_notes[headline]['what']}",
+                   "never_holds_T_x_V": path_notes[headline]["never_holds_T_x_V"],
+                   "transient_bytes": path_notes[headline]["transient_bytes"],
                    "input_sets_rotated": len(sets)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS,
-                     "frac_at_held_clock": (achieved / (PEAK_BF16_TFLOPS * clock.summary()["median_mhz"] / PEAK_CLOCK_MHZ))
-                     if clock.summary() else None,
+                     "frac_at_held_clock": (achieved / (PEAK_BF16_TFLOPS * clock_summary["median_mhz"] / PEAK_CLOCK_MHZ))
+                     if clock_summary else None,
                      "traffic": prof[0] if prof else None,
                      "traffic_source": (prof[1] + " (rocprofv3 --pmc runs of this command; not measured in this run)") if prof else None,
-                     "kernel": phases[0]["kernel"], "kernel_ms": k_ms,
-                     "kernel_launches_timed": len(fwd_events),
-                     "algorithmic_flops_per_launch": thv,
-                     "phases": phases, "phase_brackets_dropped": dropped,
+                     "kernel": head["phases"][0]["kernel"], "kernel_ms": k_ms,
+                     "kernel_launches_timed": k_n,
+                     "algorithmic_flops_per_launch": flops_launch,
+                     "phases": head["phases"], "phase_brackets_dropped": head["phase_brackets_dropped"],
                      "library_yardstick": yardstick,
                      "peak_note": f"published peak = {PEAK_CLOCK_MHZ:.0f} MHz x 256 CUs x 4096 flop/cycle; the clock the "
                                   "device held during the timed steps is under 'clock'"},
-        "clock": clock.summary(),
+        "clock": clock_summary,
         "parity": parity,
-        "ms_per_step_median": per_step[len(per_step) // 2], "ms_per_step_min": per_step[0],
-        "path_mfma_frac": alg_flops_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-        "path_algorithmic_tflops": alg_flops_step / (ms * 1e-3) / 1e12,
-        # what the matrix pipeline executes: with kept logits the three algorithmic products, otherwise a fourth
-        "path_executed_tflops": executed / (ms * 1e-3) / 1e12,
+        "ms_per_step_median": head["ms_per_step_median"], "ms_per_step_min": head["ms_per_step_min"],
+        "path_mfma_frac": head["path_mfma_frac"],
+        "path_algorithmic_tflops": head["path_algorithmic_tflops"],
+        # what the matrix pipeline executes: three products where numerators are kept, a fourth where logits are recomputed
+        "path_executed_tflops": head["path_executed_tflops"],
+        "alt_paths": alt or None,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.config, p["chunk"], args.seed)
+        line["cpu_baseline"] = cpu_baseline(args.config, chunk_arg, args.seed)
     print(json.dumps(line), flush=True)
 
 

@@ -115,7 +115,7 @@ int fgrpo_lmhead_bwd(const void* hidden, const void* weight, const void* bias,
  * Range: E[t][v] = exp(x_tv / temperature - ref_t) in bf16 with ref_t = max(target logit, largest logit among the
  * first 512 vocabulary rows) / temperature + 40: finite as long as no logit of a scored token lies more than 123
  * (in units of log probability) above that maximum; the forward raises a flag in the buffer otherwise,
- * fgrpo_keep_overflowed() reads it (it waits for `stream`), and the caller must then use fgrpo_lmhead_bwd.  Rows of ignored tokens are stored as exact zeros.
+ * and fgrpo_lmhead_bwd_kept, which reads it on the device, then recomputes dLogits into the buffer before its two products (fgrpo_keep_overflowed() reports the flag to the host).  Rows of ignored tokens are stored as exact zeros.
  * logits_keep: fgrpo_logits_keep_bytes(T, V) bytes, 16-byte aligned: [ceil(V/256)][round_up(T,256)][256] bf16,
  * then the references and the flag.  workspace of the backward: fgrpo_lmhead_bwd_kept_workspace bytes (the token
  * factors, the scaled transposed copy of hidden, and an fp32 dH accumulator used only when the tuning key keep_panels splits
@@ -132,8 +132,11 @@ int fgrpo_logprob_fwd_keep(const void* hidden, const void* weight, const void* b
                            float* lp_out, float* ent_out, float* lse_out,
                            void* logits_keep, size_t logits_keep_bytes,
                            void* workspace, size_t workspace_bytes, void* stream);
-/* 1 when the kept values may have overflowed (use fgrpo_lmhead_bwd), 0 when they are good, negative on error.
- * Synchronises `stream`. */
+/* 1 when the kept values may have overflowed, 0 when they are good, negative on error.  Synchronises `stream`.
+ * A query for tests and reports: fgrpo_lmhead_bwd_kept and fgrpo_grpo_step_chunked read the flag on the device
+ * themselves (when it is set, a launch that otherwise returns at once overwrites the buffer with dLogits recomputed
+ * from the operands, and the same two products then give the recomputing backward's gradients), so no caller has to
+ * wait for the forward before queueing the backward. */
 int fgrpo_keep_overflowed(const void* logits_keep, int T, int V, void* stream);
 size_t fgrpo_lmhead_bwd_kept_workspace(int T, int H, int V, int dtype);
 int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bias,
@@ -151,9 +154,10 @@ int fgrpo_lmhead_bwd_kept(const void* hidden, const void* weight, const void* bi
  * brackets are counted as dropped).  Meant for one stream at a time.  _end waits
  * for the last event and returns, per phase, the summed milliseconds and the number of brackets:
  * phase 0 = dLogits (recomputing kernel, or the in-place pass over kept logits), 1 = dHidden product,
- * 2 = dW product, 3 = everything else (operand staging, bias sums).  Returns the number of dropped brackets
+ * 2 = dW product, 3 = everything else (operand staging, bias sums, the objective kernels of
+ * fgrpo_grpo_step_chunked), 4 = the forward launches of fgrpo_grpo_step_chunked.  Returns the number of dropped brackets
  * (0 = all timed) or a negative error.  Timing is off unless begun; no counterpart in the reference. */
-#define FGRPO_NUM_PHASES 4
+#define FGRPO_NUM_PHASES 5
 #define FGRPO_MAX_TIMED_PHASES 1024
 int fgrpo_phase_timing_begin(void);
 int fgrpo_phase_timing_end(float* ms_by_phase, int* brackets_by_phase);
@@ -175,6 +179,51 @@ int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, co
                    float* loss_out, float* g_out, float* log_ratio, float* clip1,
                    float* unclipped, float* clipped, float* scal_out,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- the whole training step of one packed micro-batch, token chunk by token chunk --------------------------
+ * Replaces the chunk loop of grpo_loss_and_entropy_ce_fn (grpo_loss.py:280-316), the objective behind it
+ * (grpo_loss.py:318-348) AND what autograd later derives from them, in one call that never holds more than one
+ * token chunk of [. x V]: for each chunk of `chunk` tokens
+ *   forward with kept numerators (fgrpo_logprob_fwd_keep) into ONE chunk-sized buffer  ->  the objective on the
+ *   chunk's tokens  ->  that chunk's rows of dH (written once)  ->  its contribution to dW (and dbias), carried
+ *   in fp32 from chunk to chunk in a fixed order, converted by the last chunk's product.
+ * This is possible because every normaliser of the objective (valid tokens, tokens per sample, samples) depends on
+ * the labels and cu_seqlens only: fgrpo_loss_prepare forms them first - tokw_out [T] = 1 / (valid tokens of the
+ * token's sample) and seg_cnt_out [nseq] for FGRPO_AGG_SAMPLE_MEAN (both may be NULL for TOKEN_MEAN), pre_out [4]
+ * doubles = {normaliser, valid tokens, non-empty samples, 1 / normaliser rounded to fp32} - and
+ * g_t = d loss / d lp_t is final as soon as lp_t is.  The gradients are those of the loss itself (upstream gradient
+ * 1); a caller whose autograd later delivers another upstream scalar multiplies them with fgrpo_scale_inplace
+ * (x[i] *= *scale_dev for n elements of `dtype`; a scale of exactly 1 returns without touching the array).
+ * Executed matrix work: 6 T H V (the reference's own three products), against 8 T H V for the recomputing pair;
+ * transient: fgrpo_logits_keep_bytes(chunk, V) + the fp32 dW sum (V x H x 4 bytes, only with more than one chunk).
+ * chunk_tokens <= 0: 8192.  The chunk used is fgrpo_grpo_step_chunk_tokens(T, chunk_tokens): the bound rounded down
+ * to whole 256-token tiles, then the tokens dealt evenly over ceil(T / bound) chunks.  Results do not depend on the
+ * chunk size beyond fp32 summation order (of a token's vocabulary partial sums, whose split follows the token count
+ * of a launch, and of dW across chunks): two calls with the same chunk size are bit-identical.
+ * old_lp / ref_lp / tokw may be NULL (ratio 1 / no KL term / token mean); kl_beta as in fgrpo_loss_fwd.  Outputs as
+ * in fgrpo_logprob_fwd and fgrpo_loss_fwd (lse_out and g_out are required: the gradients are formed from them);
+ * dH_out [T x H], dW_out [V x H], dbias_out [V] in `dtype`, each may be NULL.  Supported
+ * (fgrpo_grpo_step_chunked_supported() != 0) where fgrpo_keep_supported holds for the chunk and for the shorter last
+ * chunk; otherwise FGRPO_ERR_UNSUPPORTED (use the recomputing pair).
+ * Out-of-range chunks (see fgrpo_logprob_fwd_keep) are recomputed on the device, chunk by chunk, without a host
+ * synchronisation: the call can be captured in a HIP graph. */
+int fgrpo_loss_prepare(const int64_t* labels_shifted, const int32_t* cu_seqlens, int nseq, int T,
+                       int agg_mode, double denom_override,
+                       float* tokw_out, int32_t* seg_cnt_out, double* pre_out, void* stream);
+int fgrpo_grpo_step_chunk_tokens(int T, int chunk_tokens);
+int fgrpo_grpo_step_chunked_supported(int T, int H, int V, int dtype, int chunk_tokens);
+size_t fgrpo_grpo_step_chunked_workspace(int T, int H, int V, int dtype, int chunk_tokens);
+int fgrpo_grpo_step_chunked(const void* hidden, const void* weight, const void* bias,
+                            const int64_t* labels_shifted, const float* old_lp, const float* ref_lp,
+                            const float* adv, const float* tokw, const double* pre,
+                            float inv_temperature, int T, int H, int V, int dtype,
+                            float clip_low, float clip_high, float clip_ratio_c, float kl_beta,
+                            int chunk_tokens,
+                            float* lp_out, float* ent_out, float* lse_out, float* loss_out, float* g_out,
+                            float* log_ratio, float* clip1, float* unclipped, float* clipped, float* scal_out,
+                            void* dH_out, void* dW_out, void* dbias_out,
+                            void* workspace, size_t workspace_bytes, void* stream);
+int fgrpo_scale_inplace(void* x, long long n, int dtype, const float* scale_dev, void* stream);
 
 /* ---- diagnostics on the output-token positions ---------------------------------
  * Replaces the ~20 .item() reductions of compute_dual_clip_grpo_loss

@@ -100,9 +100,10 @@ def test_kept_logits_panel_split_matches_single_launch(dev):
 def test_kept_values_out_of_range_fall_back_to_recomputation(dev):
     """The kept numerators are exp(x_v - ref - 40) in bf16 with ref = max(target logit, largest logit among the first
     512 vocabulary entries): a row whose largest logit exceeds both by more than 128 would overflow them.  The
-    forward flags it, and the backward then recomputes: same gradients, bit for bit, as with keep_logits=False;
-    the forward's own outputs never depend on the kept values.  The same dominant entry INSIDE the sampled rows
-    raises no flag."""
+    forward flags it, and the backward - which reads the flag on the device, no host wait - then overwrites the
+    buffer with dLogits recomputed from the operands before its two products: the recomputing backward's gradients
+    (the same bf16 dLogits; the fp32 sums run in another order), finite everywhere; the forward's own outputs never
+    depend on the kept values.  The same dominant entry INSIDE the sampled rows raises no flag."""
     from fgrpo import ops
     T, H, V = 8192, 1024, 8192
     gen = torch.Generator().manual_seed(21)
@@ -122,8 +123,11 @@ def test_kept_values_out_of_range_fall_back_to_recomputation(dev):
         out = ops.fused_grpo_loss(h, w, None, y_d, None, adv_d, keep_logits=keep)
         out[0].backward()
         grads.append((h.grad, w.grad, out[0].detach()))
-    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
-    assert torch.equal(grads[0][2], grads[1][2]) and torch.isfinite(grads[0][1].float()).all()
+    cos64 = lambda a, b: float((a.double().flatten() @ b.double().flatten()) / (a.double().norm() * b.double().norm()))
+    assert cos64(grads[0][0], grads[1][0]) >= 0.99999 and cos64(grads[0][1], grads[1][1]) >= 0.99999
+    assert (grads[0][0].float() - grads[1][0].float()).abs().max() <= 2e-2 * grads[1][0].float().abs().max()
+    assert torch.equal(grads[0][2], grads[1][2])
+    assert torch.isfinite(grads[0][0].float()).all() and torch.isfinite(grads[0][1].float()).all()
     # the dominant entry among the sampled rows: the reference follows it, nothing overflows
     W1 = W.clone()
     W1[4000] = W[4001]
@@ -307,15 +311,17 @@ def test_keep_refuses_what_it_cannot_do(dev):
 
 
 # ------------------------------------------------------------------ full benchmark sizes through the drop-in
-@pytest.mark.parametrize("name,keep,tokens", [("cfg1", True, None), ("cfg1", False, None), ("cfg2", True, None),
-                                              ("cfg2", False, None), ("cfg4", True, None), ("cfg4", False, None),
-                                              ("cfg1", True, 33000)])
+@pytest.mark.parametrize("name,keep,tokens", [("cfg1", "chunked", None), ("cfg1", True, None), ("cfg1", False, None),
+                                              ("cfg2", "chunked", None), ("cfg2", True, None), ("cfg2", False, None),
+                                              ("cfg4", "chunked", None), ("cfg4", True, None), ("cfg4", False, None),
+                                              ("cfg1", "chunked", 33000), ("cfg1", True, 33000)])
 def test_full_size_through_the_drop_in(dev, name, keep, tokens):
     """grpo_loss_and_entropy_ce_fn exactly as bench.py calls it (KL to the reference policy, mean over samples of
     per-sample token means, cu_seqlens, the configuration's chunk hint), then backward with a non-unit upstream
     scale.  Checked: loss and the four per-token diagnostics against the oracle's objective evaluated on the
     kernel's per-token logprobs; sampled rows of dH and of dW against the closed form with the oracle's per-token
-    gradient; columns of dW summing to zero."""
+    gradient; columns of dW summing to zero.  keep: "chunked" = the default, the whole step in token chunks of twice
+    the configuration's chunk size; True = numerators of the whole batch kept; False = logits recomputed."""
     import grpo_loss as G
     from fgrpo import ops
     from fgrpo.synthetic import make_workload
