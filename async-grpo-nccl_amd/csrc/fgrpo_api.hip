@@ -505,9 +505,47 @@ int* keep_flag_of(void* keep, int T, int V) {
   return (int*)((char*)keep + keep_block_bytes(T, V) + 2 * (size_t)round_up(T, 256) * sizeof(float));
 }
 
+// Per-token references and target logits of a kept buffer, and its overflow flag.  They lie behind the numerators
+// in the buffer itself - unless the caller has formed them already, for the tokens of many launches at once
+// (ready: the forward then skips its own pre-pass, and the flag was cleared with them).
+struct KeepAux {
+  float* ref2;
+  float* xy;
+  int* flag;
+  bool ready;
+};
+KeepAux keep_aux_of(void* keep, int T, int V) {
+  return KeepAux{keep_ref2_of(keep, T, V), keep_xy_of(keep, T, V), keep_flag_of(keep, T, V), false};
+}
+
+// The pre-pass of the kept forward: the reference's sample of the vocabulary - the plain forward kernel over the
+// first rows of W; only the maxima of its per-split partials are used - then one dot product per token.
+// `p`: the forward's parameters for these tokens (operands staged, bias, labels, temperature); part: scratch for
+// min(2, nsplit) x T partials.
+int keep_prepass(const FwdParams& p, const void* hidden, const void* weight, const int64_t* labels, int T, int H, int V,
+                 int nsplit, float4* part, const KeepAux& aux, int nflags, hipStream_t st) {
+  FwdParams sp = p;
+  const int vs = V < kKeepSampleRows ? V : kKeepSampleRows;
+  sp.g.M = vs;
+  sp.g.N = T;
+  sp.tiles_v = (vs + kCfg[8].bm - 1) / kCfg[8].bm;
+  sp.tiles_t = (T + kCfg[8].bn - 1) / kCfg[8].bn;
+  sp.nsplit = sp.tiles_v < nsplit ? sp.tiles_v : nsplit;
+  sp.part = part;
+  sp.keep = nullptr;
+  int rc = launch_fwd_variant(8, sp, st);
+  if (rc) return rc;
+  KeepRefParams r{(const bf16_t*)hidden, (const bf16_t*)weight, p.bias, (const long long*)labels, T, H, V, p.inv_temp,
+                  part, sp.nsplit, aux.ref2, aux.xy, aux.flag, nflags};
+  hipLaunchKernelGGL(keep_reference_kernel, dim3((T + 3) / 4), dim3(256), 0, st, r);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, const int64_t* labels, float inv_temp,
                       int T, int H, int V, int dtype, float* lp_out, float* ent_out, float* lse_out, void* ws,
-                      size_t ws_bytes, void* stream, void* keep = nullptr, const Tuning* snapshot = nullptr) {
+                      size_t ws_bytes, void* stream, void* keep = nullptr, const Tuning* snapshot = nullptr,
+                      const KeepAux* aux_in = nullptr) {
   hipStream_t st = (hipStream_t)stream;
   if (!hidden || !weight || !labels || !lp_out) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: null argument");
   if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "logprob_fwd: T=%d H=%d V=%d", T, H, V);
@@ -547,23 +585,13 @@ int logprob_fwd_impl(const void* hidden, const void* weight, const void* bias, c
   if (keep) {
     p.keep = (bf16_t*)keep;
     p.keep_blk = (long long)pl.tiles_t * kCfg[8].bn * 256;
-    float* ref2 = keep_ref2_of(keep, T, V);
-    int* flag = keep_flag_of(keep, T, V);
-    // the reference's sample of the vocabulary: the plain forward kernel over the first rows of W; only the maxima
-    // of its per-split partials are used (the main launch below overwrites the partials afterwards)
-    FwdParams sp = p;
-    const int vs = V < kKeepSampleRows ? V : kKeepSampleRows;
-    sp.g.M = vs;
-    sp.tiles_v = (vs + kCfg[8].bm - 1) / kCfg[8].bm;
-    sp.nsplit = sp.tiles_v < pl.nsplit ? sp.tiles_v : pl.nsplit;
-    rc = launch_fwd_variant(8, sp, st);
-    if (rc) return rc;
-    KeepRefParams r{(const bf16_t*)hidden, (const bf16_t*)weight, p.bias, (const long long*)labels, T, H, V, inv_temp,
-                    pl.part, sp.nsplit, ref2, keep_xy_of(keep, T, V), flag};
-    hipLaunchKernelGGL(keep_reference_kernel, dim3((T + 3) / 4), dim3(256), 0, st, r);
-    HIP_TRY(hipGetLastError());
-    p.keep_ref2 = ref2;
-    p.keep_flag = flag;
+    const KeepAux aux = aux_in ? *aux_in : keep_aux_of(keep, T, V);
+    if (!aux.ready) {     // (the main launch below overwrites the sample's partials afterwards)
+      rc = keep_prepass(p, hidden, weight, labels, T, H, V, pl.nsplit, pl.part, aux, 1, st);
+      if (rc) return rc;
+    }
+    p.keep_ref2 = aux.ref2;
+    p.keep_flag = aux.flag;
   }
   // One launch per token region: tokens [t0, t0 + count) with `nsplit` vocabulary splits, then their merge.
   auto run_region = [&](int t0, int count, int nsplit, float4* part) -> int {
@@ -973,7 +1001,7 @@ struct KeptBwdSums {
 int kept_bwd_impl(const Tuning& tn, const void* hidden, const void* weight, const void* bias, const int64_t* labels,
                   const float* lse, const float* g, const float* gout_dev, float inv_temp, int T, int H, int V,
                   void* logits_keep, void* dH_out, void* dW_out, void* dbias_out, const KeptBwdSums& sums, void* ws,
-                  size_t ws_bytes, hipStream_t st) {
+                  size_t ws_bytes, hipStream_t st, const KeepAux* aux_in = nullptr) {
   const bool want_dh = dH_out != nullptr, want_dw = dW_out != nullptr || sums.dw_out_f32 != nullptr;
   const bool want_db = dbias_out != nullptr || sums.db_out_f32 != nullptr;
   KeptBwdPlan pl;
@@ -984,13 +1012,14 @@ int kept_bwd_impl(const Tuning& tn, const void* hidden, const void* weight, cons
   const long long blk = (long long)Tpad * 256;
   bf16_t* ek = (bf16_t*)logits_keep;
   const int panel = pl.panel, npanels = pl.npanels;
-  int* flag = keep_flag_of(logits_keep, T, V);
+  const KeepAux aux = aux_in ? *aux_in : keep_aux_of(logits_keep, T, V);
+  int* flag = aux.flag;
   // rows without a gradient (zero advantage, ignored label) are skipped by 256-row tile (dH) and 64-row K step (dW)
   const bool skip_dead = tn.keep_skip_dead != 0 && (T + 63) / 64 <= kLiveMaxChunks;
 
   {
     PhaseScope ph(kPhaseDlogits, st);
-    KeepPrepParams k{ek, blk, keep_ref2_of(logits_keep, T, V), keep_xy_of(logits_keep, T, V), (const long long*)labels, lse, g, gout_dev, inv_temp,
+    KeepPrepParams k{ek, blk, aux.ref2, aux.xy, (const long long*)labels, lse, g, gout_dev, inv_temp,
                      (const bf16_t*)hidden, T, H, V, pl.row_scale, flag};
     hipLaunchKernelGGL(keep_backward_prep_kernel, dim3((T + 3) / 4), dim3(256), 0, st, k);
     HIP_TRY(hipGetLastError());
@@ -1318,6 +1347,11 @@ struct ChunkedPlan {
   float* dw_acc;
   float* db_acc;
   double* partial;
+  // the kept forward's pre-pass, run once for the tokens of every chunk: references, target logits, one overflow
+  // flag per chunk, and the scratch of the pass itself
+  float *ref2, *xy, *pre_xt, *pre_bias32;
+  int* flags;
+  float4* pre_part;
   size_t bytes;
 };
 void plan_chunked(const Tuning& tn, ChunkedPlan& pl, void* ws, int T, int H, int V, int chunk_tokens, bool has_bias,
@@ -1344,6 +1378,12 @@ void plan_chunked(const Tuning& tn, ChunkedPlan& pl, void* ws, int T, int H, int
   pl.dw_acc = (want_dw && pl.nchunks > 1) ? cv.take<float>((size_t)V * H) : nullptr;
   pl.db_acc = (want_db && pl.nchunks > 1) ? cv.take<float>((size_t)V) : nullptr;
   pl.partial = cv.take<double>(2 * (size_t)((T + kLossThreads - 1) / kLossThreads));
+  pl.ref2 = cv.take<float>((size_t)T);
+  pl.xy = cv.take<float>((size_t)T);
+  pl.flags = cv.take<int>((size_t)pl.nchunks);
+  pl.pre_part = cv.take<float4>(2 * (size_t)T);
+  pl.pre_xt = cv.take<float>((size_t)T);
+  pl.pre_bias32 = has_bias ? cv.take<float>((size_t)V) : nullptr;
   pl.bytes = cv.total();
 }
 }  // namespace
@@ -1407,16 +1447,38 @@ int fgrpo_grpo_step_chunked(const void* hidden, const void* weight, const void* 
   lp.loss = loss_out;
   lp.scal = scal_out;
 
+  {
+    // references of the kept numerators for the tokens of every chunk, in one pass before the first chunk
+    PhaseScope ph(kPhaseFwd, st);
+    FwdParams bp;
+    memset(&bp, 0, sizeof(bp));
+    int rc = stage_logit_operands(bp.g, hidden, weight, T, H, V, dtype, false, H, nullptr, nullptr, nullptr, nullptr, st);
+    if (rc) return rc;
+    if (bias) {
+      hipLaunchKernelGGL(to_f32_kernel, dim3((V + 255) / 256), dim3(256), 0, st, bias, 0, pl.pre_bias32, V);
+      HIP_TRY(hipGetLastError());
+    }
+    bp.bias = bias ? pl.pre_bias32 : nullptr;
+    bp.labels = (const long long*)labels;
+    bp.inv_temp = inv_temp;
+    bp.group_t = tn.fwd_group_t > 0 ? tn.fwd_group_t : 1;
+    bp.xt = pl.pre_xt;
+    rc = keep_prepass(bp, hidden, weight, labels, T, H, V, 2, pl.pre_part, KeepAux{pl.ref2, pl.xy, pl.flags, true},
+                      pl.nchunks, st);
+    if (rc) return rc;
+  }
   const size_t esz = sizeof(bf16_t);
   for (int ci = 0; ci < pl.nchunks; ++ci) {
     const int t0 = ci * pl.chunk;
     const int cnt = (T - t0) < pl.chunk ? (T - t0) : pl.chunk;
     const char* h_c = (const char*)hidden + (size_t)t0 * H * esz;
+    const KeepAux aux{pl.ref2 + t0, pl.xy + t0, pl.flags + ci, true};
     int rc;
     {
       PhaseScope ph(kPhaseFwd, st);
       rc = logprob_fwd_impl(h_c, weight, bias, labels + t0, inv_temp, cnt, H, V, dtype, lp_out + t0,
-                            ent_out ? ent_out + t0 : nullptr, lse_out + t0, pl.fwd_ws, pl.fwd_bytes, stream, pl.keep, &tn);
+                            ent_out ? ent_out + t0 : nullptr, lse_out + t0, pl.fwd_ws, pl.fwd_bytes, stream, pl.keep, &tn,
+                            &aux);
     }
     if (rc) return rc;
     {
@@ -1452,7 +1514,7 @@ int fgrpo_grpo_step_chunked(const void* hidden, const void* weight, const void* 
       }
       rc = kept_bwd_impl(tn, h_c, weight, bias, labels + t0, lse_out + t0, g_out + t0, nullptr, inv_temp, cnt, H, V,
                          pl.keep, dH_out ? (char*)dH_out + (size_t)t0 * H * esz : nullptr, dW_out, dbias_out, sums,
-                         pl.bwd_ws, pl.bwd_bytes, st);
+                         pl.bwd_ws, pl.bwd_bytes, st, &aux);
       if (rc) return rc;
     }
   }

@@ -179,13 +179,15 @@ struct KeepRefParams {
   int sample_splits;
   float* ref2;               // [T] out
   float* xy;                 // [T] out: the target's logit x_t[y_t] / temperature (0 for tokens without one)
-  int* flag;                 // cleared here (one int)
+  int* flag;                 // cleared here: nflags ints (one per forward launch that will raise it)
+  int nflags;
 };
 constexpr int kKeepSampleRows = 512;
 
 __global__ __launch_bounds__(256) void keep_reference_kernel(const KeepRefParams p) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (blockIdx.x == 0 && threadIdx.x == 0) *p.flag = 0;
+  if (blockIdx.x == 0)
+    for (int i = threadIdx.x; i < p.nflags; i += 256) p.flag[i] = 0;
   if (t >= p.T) return;
   const long long lab = p.labels[t];
   if (lab < 0 || lab >= p.V) {                 // ignored (-100) or invalid: no gradient, row stored as zeros
@@ -391,11 +393,19 @@ __global__ __launch_bounds__(1024) void keep_live_runs_kernel(const KeepLivePara
   __shared__ int starts_before[1024 + 1], live_before[1024 + 1];
   const int tid = threadIdx.x;
   // chunk flags: one wavefront per chunk, 64 rows each
-  for (int c = tid >> 6; c < p.n_chunks; c += 16) {
-    const int t = c * 64 + (tid & 63);
-    const bool on = t < p.T && p.row_scale[t] != 0.f;
-    const bool any = __builtin_amdgcn_ballot_w64(on) != 0;
-    if ((tid & 63) == 0) live[c] = any ? 1 : 0;
+  // (four chunks per wavefront and round, so that four loads are in flight at a time)
+  for (int c4 = (tid >> 6) * 4; c4 < p.n_chunks; c4 += 64) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = (c4 + k) * 64 + (tid & 63);
+      v[k] = (c4 + k < p.n_chunks && t < p.T) ? p.row_scale[t] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool any = __builtin_amdgcn_ballot_w64(v[k] != 0.f) != 0;
+      if ((tid & 63) == 0 && c4 + k < p.n_chunks) live[c4 + k] = any ? 1 : 0;
+    }
   }
   __syncthreads();
   for (int m = tid; m * 4 < p.n_chunks; m += 1024) {
@@ -410,15 +420,32 @@ __global__ __launch_bounds__(1024) void keep_live_runs_kernel(const KeepLivePara
     nl += live[c];
     ns += live[c] && (c == 0 || !live[c - 1]);
   }
-  starts_before[tid + 1] = ns;
-  live_before[tid + 1] = nl;
-  if (tid == 0) starts_before[0] = live_before[0] = 0;
-  __syncthreads();
-  if (tid == 0) {        // 1024 additions: a serial scan is fine here
-    for (int i = 1; i <= 1024; ++i) {
-      starts_before[i] += starts_before[i - 1];
-      live_before[i] += live_before[i - 1];
+  // inclusive prefix of (ns, nl) over the 1024 threads: shuffles inside the wavefront, the 16 wavefront totals in LDS
+  {
+    int is = ns, il = nl;
+    const int lane = tid & 63, wv = tid >> 6;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int us = __shfl_up(is, d, 64), ul = __shfl_up(il, d, 64);
+      if (lane >= d) {
+        is += us;
+        il += ul;
+      }
     }
+    __shared__ int wave_s[16], wave_l[16];
+    if (lane == 63) {
+      wave_s[wv] = is;
+      wave_l[wv] = il;
+    }
+    __syncthreads();
+    int bs = 0, bl = 0;
+    for (int w = 0; w < wv; ++w) {
+      bs += wave_s[w];
+      bl += wave_l[w];
+    }
+    starts_before[tid + 1] = bs + is;
+    live_before[tid + 1] = bl + il;
+    if (tid == 0) starts_before[0] = live_before[0] = 0;
   }
   __syncthreads();
   const int n_runs = starts_before[1024], n_live = live_before[1024];
