@@ -921,7 +921,7 @@ struct DhSplitPlan {
   int main_tiles;   // == tiles_m: no split
   int ksplit, kchunk;
 };
-constexpr int kDhPartRounds = 3;      // fp32 tiles the split contraction may write: this many per CU
+constexpr int kDhPartRounds = 8;      // fp32 tiles the split contraction may write: this many per CU (the workspace is sized from the plan)
 DhSplitPlan plan_tail_split(int T, int H, int kv) {
   const int tiles_m = (T + 255) / 256, tiles_n = (H + 255) / 256, slots = num_cus(), per_xcd = slots / 8;
   DhSplitPlan d{tiles_m, 1, 0};
@@ -932,8 +932,13 @@ DhSplitPlan plan_tail_split(int T, int H, int kv) {
   const int blocks = (kv + 255) / 256;                         // 256-column blocks of the contraction
   double best = (double)whole_rounds(tiles_m);
   const int full = tiles_m * tiles_n / slots;
-  for (int f = full; f >= 0 && f >= full - 1; --f) {
-    const int main_tiles = 8 * (f * per_xcd / tiles_n);        // whole rounds on every XCD under either raster
+  // candidates: the last partial round alone in pieces (after `full` or `full - 1` whole rounds), or every tile in
+  // pieces - then the launch's work is a whole number of pieces whatever the tile count (T = 16384, H = 3584: 896
+  // tiles = 3.5 rounds, four as whole tiles; as 1792 half contractions seven rounds of half the length)
+  int mains[3] = {8 * (full * per_xcd / tiles_n), full > 0 ? 8 * ((full - 1) * per_xcd / tiles_n) : 0, 0};
+  for (int c = 0; c < 3; ++c) {
+    const int main_tiles = mains[c];
+    if (c > 0 && main_tiles == mains[c - 1]) continue;
     const int tail = (tiles_m - main_tiles) * tiles_n;
     if (tail <= 0) continue;
     for (int ks = 2; ks <= 16 && tail * ks <= kDhPartRounds * slots; ++ks) {

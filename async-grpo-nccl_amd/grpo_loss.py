@@ -419,10 +419,9 @@ def compute_dual_clip_grpo_loss(
     extra = {}
     if ops.COMPACT_MIN_TOKENS <= int(labels.numel()) and \
             0 < int(output_indices.numel()) < ops.COMPACT_MAX_VALID_FRACTION * int(labels.numel()):
-        # output_indices are the rows themselves when every labelled token is an output token (their host-side
-        # counts agree): nothing to count on the device then; otherwise the rows are found from the labels
-        n_host = minibatch.get("_num_output_tokens_non_masked_host", None)
-        extra["compact_masked_tokens"] = output_indices if (n_host is not None and int(n_host) == int(output_indices.numel())) else True
+        # output_indices are the rows themselves when post_process_batch has established, on the host, that they
+        # list exactly the positions with a valid next-token label; otherwise the rows are found from the labels
+        extra["compact_masked_tokens"] = output_indices if minibatch.get("_labels_are_output_tokens", False) else True
     grpo_output = policy_model(
         input_ids=batch_ids,
         attention_mask=minibatch.get("attention_mask", None),

@@ -134,11 +134,16 @@ def get_output_logits_indices(batched_questions, device):
     return ops.output_indices(il, ol, device), ol
 
 
-def get_input_for_logprobs(batched_questions, output_indices, device):
+def get_input_for_logprobs(batched_questions, output_indices, device, info=None):
     """Concatenated ids / position ids / labels as [1, T] int64 device tensors
     (reference: sample_processing_utils.py:114-125).  One pinned staging buffer,
     one copy.  Samples that carry no ``labels`` get them built on the device from
-    ``input_len`` / ``output_len`` (the rule of vllm_worker.py:768-774)."""
+    ``input_len`` / ``output_len`` (the rule of vllm_worker.py:768-774).
+    ``info`` (a dict, optional) receives what is known on the host while the labels
+    are packed: ``num_scored`` (labelled tokens) and ``labels_are_output_tokens``
+    (True when the positions whose next-token label is valid are exactly the
+    output positions of (input_len, output_len) - by construction when the labels
+    are built from those lengths, otherwise checked here on the host copy)."""
     lens = [len(s["sample_ids"]) for s in batched_questions]
     n_tok = sum(lens)
     have_labels = all("labels" in s for s in batched_questions)
@@ -149,12 +154,22 @@ def get_input_for_logprobs(batched_questions, output_indices, device):
     _fill(view[1], batched_questions, "sample_position_ids", lens)
     if have_labels:
         _fill(view[2], batched_questions, "labels", lens)
-        get_input_for_logprobs.last_scored = int(np.count_nonzero(view[2] != -100))
+        if info is not None:
+            info["num_scored"] = int(np.count_nonzero(view[2] != -100))
+            same = False
+            if all("input_len" in s and "output_len" in s for s in batched_questions):
+                il, ol = _lens(batched_questions)
+                # position t is scored when the label of token t + 1 is valid (the last position never is)
+                same = int((il + ol).sum()) == n_tok and \
+                    np.array_equal(np.flatnonzero(view[2][1:] != -100), get_output_logits_indices_numba(il, ol))
+            info["labels_are_output_tokens"] = bool(same)
     dev = host.to(device, non_blocking=True)
     if have_labels:
         return dev[0:1], dev[1:2], dev[2:3]
     il, ol = _lens(batched_questions)
-    get_input_for_logprobs.last_scored = int(ol.sum())
+    if info is not None:
+        info["num_scored"] = int(ol.sum())
+        info["labels_are_output_tokens"] = True
     return dev[0:1], dev[1:2], ops.build_labels(dev[0:1], il, ol)
 
 
@@ -220,7 +235,8 @@ def post_process_batch(batched_questions, device, constant_length_samples=None):
         stage_dev = stage.to(device, non_blocking=True)
         reference_output_logprobs, reference_output_entropies = stage_dev[0], stage_dev[1]
 
-    batch_ids, batch_position_ids, labels = get_input_for_logprobs(batched_questions, output_indices, device)
+    label_info = {}
+    batch_ids, batch_position_ids, labels = get_input_for_logprobs(batched_questions, output_indices, device, label_info)
 
     modified = [q for q in batched_questions if q['modified_reward'] is not None]
     plain = [q for q in batched_questions if q['modified_reward'] is None]
@@ -253,7 +269,10 @@ def post_process_batch(batched_questions, device, constant_length_samples=None):
         "cu_seqlens": cu,
         # not in the reference: the labelled-token count as a host integer (known while the labels are packed), so
         # that the trainer's all-masked check needs no device read
-        "_num_output_tokens_non_masked_host": float(get_input_for_logprobs.last_scored),
+        "_num_output_tokens_non_masked_host": float(label_info["num_scored"]),
+        # not in the reference: whether output_indices lists exactly the positions with a valid next-token label
+        # (then the loss may hand them to the LM head as its row list without looking at the labels again)
+        "_labels_are_output_tokens": bool(label_info["labels_are_output_tokens"]),
     }
     for k, key in enumerate(counters):
         out[key] = counter_vec[k]

@@ -169,8 +169,8 @@ def test_out_of_range_chunk_is_recomputed_on_the_device(dev):
 def test_transient_memory_is_one_chunk(dev):
     """Peak memory beyond the inputs and the outputs (gradients, per-token vectors) is the call's workspace: one
     chunk of kept numerators - 2 * loss_chunksize tokens x V in bf16 - the fp32 dW sum, and per-chunk scratch
-    bounded by the device, not by the batch (fp32 pieces of dHidden's split contraction, at most three 256 x 256
-    tiles per CU = 201 MB; the scaled transposed copy of the chunk's hidden rows)."""
+    bounded by the device, not by the batch (fp32 pieces of dHidden's split contraction, at most eight 256 x 256
+    tiles per CU = 537 MB; the scaled transposed copy of the chunk's hidden rows)."""
     import grpo_loss as G
     from fgrpo import _lib, ops
     w = filling_workload(38, tokens=16384, V=32000)
@@ -195,7 +195,7 @@ def test_transient_memory_is_one_chunk(dev):
     chunk_bytes = 2 * Lc * V * 2
     dw_sum = 4 * V * H
     ws = _lib.load().fgrpo_grpo_step_chunked_workspace(T, H, V, _lib.BF16, chunk)
-    scratch_max = 3 * 256 * 256 * 256 * 4 + 2 * H * (chunk + 192) + (4 << 20)
+    scratch_max = 8 * 256 * 256 * 256 * 4 + 2 * H * (chunk + 192) + (4 << 20)
     assert ws <= 1.01 * chunk_bytes + dw_sum + scratch_max, (ws, chunk_bytes, dw_sum)
     assert peak - outputs <= ws + (8 << 20), (peak, outputs, ws)
     # and far below what keeping the whole batch takes

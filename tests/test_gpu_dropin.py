@@ -350,6 +350,46 @@ def test_training_forward_metrics_and_backward(dev, entropy_coeff):
     assert torch.nn.functional.cosine_similarity(gp.flatten(), cpu_model.model.proj.weight.grad.flatten(), dim=0) > 0.9999
 
 
+def test_labels_that_are_not_the_output_tokens_are_noticed(dev):
+    """Labels that mask some generated tokens and score as many prompt tokens hold the same NUMBER of valid entries
+    as output_indices but not the same positions.  post_process_batch says so (the flag it sets from a host-side
+    comparison), and the loss then finds its rows from the labels instead of taking output_indices for them: the
+    loss equals the oracle's on those labels."""
+    import sample_processing_utils as spu
+    import grpo_loss as G
+    from fgrpo import ops
+    rng = np.random.default_rng(5)
+    V, H = 512, 64
+    samples = []
+    for i in range(40):
+        li, lo = int(rng.integers(20, 60)), int(rng.integers(20, 60))
+        ids = rng.integers(0, V, li + lo).tolist()
+        labels = O.make_labels(ids, li, lo)
+        labels[li], labels[li + 1] = -100, -100           # two generated tokens masked ...
+        labels[3], labels[4] = ids[3], ids[4]             # ... two prompt tokens scored instead
+        samples.append(dict(sample_ids=ids, sample_position_ids=list(range(li + lo)), labels=labels, input_len=li,
+                            output_len=lo, advantage=float(rng.normal()), sample_logprobs=[-6.0] * (li + lo),
+                            sample_entropies=None, reward=1.0, modified_reward=None, delimiter_not_found=False,
+                            truncated_sample=False))
+    batch = spu.post_process_batch(samples, dev)
+    assert batch["_labels_are_output_tokens"] is False
+    assert int(batch["_num_output_tokens_non_masked_host"]) == int(batch["output_indices"].numel())
+    plain = [dict(s, labels=O.make_labels(s["sample_ids"], s["input_len"], s["output_len"])) for s in samples]
+    assert spu.post_process_batch(plain, dev)["_labels_are_output_tokens"] is True
+    assert spu.post_process_batch([{k: v for k, v in s.items() if k != "labels"} for s in plain], dev)["_labels_are_output_tokens"] is True
+
+    model, G = _patched(dev, "training")
+    assert ops.COMPACT_MIN_TOKENS <= batch["labels"].numel()
+    loss, _ = G.compute_dual_clip_grpo_loss(model, batch, 0.2, 0.28, 3.0)
+    import copy
+    cpu_model = copy.deepcopy(model).cpu().float()
+    cb = O.pack_samples(samples)
+    hid = cpu_model.model(input_ids=cb["batch_ids"], position_ids=cb["batch_position_ids"])[0]
+    want = O.grpo_loss_and_entropy(cpu_model.lm_head.weight, None, hid, cb["labels"], 1.0, cb["reference_output_logprobs"],
+                                   cb["advantages"], 0.2, 0.28, 3.0)[0]
+    assert abs(loss.item() - want.item()) <= 2e-4 * max(1.0, abs(want.item()))
+
+
 @pytest.mark.parametrize("n_tok", [3000, 50000, 700000])
 def test_diagnostics_vector_against_direct_sums(dev, n_tok):
     """The 16 sums behind the metric dictionary (reference: grpo_loss.py:408-498), from one work-group for few
