@@ -320,7 +320,8 @@ def test_full_size_through_the_drop_in(dev, name, keep, tokens):
     per-sample token means, cu_seqlens, the configuration's chunk hint), then backward with a non-unit upstream
     scale.  Checked: loss and the four per-token diagnostics against the oracle's objective evaluated on the
     kernel's per-token logprobs; sampled rows of dH and of dW against the closed form with the oracle's per-token
-    gradient; columns of dW summing to zero.  keep: "chunked" = the default, the whole step in token chunks of twice
+    gradient (with every row's soft-max normaliser taken from plain torch, which also pins the kernel's lse on all
+    T rows); columns of dW summing to zero.  keep: "chunked" = the default, the whole step in token chunks of twice
     the configuration's chunk size; True = numerators of the whole batch kept; False = logits recomputed."""
     import grpo_loss as G
     from fgrpo import ops
@@ -365,9 +366,16 @@ def test_full_size_through_the_drop_in(dev, name, keep, tokens):
     safe = shifted[rows].clamp(min=0)
     want_dH = g[rows, None] * (w.weight.float()[safe] - prob @ w.weight.float())
     assert cos(hidden.grad.reshape(T, H)[rows], want_dH) >= COS_MIN
+    # the soft-max normaliser of EVERY row from plain torch (fp32 matmul + logsumexp, a block of rows at a time):
+    # it pins the kernel's lse on all T rows and is what the closed form of the sampled dW rows uses
+    w32 = w.weight.float()
+    lse_ref = torch.empty(T, dtype=torch.float32, device=dev)
+    for a in range(0, T, 2048):
+        lse_ref[a:a + 2048] = torch.logsumexp(hs2[a:a + 2048].float() @ w32.t(), dim=-1)
+    assert (lse - lse_ref).abs().max().item() <= LP_TOL_BF16
     vs = torch.randperm(V, generator=gsel)[:16].to(dev)
     xv = hs2.float() @ w.weight[vs].float().t()
-    coef = g[:, None] * ((shifted[:, None] == vs[None, :]).float() - torch.exp(xv - lse[:, None]))
+    coef = g[:, None] * ((shifted[:, None] == vs[None, :]).float() - torch.exp(xv - lse_ref[:, None]))
     want_dW = coef.t() @ hs2.float()
     assert cos(weight.grad[vs], want_dW) >= COS_MIN
     col = weight.grad.float().sum(0)
