@@ -1454,7 +1454,8 @@ int fgrpo_grpo_step_chunked(const void* hidden, const void* weight, const void* 
 
   {
     // references of the kept numerators for the tokens of every chunk, in one pass before the first chunk
-    PhaseScope ph(kPhaseFwd, st);
+    // (timed with "everything else": the forward brackets then hold one forward launch and its merge each)
+    PhaseScope ph(kPhaseOther, st);
     FwdParams bp;
     memset(&bp, 0, sizeof(bp));
     int rc = stage_logit_operands(bp.g, hidden, weight, T, H, V, dtype, false, H, nullptr, nullptr, nullptr, nullptr, st);

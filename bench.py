@@ -26,8 +26,13 @@ PEAK_CLOCK_MHZ = 2400.0
 # --copy-probe.  Not measured in the run that prints it: the figure belongs to the binary and workload named in the
 # profile summary it cites, and is None for workloads that were not profiled.
 PROFILED_TRAFFIC = {
-    # (workload, path): (bytes per launch of the forward kernel, summary under profiles/)
-    ("cfg1", "whole"): (3.2489e+10, "profiles/lmhead_fwd_kernel_cfg1_traffic_pmc.txt"),
+    # (workload, path): (bytes per launch of the forward kernel, summary under profiles/); a launch of the chunked
+    # path is one token chunk
+    ("cfg1", "chunked"): (8.116e+09, "profiles/lmhead_chunked_step_cfg1_counters_pmc.txt"),
+    ("cfg1", "whole"): (3.256e+10, "profiles/lmhead_whole_batch_kept_cfg1_counters_pmc.txt"),
+    ("cfg2", "chunked"): (3.121e+10, "profiles/lmhead_chunked_step_cfg2_counters_pmc.txt"),
+    ("cfg3", "forward"): (3.387e+11, "profiles/lmhead_fwd_kernel_cfg3_counters_pmc.txt"),
+    ("cfg4", "chunked"): (2.172e+10, "profiles/lmhead_chunked_step_cfg4_counters_pmc.txt"),
 }
 
 
@@ -569,7 +574,8 @@ def main():
             phases.append(phase("gemm_store_kernel dHidden", phase_ms["dh"], phase_n["dh"], steps, thv))
             phases.append(phase("gemm_store_kernel dW" + (" (fp32 sum across chunks)" if path == "chunked" and n_chunks > 1 else ""),
                                 phase_ms["dw"], phase_n["dw"], steps, thv))
-            phases.append(phase("objective, normalisers, upstream scale, bias sums", phase_ms["other"], phase_n["other"], steps, 0.0))
+            phases.append(phase("everything else inside the library calls (chunked: reference pre-pass of the kept numerators, objective kernels; bias sums)",
+                                phase_ms["other"], phase_n["other"], steps, 0.0))
         alg = (1.0 if fwd_only else 3.0) * thv
         res = {"path": path, **path_notes[path], "steps": steps, "warmup": warmup, "ms_per_step": ms,
                "ms_per_step_median": per_step[len(per_step) // 2], "ms_per_step_min": per_step[0],
