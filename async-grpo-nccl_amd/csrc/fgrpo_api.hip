@@ -922,9 +922,10 @@ struct DhSplitPlan {
   int ksplit, kchunk;
 };
 constexpr int kDhPartRounds = 8;      // fp32 tiles the split contraction may write: this many per CU (the workspace is sized from the plan)
-DhSplitPlan plan_tail_split(int T, int H, int kv) {
+DhSplitPlan plan_tail_split(int T, int H, int kv, double* rounds_out = nullptr) {
   const int tiles_m = (T + 255) / 256, tiles_n = (H + 255) / 256, slots = num_cus(), per_xcd = slots / 8;
   DhSplitPlan d{tiles_m, 1, 0};
+  if (rounds_out) *rounds_out = (double)(((long long)tiles_m * tiles_n + slots - 1) / slots);
   if (H % 4 != 0 || tiles_n > per_xcd) return d;
   // time in device rounds of whole tiles.  Whole-tile launches deal row tiles round-robin to the 8 XCDs (or hand
   // each a contiguous range): an XCD runs its share x tiles_n work-groups on slots / 8 CUs.
@@ -954,6 +955,7 @@ DhSplitPlan plan_tail_split(int T, int H, int kv) {
       }
     }
   }
+  if (rounds_out) *rounds_out = best;
   return d;
 }
 // Row length of the scaled, transposed copy of hidden: the padded token count plus 192 elements.  Rows 2 * Tpad bytes
@@ -1330,15 +1332,40 @@ int fgrpo_loss_prepare(const int64_t* labels, const int32_t* cu, int nseq, int T
 }
 
 namespace {
-// Token chunk of the chunked step: the caller's bound rounded to whole 256-token tiles, then the tokens dealt evenly
-// over the chunks that bound needs (a last chunk of a few hundred tokens would pay whole passes over the dW sum).
-int fused_chunk_tokens(int T, int chunk_tokens) {
+// Token chunk of the chunked step.  The caller's bound is rounded down to whole 256-token tiles; under it two ways of
+// cutting T tokens are weighed: the tokens dealt evenly over the chunks the bound needs, or whole chunks of the bound
+// and one shorter chunk for the rest.  What decides is how the chunks' tile counts fall on the device: T = 33000 is
+// 129 token tiles; five chunks of 26 give the forward 26 x 9 = 234 work-groups per launch (a tenth of the CUs idle,
+// measured 38.1 ms/step), four chunks of 32 and one of a single tile run the four at the full-device shape.  The
+// estimate counts K steps of 64 per CU: a forward tile H / 64 + its epilogue, a dHidden round V / 64 (in pieces
+// where plan_tail_split says so), a dW tile tokens / 64 + the read-modify-write of its fp32 sums.
+double chunk_cost_estimate(int cnt, int H, int V) {
+  const int slots = num_cus();
+  const int tiles_t = (cnt + 255) / 256, tiles_v = (V + 255) / 256, tiles_h = (H + 255) / 256;
+  const int prefer = (16384LL * H * 2 > (192LL << 20)) ? 8 : 4;
+  const int ns = choose_nsplit(tiles_t, tiles_v, slots, 0, prefer);
+  const double fwd = (double)split_cost(tiles_t, tiles_v, slots, ns) * (H / 64.0 + 5.0);
+  double dh_rounds = 0.0;
+  (void)plan_tail_split(cnt, H, (int)round_up(V, 256), &dh_rounds);
+  const double dh = dh_rounds * (round_up(V, 256) / 64.0 + 8.0);
+  const double dw = (double)(((long long)tiles_v * tiles_h + slots - 1) / slots) * (round_up(cnt, 256) / 64.0 + 12.0);
+  return fwd + dh + dw + 40.0;     // + the small launches of a chunk
+}
+int fused_chunk_tokens(const Tuning& tn, int T, int H, int V, int chunk_tokens) {
   long long c = chunk_tokens > 0 ? chunk_tokens : 8192;
   c = c / 256 * 256;
   if (c < 256) c = 256;
   if (c >= T) return (int)round_up(T, 256);
   const long long n = (T + c - 1) / c;
-  return (int)round_up((T + n - 1) / n, 256);
+  const int even = (int)round_up((T + n - 1) / n, 256);
+  if (even == c || H <= 0 || V <= 0) return even;
+  const int rest_c = T - (int)(T / c * c);
+  if (rest_c > 0 && !keep_supported(tn, rest_c, H, V, FGRPO_BF16)) return even;   // a short last chunk the kernels would refuse
+  auto total = [&](int chunk) {
+    const int full = T / chunk, rest = T - full * chunk;
+    return full * chunk_cost_estimate(chunk, H, V) + (rest > 0 ? chunk_cost_estimate(rest, H, V) : 0.0);
+  };
+  return total((int)c) < total(even) ? (int)c : even;
 }
 
 struct ChunkedPlan {
@@ -1361,7 +1388,7 @@ struct ChunkedPlan {
 };
 void plan_chunked(const Tuning& tn, ChunkedPlan& pl, void* ws, int T, int H, int V, int chunk_tokens, bool has_bias,
                   bool want_dh, bool want_dw, bool want_db) {
-  pl.chunk = fused_chunk_tokens(T, chunk_tokens);
+  pl.chunk = fused_chunk_tokens(tn, T, H, V, chunk_tokens);
   pl.nchunks = (T + pl.chunk - 1) / pl.chunk;
   const int last = T - (pl.nchunks - 1) * pl.chunk;
   pl.keep_bytes = keep_bytes(pl.chunk < T ? pl.chunk : T, V);
@@ -1397,7 +1424,7 @@ namespace {
 // every chunk - the full ones and the shorter last one - must be a problem the kept-numerators pair handles
 bool chunked_supported(const Tuning& tn, int T, int H, int V, int dtype, int chunk_tokens) {
   if (T <= 0 || H <= 0 || V <= 0) return false;
-  const int chunk = fused_chunk_tokens(T, chunk_tokens);
+  const int chunk = fused_chunk_tokens(tn, T, H, V, chunk_tokens);
   const int nchunks = (T + chunk - 1) / chunk;
   const int last = T - (nchunks - 1) * chunk;
   return keep_supported(tn, chunk < T ? chunk : T, H, V, dtype) && keep_supported(tn, last, H, V, dtype);
@@ -1408,9 +1435,9 @@ int fgrpo_grpo_step_chunked_supported(int T, int H, int V, int dtype, int chunk_
   return chunked_supported(g_tune, T, H, V, dtype, chunk_tokens) ? 1 : 0;
 }
 
-int fgrpo_grpo_step_chunk_tokens(int T, int chunk_tokens) {
-  if (T <= 0) return fail(FGRPO_ERR_BAD_ARG, "grpo_step_chunk_tokens: T=%d", T);
-  return fused_chunk_tokens(T, chunk_tokens);
+int fgrpo_grpo_step_chunk_tokens(int T, int H, int V, int chunk_tokens) {
+  if (T <= 0 || H <= 0 || V <= 0) return fail(FGRPO_ERR_BAD_ARG, "grpo_step_chunk_tokens: T=%d H=%d V=%d", T, H, V);
+  return fused_chunk_tokens(g_tune, T, H, V, chunk_tokens);
 }
 
 size_t fgrpo_grpo_step_chunked_workspace(int T, int H, int V, int dtype, int chunk_tokens) {

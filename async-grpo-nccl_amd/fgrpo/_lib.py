@@ -45,7 +45,7 @@ SIGNATURES = {
     "fgrpo_loss_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _f, _f, _i, _d,
                             _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgrpo_loss_prepare": (_i, [_vp, _vp, _i, _i, _i, _d, _vp, _vp, _vp, _vp]),
-    "fgrpo_grpo_step_chunk_tokens": (_i, [_i, _i]),
+    "fgrpo_grpo_step_chunk_tokens": (_i, [_i, _i, _i, _i]),
     "fgrpo_grpo_step_chunked_supported": (_i, [_i, _i, _i, _i, _i]),
     "fgrpo_grpo_step_chunked_workspace": (_sz, [_i, _i, _i, _i, _i]),
     "fgrpo_grpo_step_chunked": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _f, _f, _f, _f, _i,

@@ -596,10 +596,11 @@ def chunk_bound_for(V: int, loss_chunksize: Optional[int] = None) -> int:
     return max(256, min(bound, by_bytes) // 256 * 256)
 
 
-def chunk_tokens_for(T: int, V: int, loss_chunksize: Optional[int] = None) -> int:
-    """Token chunk the chunked step uses for a packed batch of T tokens: the bound, then the tokens dealt evenly over
-    the chunks that bound needs (whole 256-token tiles)."""
-    return int(_lib.load().fgrpo_grpo_step_chunk_tokens(int(T), chunk_bound_for(V, loss_chunksize)))
+def chunk_tokens_for(T: int, H: int, V: int, loss_chunksize: Optional[int] = None) -> int:
+    """Token chunk the chunked step uses for a packed batch of T tokens: under the bound, either the tokens dealt
+    evenly over the chunks the bound needs or whole chunks of the bound and a shorter last one (whole 256-token
+    tiles; the library picks by how the tile counts fill the device)."""
+    return int(_lib.load().fgrpo_grpo_step_chunk_tokens(int(T), int(H), int(V), chunk_bound_for(V, loss_chunksize)))
 
 
 def _want_keep(T: int, H: int, V: int, dtype, needs_grad: bool, keep_logits=None) -> bool:

@@ -476,7 +476,7 @@ def main():
         return out
 
     # Which way to the gradients each timed path takes (fgrpo.ops.KEEP_LOGITS); the headline is the default.
-    chunk_tok = ops.chunk_tokens_for(T, V, chunk_arg)
+    chunk_tok = ops.chunk_tokens_for(T, H, V, chunk_arg)
     chunked_ok = (not fwd_only) and ops.chunked_supported(T, H, V, w.dtype, chunk_tok)
     whole_ok = (not fwd_only) and ops.keep_supported(T, H, V, w.dtype)
     headline = {"auto": "chunked" if chunked_ok else "recompute", "chunked": "chunked", "on": "whole", "whole": "whole",
@@ -487,7 +487,7 @@ def main():
     lib = ops._lib.load()
     path_notes = {
         "chunked": {"never_holds_T_x_V": True, "executed_products": 3,
-                    "what": f"the whole step in {n_chunks} token chunks of {chunk_tok}: forward keeping one chunk of bf16 soft-max "
+                    "what": f"the whole step in {n_chunks} token chunks of {chunk_tok}" + (f" (the last one {T - (n_chunks - 1) * chunk_tok})" if T % chunk_tok else "") + ": forward keeping one chunk of bf16 soft-max "
                             "numerators, objective, dHidden rows, dW summed in fp32 across chunks; backward() scales by the upstream scalar",
                     "transient_bytes": int(lib.fgrpo_grpo_step_chunked_workspace(T, H, V, ops._lib.BF16, chunk_tok)) if chunked_ok else None,
                     "transient_of_which_kept_numerators_bytes": int(ops.logits_keep_bytes(min(T, chunk_tok), V)) if chunked_ok else None,

@@ -190,7 +190,7 @@ def test_transient_memory_is_one_chunk(dev):
     torch.cuda.synchronize()
     peak = torch.cuda.max_memory_allocated(dev) - base
     outputs = 2 * T * H + 2 * V * H + 16 * 4 * T            # dH, dW, the per-token vectors
-    chunk = ops.chunk_tokens_for(T, V, Lc)
+    chunk = ops.chunk_tokens_for(T, H, V, Lc)
     assert chunk == 2 * Lc
     chunk_bytes = 2 * Lc * V * 2
     dw_sum = 4 * V * H
