@@ -5,8 +5,10 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <initializer_list>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "host_common.h"
 #include "prep_kernels.h"
@@ -1331,13 +1333,15 @@ int fgrpo_loss_prepare(const int64_t* labels, const int32_t* cu, int nseq, int T
   return 0;
 }
 
+extern "C++" {
 namespace {
-// Token chunk of the chunked step.  The caller's bound is rounded down to whole 256-token tiles; under it two ways of
-// cutting T tokens are weighed: the tokens dealt evenly over the chunks the bound needs, or whole chunks of the bound
-// and one shorter chunk for the rest.  What decides is how the chunks' tile counts fall on the device: T = 33000 is
-// 129 token tiles; five chunks of 26 give the forward 26 x 9 = 234 work-groups per launch (a tenth of the CUs idle,
-// measured 38.1 ms/step), four chunks of 32 and one of a single tile run the four at the full-device shape.  The
-// estimate counts K steps of 64 per CU: a forward tile H / 64 + its epilogue, a dHidden round V / 64 (in pieces
+// Token chunks of the chunked step.  The caller's bound is rounded down to whole 256-token tiles; under it three ways
+// of cutting T tokens are weighed: the tokens dealt evenly over the chunks the bound needs; whole chunks of the bound
+// and one shorter chunk for the rest; or whole chunks, with the last of them and the rest dealt evenly over two.
+// What decides is how the chunks' tile counts fall on the device: T = 33000 is 129 token tiles; five chunks of 26 give
+// the forward 26 x 9 = 234 work-groups per launch (a tenth of the CUs idle, measured 38.1 ms/step); four chunks of 32
+// run at the full-device shape but leave one tile that pays a whole pass over the dW sums (36.5 ms); three of 32 and
+// two of 17 and 16 avoid both.  The estimate counts K steps of 64 per CU: a forward tile H / 64 + its epilogue, a dHidden round V / 64 (in pieces
 // where plan_tail_split says so), a dW tile tokens / 64 + the read-modify-write of its fp32 sums.
 double chunk_cost_estimate(int cnt, int H, int V) {
   const int slots = num_cus();
@@ -1351,25 +1355,61 @@ double chunk_cost_estimate(int cnt, int H, int V) {
   const double dw = (double)(((long long)tiles_v * tiles_h + slots - 1) / slots) * (round_up(cnt, 256) / 64.0 + 12.0);
   return fwd + dh + dw + 40.0;     // + the small launches of a chunk
 }
-int fused_chunk_tokens(const Tuning& tn, int T, int H, int V, int chunk_tokens) {
+// The chunks of a call, in token order (every size but the last a multiple of 256, none above the bound).
+std::vector<int> chunk_sizes(const Tuning& tn, int T, int H, int V, int chunk_tokens) {
   long long c = chunk_tokens > 0 ? chunk_tokens : 8192;
   c = c / 256 * 256;
   if (c < 256) c = 256;
-  if (c >= T) return (int)round_up(T, 256);
-  const long long n = (T + c - 1) / c;
+  if (c >= T) return std::vector<int>(1, T);
+  const int n = (int)((T + c - 1) / c);
   const int even = (int)round_up((T + n - 1) / n, 256);
-  if (even == c || H <= 0 || V <= 0) return even;
-  const int rest_c = T - (int)(T / c * c);
-  if (rest_c > 0 && !keep_supported(tn, rest_c, H, V, FGRPO_BF16)) return even;   // a short last chunk the kernels would refuse
-  auto total = [&](int chunk) {
-    const int full = T / chunk, rest = T - full * chunk;
-    return full * chunk_cost_estimate(chunk, H, V) + (rest > 0 ? chunk_cost_estimate(rest, H, V) : 0.0);
+  auto cut = [&](int chunk, int nfull, std::initializer_list<int> tail) {
+    std::vector<int> v((size_t)nfull, chunk);
+    for (int t : tail)
+      if (t > 0) v.push_back(t);
+    return v;
   };
-  return total((int)c) < total(even) ? (int)c : even;
+  std::vector<std::vector<int>> cand;
+  cand.push_back(cut(even, (T - 1) / even, {T - (T - 1) / even * even}));          // the tokens dealt evenly
+  const int full = (int)(T / c), rest = T - full * (int)c;
+  if (even != c && H > 0 && V > 0) {
+    cand.push_back(cut((int)c, full, {rest}));                                       // whole chunks and the rest
+    if (rest > 0 && full >= 1) {                                                     // ... or the last whole chunk and the rest, halved
+      const int h1 = (int)round_up(((int)c + rest + 1) / 2, 256);
+      cand.push_back(cut((int)c, full - 1, {h1, (int)c + rest - h1}));
+    }
+  }
+  size_t best = 0;
+  double best_cost = -1.0;
+  for (size_t i = 0; i < cand.size(); ++i) {
+    bool ok = true;
+    double cost = 0.0;
+    int prev = -1;
+    double prev_cost = 0.0;
+    for (int sz : cand[i]) {
+      if (sz != prev) {
+        ok = ok && (i == 0 || keep_supported(tn, sz, H, V, FGRPO_BF16));   // a chunk the kernels would refuse rules a cut out
+        prev_cost = (H > 0 && V > 0) ? chunk_cost_estimate(sz, H, V) : 0.0;
+        prev = sz;
+      }
+      cost += prev_cost;
+    }
+    if (ok && (best_cost < 0.0 || cost < best_cost)) {
+      best_cost = cost;
+      best = i;
+    }
+  }
+  return cand[best];
+}
+int fused_chunk_tokens(const Tuning& tn, int T, int H, int V, int chunk_tokens) {
+  int m = 0;
+  for (int sz : chunk_sizes(tn, T, H, V, chunk_tokens)) m = sz > m ? sz : m;
+  return (int)round_up(m, 256);
 }
 
 struct ChunkedPlan {
-  int chunk, nchunks;
+  std::vector<int> sizes;   // tokens of each chunk, in order
+  int chunk, nchunks;       // the largest chunk (whole tiles); number of chunks
   void* keep;
   size_t keep_bytes;
   void* fwd_ws;
@@ -1388,12 +1428,16 @@ struct ChunkedPlan {
 };
 void plan_chunked(const Tuning& tn, ChunkedPlan& pl, void* ws, int T, int H, int V, int chunk_tokens, bool has_bias,
                   bool want_dh, bool want_dw, bool want_db) {
-  pl.chunk = fused_chunk_tokens(tn, T, H, V, chunk_tokens);
-  pl.nchunks = (T + pl.chunk - 1) / pl.chunk;
-  const int last = T - (pl.nchunks - 1) * pl.chunk;
-  pl.keep_bytes = keep_bytes(pl.chunk < T ? pl.chunk : T, V);
+  pl.sizes = chunk_sizes(tn, T, H, V, chunk_tokens);
+  pl.nchunks = (int)pl.sizes.size();
+  pl.chunk = 0;
+  for (int sz : pl.sizes) pl.chunk = sz > pl.chunk ? sz : pl.chunk;
+  pl.keep_bytes = keep_bytes(pl.chunk, V);
   pl.fwd_bytes = pl.bwd_bytes = 0;
-  for (int cnt : {pl.chunk < T ? pl.chunk : T, last}) {
+  int prev = -1;
+  for (int cnt : pl.sizes) {
+    if (cnt == prev) continue;
+    prev = cnt;
     Tuning tf = tn;
     tf.fwd_variant = 8;
     FwdPlan fp;
@@ -1419,15 +1463,15 @@ void plan_chunked(const Tuning& tn, ChunkedPlan& pl, void* ws, int T, int H, int
   pl.bytes = cv.total();
 }
 }  // namespace
+}  // extern "C++"
 
 namespace {
 // every chunk - the full ones and the shorter last one - must be a problem the kept-numerators pair handles
 bool chunked_supported(const Tuning& tn, int T, int H, int V, int dtype, int chunk_tokens) {
   if (T <= 0 || H <= 0 || V <= 0) return false;
-  const int chunk = fused_chunk_tokens(tn, T, H, V, chunk_tokens);
-  const int nchunks = (T + chunk - 1) / chunk;
-  const int last = T - (nchunks - 1) * chunk;
-  return keep_supported(tn, chunk < T ? chunk : T, H, V, dtype) && keep_supported(tn, last, H, V, dtype);
+  for (int sz : chunk_sizes(tn, T, H, V, chunk_tokens))
+    if (!keep_supported(tn, sz, H, V, dtype)) return false;
+  return true;
 }
 }  // namespace
 
@@ -1501,9 +1545,10 @@ int fgrpo_grpo_step_chunked(const void* hidden, const void* weight, const void* 
     if (rc) return rc;
   }
   const size_t esz = sizeof(bf16_t);
+  std::vector<int> first(pl.sizes.size(), 0);          // first token of each chunk
+  for (size_t i = 1; i < first.size(); ++i) first[i] = first[i - 1] + pl.sizes[i - 1];
   for (int ci = 0; ci < pl.nchunks; ++ci) {
-    const int t0 = ci * pl.chunk;
-    const int cnt = (T - t0) < pl.chunk ? (T - t0) : pl.chunk;
+    const int t0 = first[ci], cnt = pl.sizes[ci];
     const char* h_c = (const char*)hidden + (size_t)t0 * H * esz;
     const KeepAux aux{pl.ref2 + t0, pl.xy + t0, pl.flags + ci, true};
     int rc;

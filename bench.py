@@ -483,11 +483,11 @@ def main():
                 "off": "recompute", "recompute": "recompute"}[args.keep_logits]
     if fwd_only:
         headline = "forward"
-    n_chunks = (T + chunk_tok - 1) // chunk_tok if chunked_ok else 1
+    n_chunks = (T + chunk_tok - 1) // chunk_tok if chunked_ok else 1      # (the library may cut the last two chunks evenly)
     lib = ops._lib.load()
     path_notes = {
         "chunked": {"never_holds_T_x_V": True, "executed_products": 3,
-                    "what": f"the whole step in {n_chunks} token chunks of {chunk_tok}" + (f" (the last one {T - (n_chunks - 1) * chunk_tok})" if T % chunk_tok else "") + ": forward keeping one chunk of bf16 soft-max "
+                    "what": f"the whole step in {n_chunks} token chunks of at most {chunk_tok}: forward keeping one chunk of bf16 soft-max "
                             "numerators, objective, dHidden rows, dW summed in fp32 across chunks; backward() scales by the upstream scalar",
                     "transient_bytes": int(lib.fgrpo_grpo_step_chunked_workspace(T, H, V, ops._lib.BF16, chunk_tok)) if chunked_ok else None,
                     "transient_of_which_kept_numerators_bytes": int(ops.logits_keep_bytes(min(T, chunk_tok), V)) if chunked_ok else None,

@@ -196,10 +196,11 @@ int fgrpo_loss_fwd(const float* lp, const float* old_lp, const float* ref_lp, co
  * (x[i] *= *scale_dev for n elements of `dtype`; a scale of exactly 1 returns without touching the array).
  * Executed matrix work: 6 T H V (the reference's own three products), against 8 T H V for the recomputing pair;
  * transient: fgrpo_logits_keep_bytes(chunk, V) + the fp32 dW sum (V x H x 4 bytes, only with more than one chunk).
- * chunk_tokens <= 0: 8192.  The chunk used is fgrpo_grpo_step_chunk_tokens(T, H, V, chunk_tokens): the bound rounded
- * down to whole 256-token tiles, then either the tokens dealt evenly over ceil(T / bound) chunks or whole chunks of
- * the bound and a shorter last one, whichever fills the device better (an estimate from the tile counts; it depends
- * on the arguments only).  Results do not depend on the
+ * chunk_tokens <= 0: 8192.  No chunk exceeds the bound (rounded down to whole 256-token tiles); under it the tokens
+ * are dealt evenly over ceil(T / bound) chunks, or cut into whole chunks of the bound and a shorter last one, or into
+ * whole chunks with the last of them and the rest dealt over two - whichever fills the device best (an estimate from
+ * the tile counts; it depends on the arguments only).  fgrpo_grpo_step_chunk_tokens(T, H, V, chunk_tokens) returns
+ * the largest chunk of the call (whole tiles): what the kept-numerator buffer is sized for.  Results do not depend on the
  * chunk size beyond fp32 summation order (of a token's vocabulary partial sums, whose split follows the token count
  * of a launch, and of dW across chunks): two calls with the same chunk size are bit-identical.
  * old_lp / ref_lp / tokw may be NULL (ratio 1 / no KL term / token mean); kl_beta as in fgrpo_loss_fwd.  Outputs as
