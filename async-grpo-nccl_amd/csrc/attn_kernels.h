@@ -679,6 +679,464 @@ __global__ __launch_bounds__(256) void varlen_attn_dkv_kernel(AttnParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// dK, dV with two wavefronts per SIMD: grid (Hkv, ceil(T/128)), 512 threads.  The same walk and the same arithmetic,
+// in the same order, as varlen_attn_dkv_kernel (results are bit-identical); the work of a 32-key wavefront is
+// dealt to a PAIR of wavefronts (w, w + 4: one SIMD) so that each fits 256 registers:
+//   role A (w < 4) holds the K rows:  S = Q K^T, P = exp(S * scale - lse)        -> P (fp32) to its partner through LDS
+//   role B         holds the V rows:  dP = dO V^T, dS = P * (dP - delta) / scale  -> dS (bf16 operand) to its partner
+// and each owns one half of the head dimension of BOTH accumulators (dV += P^T dO, dK += dS^T Q), so no product is
+// computed twice and the Q / dO tiles are read from LDS exactly as often as by the single wavefront.
+// The sub-blocks of 32 queries (all steps of all query heads of the group, one sequence n = 0, 1, ..) run as a
+// software pipeline with ONE barrier per sub-block; between barriers n - 1 and n
+//   A:  S(n) and dK_A(n - 2) interleaved (dS(n - 2) came from the partner an interval ago);  P(n) -> LDS;  dV_A(n)
+//   B:  P(n - 1) from LDS, dS(n - 1) -> LDS;  dV_B(n - 1), dK_B(n - 1) and dP(n) interleaved
+// so that each wavefront has 16 matrix instructions and its share of the softmax arithmetic in every interval, A
+// starting with the former and B with the latter: the partner's matrix instructions run under a wavefront's vector
+// arithmetic, which a lone wavefront per SIMD cannot have.  P and dS have two LDS slots each (written for one
+// sub-block while the previous one is read); the Q / dO tiles and the per-query scalars have three buffers (the
+// tile before the current one is still read, the next one is being written).
+// Tiles travel global -> LDS directly (buffer_load ... lds, rows past the end of the queries read as zero), a step
+// ahead; every LDS access of the loop is inline assembly with its own counted waits (the compiler would otherwise
+// wait for the tile loads in flight at each LDS access it can see, and streams fragments one per matrix
+// instruction when left to schedule them).  The barriers are bare s_barrier instructions behind a wait for the
+// wavefront's own LDS traffic.  Every wavefront passes every barrier (steps outside a pair's query range skip the
+// arithmetic only).
+// ---------------------------------------------------------------------------------------------------------
+template <int HD>
+constexpr int kAttnDkv2Lds = 3 * 2 * kAttnBK * HD * 2 + 2 * 4 * 64 * 64 + 2 * 4 * 64 * 32 + 3 * 4 * kAttnBK * 4;
+
+template <int OFF>
+__device__ __forceinline__ u32x4_t lds_read_u128_asm(uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "DS offset field");
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ void lds_write_u128_asm(uint32_t addr, u32x4_t v) {
+  static_assert(OFF >= 0 && OFF < 65536, "DS offset field");
+  asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(v), "i"(OFF) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void lds_write_u32_asm(uint32_t addr, uint32_t v) {
+  static_assert(OFF >= 0 && OFF < 65536, "DS offset field");
+  asm volatile("ds_write_b32 %0, %1 offset:%2" : : "v"(addr), "v"(v), "i"(OFF) : "memory");
+}
+
+template <int HD>
+__global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
+  constexpr int KS = HD / 16, DB = HD / 32, DH = DB / 2, kAttnTile = kAttnBK * HD * 2, kHD = HD;
+  constexpr int RPI = 1024 / (HD * 2);                 // tile rows one direct-to-LDS instruction fills (64 lanes x 16 bytes)
+  constexpr int NLD = kAttnBK / RPI / 8;               // such instructions per wavefront and tile
+  constexpr int kRows = 4 * kAttnBK * 4;               // bytes of a buffer of per-query scalars: lse2 | delta | lo | hi
+  constexpr int kXp = 3 * 2 * kAttnTile;               // P, fp32: [slot][pair][4][64 lanes] x 16 bytes
+  constexpr int kXd = kXp + 2 * 4 * 64 * 64;           // dS, bf16 operands: [slot][pair][2][64 lanes] x 16 bytes
+  constexpr int kRw = kXd + 2 * 4 * 64 * 32;           // [buffer][lse2 | delta | lo | hi][64]
+  static_assert(kRw + 3 * kRows == kAttnDkv2Lds<HD>, "LDS layout");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const uint32_t lds0 = lds_addr(smem);
+  const int lane = threadIdx.x & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pw = wave & 3;                             // the pair's 32 keys
+  const bool role_a = wave < 4;
+  const int dh = role_a ? 0 : DH;                      // first 32-column block of this wavefront's half
+  const int hkv = blockIdx.x, G = p.Hq / p.Hkv;
+  const int k0 = min(max(p.order_k[blockIdx.y], 0), (int)gridDim.y - 1) * kAttnBQ;   // clamped: the list may come from the caller
+  const int key = k0 + 32 * pw + (lane & 31);
+  const bool valid = key < p.T;
+  const int last = (k0 + kAttnBQ - 1 < p.T ? k0 + kAttnBQ - 1 : p.T - 1);
+  const int q_begin = max(__builtin_amdgcn_readfirstlane(p.causal ? k0 : p.seg_start[k0]), 0);   // work-group-uniform loop bounds, inside [0, T]
+  const int q_end = min(__builtin_amdgcn_readfirstlane(p.seg_end[last]), p.T);
+  const int wfirst = k0 + 32 * pw, wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = wfirst < p.T;
+  const int wq_lo = wave_on ? (p.causal ? wfirst : p.seg_start[wfirst]) : 1;   // first / last query of interest
+  const int wq_hi = wave_on ? p.seg_end[wlast] - 1 : 0;
+
+  // per-lane LDS offsets: row fragments as in attn_lane, transposing fragments for this wavefront's half only
+  uint32_t rowc[KS], trh[DH][2];
+  {
+    const int g1 = (lane >> 4) & 1, j = lane & 15, r = lane & 31;
+#pragma unroll
+    for (int st = 0; st < KS; ++st) rowc[st] = r * (HD * 2) + (((2 * st + h) ^ attn_swz<HD>(r)) << 4);
+#pragma unroll
+    for (int nb = 0; nb < DH; ++nb)
+#pragma unroll
+      for (int rd = 0; rd < 2; ++rd) {
+        const int row = 4 * h + (j >> 2) + 8 * rd;
+        const int chunk = 4 * (dh + nb) + 2 * g1 + ((j & 3) >> 1);
+        trh[nb][rd] = row * (HD * 2) + ((chunk ^ attn_swz<HD>(row)) << 4) + 8 * (j & 1);
+      }
+  }
+  const uint32_t xp = lds0 + kXp + pw * (64 * 64) + lane * 16;      // + slot * 16384 + grp * 1024
+  const uint32_t xd = lds0 + kXd + pw * (64 * 32) + lane * 16;      // + slot * 8192 + s2 * 1024
+  const uint32_t rwl = lds0 + kRw + h * 16;                         // + buffer * kRows + array * 256 + (32 mq + 8 grp) * 4
+
+  // the lane's own K row (role A) or V row (role B) as the operand of the score products
+  bf16x8_t of[KS];
+  attn_row_operand(of, role_a ? p.k + (long long)(valid ? key : 0) * p.k_st + (long long)hkv * p.k_sh
+                              : p.v + (long long)(valid ? key : 0) * p.v_st + (long long)hkv * p.v_sh, valid, h);
+  const float c = p.scale * kLog2e;
+
+  f32x16_t acc_k[DH], acc_v[DH];
+#pragma unroll
+  for (int nb = 0; nb < DH; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_k[nb][r] = acc_v[nb][r] = 0.f;
+
+  // tile fetch, global -> LDS: instruction i of this wavefront fills tile rows (8 i + wave) * RPI .. + RPI - 1; lane l
+  // lands at 16 l of that KiB, i.e. row l / (HD/8), chunk slot l % (HD/8) - so it fetches the chunk the swizzle
+  // puts there
+  const long long do_st = (long long)p.Hq * kHD;
+  uint32_t foq[NLD], fod[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    const int row = (8 * i + wave) * RPI + lane / (HD / 8), ch = (lane % (HD / 8)) ^ attn_swz<HD>(row);
+    foq[i] = (uint32_t)(((long long)row * p.q_st + ch * 8) * 2);
+    fod[i] = (uint32_t)(((long long)row * do_st + ch * 8) * 2);
+  }
+
+  // tiles in walking order: query head g = 0 .. G-1, inside it the 64-query steps from q_begin to q_end
+  const int nsteps = q_end > q_begin ? (q_end - q_begin + kAttnBK - 1) / kAttnBK : 0;
+  const int NT = nsteps * G;
+  int f_g = 0, f_qb = q_begin;                 // the tile the next fetch brings
+  // raw values of the tile's per-query scalars, as fetched (nothing is computed from them until publish(): an
+  // instruction that touches them would wait for the tile loads issued before them too - the memory counter retires in order)
+  float r_lse = 0.f, r_dl = 0.f;
+  int r_lo = 0, r_end = 0, r_t = 0;
+  auto fetch_next = [&](int buf) {             // tile -> LDS buffer buf (in flight until publish()), its scalars -> registers
+    const int hq = hkv * G + f_g;
+    const bf16_t* qbase = p.q + (long long)hq * p.q_sh;
+    const bf16_t* dobase = p.dout + (long long)hq * kHD;
+    const long long rows = (long long)q_end - f_qb;
+    long long bq = rows > 0 ? (rows - 1) * p.q_st * 2 + HD * 2 : 0, bd = rows > 0 ? (rows - 1) * do_st * 2 + HD * 2 : 0;
+    if (bq > 0xffffffffLL) bq = 0xffffffffLL;
+    if (bd > 0xffffffffLL) bd = 0xffffffffLL;
+    const __amdgpu_buffer_rsrc_t rsq = make_rsrc(qbase + (long long)f_qb * p.q_st, (uint32_t)bq);
+    const __amdgpu_buffer_rsrc_t rsd = make_rsrc(dobase + (long long)f_qb * do_st, (uint32_t)bd);
+    char* qt = smem + buf * 2 * kAttnTile + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsq, FGRPO_LDS_PTR(qt + i * 8192), 16, (int)foq[i], 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsd, FGRPO_LDS_PTR(qt + kAttnTile + i * 8192), 16, (int)fod[i], 0, 0, 0);
+    }
+    if (threadIdx.x < kAttnBK) {
+      r_t = f_qb + threadIdx.x;
+      const int tc = r_t < q_end ? r_t : q_end - 1;       // q_end > q_begin here: a row that exists
+      r_lse = p.lse[(long long)hq * p.T + tc];
+      r_dl = p.delta[(long long)hq * p.T + tc];
+      r_lo = p.seg_start[tc];
+      r_end = p.seg_end[tc];
+    }
+    f_qb += kAttnBK;
+    if (f_qb >= q_end) f_qb = q_begin, ++f_g;
+  };
+  auto publish = [&](int buf) {                // before the barrier that opens the tile's first interval
+    if (threadIdx.x < kAttnBK) {
+      const bool ok = r_t < q_end;
+      const uint32_t rw = lds0 + kRw + buf * kRows + threadIdx.x * 4;
+      lds_write_u32_asm<0>(rw, __float_as_uint(ok ? r_lse * kLog2e : 0.f));
+      lds_write_u32_asm<kAttnBK * 4>(rw, __float_as_uint(ok ? r_dl : 0.f));
+      lds_write_u32_asm<2 * kAttnBK * 4>(rw, (uint32_t)(ok ? r_lo : 1));
+      lds_write_u32_asm<3 * kAttnBK * 4>(rw, (uint32_t)(ok ? (p.causal ? r_t : r_end - 1) : 0));
+    }
+  };
+  auto barrier = [&]() {
+    wait_lgkm<0>();           // this wavefront's LDS traffic has landed
+    wg_barrier();
+  };
+  // the K / V operand rows are complete here: nothing in the loop may wait for them behind the tile loads it keeps
+  // in flight (the memory counter retires in order)
+#pragma unroll
+  for (int st = 0; st < KS; ++st) asm volatile("" : "+v"(of[st]));
+
+  // all of LDS starts as zeros (see the loop)
+  for (int o = threadIdx.x * 16; o < kAttnDkv2Lds<HD>; o += 512 * 16) lds_write_u128_asm<0>(lds0 + o, u32x4_t{0u, 0u, 0u, 0u});
+  barrier();
+  if (NT > 0) {
+    fetch_next(0);
+    publish(0);
+  }
+  FGRPO_WAIT_VMCNT(0);
+  barrier();
+  // Fragment requests are inline assembly: the value is there after the matching wait, and NOTHING may read the
+  // registers before it.  The compiler does not know that (to it the request defines them), so every value goes
+  // through settle() right after its wait: an empty volatile asm that redefines the registers, which pins every
+  // use behind the wait (volatile asm statements and the wait keep their order; a plain use could otherwise be
+  // hoisted above the wait, e.g. out of both arms of a branch).
+  struct TrFrag {
+    u32x2_t lo, hi;
+  };
+  auto rd_tr = [&](uint32_t tile, auto kbc, int nb) {   // K-major fragment of 16 k rows from kbase, column block dh + nb
+    constexpr int kb = decltype(kbc)::value;
+    TrFrag f;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(f.lo) : "v"(tile + trh[nb][0]), "i"(kb * HD * 2));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(f.hi) : "v"(tile + trh[nb][1]), "i"(kb * HD * 2));
+    return f;
+  };
+  auto settle_tr = [](TrFrag& f) {
+    asm volatile("" : "+v"(f.lo), "+v"(f.hi));
+    return u32x4_t{f.lo.x, f.lo.y, f.hi.x, f.hi.y};
+  };
+  auto settle = [](u32x4_t& v) { asm volatile("" : "+v"(v)); };
+  auto mfma = [](u32x4_t a, u32x4_t b, f32x16_t acc) {
+    return FGRPO_MFMA(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc);
+  };
+  auto fence = []() { __builtin_amdgcn_sched_barrier(0); };
+  constexpr int kTr = 4 * DH;                  // LDS instructions of the transposing fragments of one product's sub-block
+
+  // The loop exists once per role (the roles keep different values across intervals).  An interval is straight-line
+  // code: the requests of a later group are in flight under the matrix instructions of an earlier one, every wait is
+  // counted.  Stages that have nothing to do - the ramps of the pipeline at the ends of a pair's query range, tiles
+  // between them that no key of the pair can see - are not branched around: A's P comes out as exact zeros (every
+  // pair masked), and each role clears what it takes from the partner's slot when that sub-block is not the
+  // pair's (the slot may then hold an older sub-block's values).  All of LDS starts as zeros, so that what such a
+  // stage multiplies by zero is never a NaN pattern.  An interval in which neither stage has work is skipped whole.
+  auto pipeline = [&](auto rolec) {
+    constexpr bool ROLE_A = decltype(rolec)::value;
+    int b_prev = 2, b_cur = 0, b_next = 1;       // LDS buffers of tiles t - 1, t, t + 1
+    int qb_cur = q_begin;
+    bool act_prev = false;
+    float dpd[16];                               // role B: dP - delta of the sub-block before the current one
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dpd[r] = 0.f;
+    for (int t = 0; t <= NT; ++t) {              // the last round only drains the pipeline
+      const uint32_t qt = lds0 + b_cur * 2 * kAttnTile, dot = qt + kAttnTile;
+      const uint32_t qt_prev = lds0 + b_prev * 2 * kAttnTile, dot_prev = qt_prev + kAttnTile;
+      const uint32_t rw = rwl + b_cur * kRows;
+      const bool act_cur = t < NT && wave_on && qb_cur <= wq_hi && qb_cur + kAttnBK > wq_lo;   // the same for both wavefronts of a pair
+      // every (query, key) pair of this step visible: all 64 queries exist, the last one's segment starts at or
+      // before the pair's first key, the first one sees its last key
+      bool all_visible = false;
+      if (ROLE_A && act_cur) {
+        int lo_last, hi_first;
+        asm volatile("ds_read_b32 %0, %2 offset:%3\n\tds_read_b32 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(lo_last), "=&v"(hi_first)
+                     : "v"(lds0 + kRw + b_cur * kRows), "i"(2 * kAttnBK * 4 + (kAttnBK - 1) * 4), "i"(3 * kAttnBK * 4));
+        all_visible = wfirst + 31 < p.T && qb_cur + kAttnBK <= q_end && __builtin_amdgcn_readfirstlane(lo_last) <= wfirst &&
+                      __builtin_amdgcn_readfirstlane(hi_first) >= wlast;
+      }
+      if (t + 1 < NT) fetch_next(b_next);        // b_next was last read two intervals ago (as the tile before the previous one)
+
+      // ---- role A: [Q rows | dS, Q^T of the tile before] S(first half) [dO^T, lse] S(second half) x dK; exp; P out; dV
+      auto run_a = [&](auto mqc) {
+        constexpr int mq = decltype(mqc)::value;
+        u32x4_t fa[KS], dsf[2], l4[4];
+        TrFrag fqk_[2][DH], fdo_[2][DH];
+        f32x16_t sc;
+        static_for<KS>([&](auto stc) { fa[decltype(stc)::value] = lds_read_u128_asm<mq * 32 * HD * 2>(qt + rowc[decltype(stc)::value]); });
+        static_for<2>([&](auto s2c) {
+          constexpr int s2 = decltype(s2c)::value;
+          dsf[s2] = lds_read_u128_asm<mq * 8192 + s2 * 1024>(xd);
+#pragma unroll
+          for (int nb = 0; nb < DH; ++nb) fqk_[s2][nb] = rd_tr(qt_prev, std::integral_constant<int, 32 * mq + 16 * s2>{}, nb);
+        });
+        wait_lgkm<2 + kTr>();                               // the Q rows are there (requested first; LDS returns in order)
+        fence();
+#pragma unroll
+        for (int st = 0; st < KS; ++st) settle(fa[st]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+        for (int st = 0; st < KS / 2; ++st) sc = mfma(fa[st], __builtin_bit_cast(u32x4_t, of[st]), sc);
+        fence();
+        static_for<2>([&](auto s2c) {
+          constexpr int s2 = decltype(s2c)::value;
+#pragma unroll
+          for (int nb = 0; nb < DH; ++nb) fdo_[s2][nb] = rd_tr(dot, std::integral_constant<int, 32 * mq + 16 * s2>{}, nb);
+        });
+        static_for<4>([&](auto gc) { l4[decltype(gc)::value] = lds_read_u128_asm<(32 * mq + 8 * decltype(gc)::value) * 4>(rw); });
+        wait_lgkm<kTr + 4>();                               // dS and the Q^T fragments are there
+        fence();
+        u32x4_t fqk[2][DH];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          settle(dsf[s2]);
+          if (!act_prev) dsf[s2] = u32x4_t{0u, 0u, 0u, 0u};     // the slot holds an older sub-block's dS
+#pragma unroll
+          for (int nb = 0; nb < DH; ++nb) fqk[s2][nb] = settle_tr(fqk_[s2][nb]);
+        }
+        // second half of the S chain and the dK products, alternating
+        static_for<(KS / 2 < 2 * DH ? 2 * DH : KS / 2)>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          if constexpr (i < KS / 2) sc = mfma(fa[KS / 2 + i], __builtin_bit_cast(u32x4_t, of[KS / 2 + i]), sc);
+          if constexpr (i < 2 * DH) acc_k[i % DH] = mfma(dsf[i / DH], fqk[i / DH][i % DH], acc_k[i % DH]);
+        });
+        fence();
+        wait_lgkm<0>();                                     // the dO^T fragments and lse are there
+        fence();
+        u32x4_t fdo[2][DH];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int nb = 0; nb < DH; ++nb) fdo[s2][nb] = settle_tr(fdo_[s2][nb]);
+#pragma unroll
+        for (int grp = 0; grp < 4; ++grp) settle(l4[grp]);
+        float pr[16];
+        if (all_visible) {
+#pragma unroll
+          for (int grp = 0; grp < 4; ++grp)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pr[4 * grp + e] = fast_exp2(__builtin_fmaf(sc[4 * grp + e], c, -__uint_as_float(l4[grp][e])));
+        } else {
+          // the key ranges of the queries: only now, when the registers of the Q fragments are free
+          u32x4_t lo4[4], hi4[4];
+          static_for<4>([&](auto gc) {
+            lo4[decltype(gc)::value] = lds_read_u128_asm<2 * kAttnBK * 4 + (32 * mq + 8 * decltype(gc)::value) * 4>(rw);
+            hi4[decltype(gc)::value] = lds_read_u128_asm<3 * kAttnBK * 4 + (32 * mq + 8 * decltype(gc)::value) * 4>(rw);
+          });
+          wait_lgkm<0>();
+          fence();
+#pragma unroll
+          for (int grp = 0; grp < 4; ++grp) settle(lo4[grp]), settle(hi4[grp]);
+#pragma unroll
+          for (int grp = 0; grp < 4; ++grp)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float x = __builtin_fmaf(sc[4 * grp + e], c, -__uint_as_float(l4[grp][e]));
+              // select before the exponential: a masked pair becomes exp2(-inf) = 0 without a branch; a tile that is not
+              // the pair's (or not there at all: the draining round) has every pair masked
+              x = ((int)(key >= (int)lo4[grp][e]) & (int)(key <= (int)hi4[grp][e]) & (int)act_cur) ? x : -INFINITY;
+              pr[4 * grp + e] = fast_exp2(x);
+            }
+        }
+        static_for<4>([&](auto gc) {
+          constexpr int grp = decltype(gc)::value;
+          lds_write_u128_asm<mq * 16384 + grp * 1024>(xp, u32x4_t{__float_as_uint(pr[4 * grp]), __float_as_uint(pr[4 * grp + 1]),
+                                                                    __float_as_uint(pr[4 * grp + 2]), __float_as_uint(pr[4 * grp + 3])});
+        });
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const u32x4_t pf = __builtin_bit_cast(u32x4_t, attn_pack8(pr + 8 * s2));
+#pragma unroll
+          for (int nb = 0; nb < DH; ++nb) acc_v[nb] = mfma(pf, fdo[s2][nb], acc_v[nb]);
+        }
+      };
+      // ---- role B: [P | dO^T, Q^T of sub-block n - 1, first 16 queries] dS, dS out [first dO rows | the other 16 queries]
+      //      dV, dK (first halves) [other dO rows] dP x (second halves) [delta] dP
+      auto run_b = [&](auto mqc, bool act1) {
+        constexpr int mq = decltype(mqc)::value, mq1 = 1 - mq;
+        // the sub-block before this one: the other half of this tile (mq = 1) or the second half of the previous tile
+        const uint32_t qt1 = mq == 0 ? qt_prev : qt, dot1 = mq == 0 ? dot_prev : dot;
+        u32x4_t fa[KS], p4[4], d4[4], dsf[2], pf[2];
+        TrFrag fq1_[2][DH], fdo1_[2][DH];
+        static_for<4>([&](auto gc) { p4[decltype(gc)::value] = lds_read_u128_asm<mq1 * 16384 + decltype(gc)::value * 1024>(xp); });
+#pragma unroll
+        for (int nb = 0; nb < DH; ++nb) {
+          fdo1_[0][nb] = rd_tr(dot1, std::integral_constant<int, 32 * mq1>{}, nb);
+          fq1_[0][nb] = rd_tr(qt1, std::integral_constant<int, 32 * mq1>{}, nb);
+        }
+        wait_lgkm<kTr>();                                   // P is there (requested first; LDS returns in order)
+        fence();
+        {
+          float ds[16], pr[16];
+#pragma unroll
+          for (int grp = 0; grp < 4; ++grp) {
+            settle(p4[grp]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              pr[4 * grp + e] = act1 ? __uint_as_float(p4[grp][e]) : 0.f;      // else the slot holds an older sub-block's P
+              ds[4 * grp + e] = pr[4 * grp + e] * dpd[4 * grp + e];
+            }
+          }
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            dsf[s2] = __builtin_bit_cast(u32x4_t, attn_pack8(ds + 8 * s2));
+            pf[s2] = __builtin_bit_cast(u32x4_t, attn_pack8(pr + 8 * s2));
+          }
+        }
+        fence();
+        lds_write_u128_asm<mq1 * 8192>(xd, dsf[0]);
+        lds_write_u128_asm<mq1 * 8192 + 1024>(xd, dsf[1]);
+        static_for<KS / 2>([&](auto stc) { fa[decltype(stc)::value] = lds_read_u128_asm<mq * 32 * HD * 2>(dot + rowc[decltype(stc)::value]); });
+#pragma unroll
+        for (int nb = 0; nb < DH; ++nb) {
+          fdo1_[1][nb] = rd_tr(dot1, std::integral_constant<int, 32 * mq1 + 16>{}, nb);
+          fq1_[1][nb] = rd_tr(qt1, std::integral_constant<int, 32 * mq1 + 16>{}, nb);
+        }
+        wait_lgkm<2 + KS / 2 + kTr>();                      // the first transposed fragments are there
+        fence();
+#pragma unroll
+        for (int nb = 0; nb < DH; ++nb) acc_v[nb] = mfma(pf[0], settle_tr(fdo1_[0][nb]), acc_v[nb]);
+#pragma unroll
+        for (int nb = 0; nb < DH; ++nb) acc_k[nb] = mfma(dsf[0], settle_tr(fq1_[0][nb]), acc_k[nb]);
+        fence();
+        static_for<KS / 2>([&](auto stc) {
+          fa[KS / 2 + decltype(stc)::value] = lds_read_u128_asm<mq * 32 * HD * 2>(dot + rowc[KS / 2 + decltype(stc)::value]);
+        });
+        wait_lgkm<KS / 2>();                                // the first dO rows and the other transposed fragments are there
+        fence();
+        u32x4_t fdo1[DH], fq1[DH];
+#pragma unroll
+        for (int nb = 0; nb < DH; ++nb) fdo1[nb] = settle_tr(fdo1_[1][nb]), fq1[nb] = settle_tr(fq1_[1][nb]);
+#pragma unroll
+        for (int st = 0; st < KS / 2; ++st) settle(fa[st]);
+        f32x16_t sc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+        static_for<(KS / 2 < 2 * DH ? 2 * DH : KS / 2)>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          if constexpr (i < KS / 2) sc = mfma(fa[i], __builtin_bit_cast(u32x4_t, of[i]), sc);
+          if constexpr (i < DH) acc_v[i] = mfma(pf[1], fdo1[i], acc_v[i]);
+          else if constexpr (i < 2 * DH) acc_k[i - DH] = mfma(dsf[1], fq1[i - DH], acc_k[i - DH]);
+        });
+        fence();
+        static_for<4>([&](auto gc) { d4[decltype(gc)::value] = lds_read_u128_asm<kAttnBK * 4 + (32 * mq + 8 * decltype(gc)::value) * 4>(rw); });
+        wait_lgkm<4>();                                     // the other dO rows are there (delta on its way)
+        fence();
+#pragma unroll
+        for (int st = KS / 2; st < KS; ++st) {
+          settle(fa[st]);
+          sc = mfma(fa[st], __builtin_bit_cast(u32x4_t, of[st]), sc);
+        }
+        fence();
+        wait_lgkm<0>();
+        fence();
+#pragma unroll
+        for (int grp = 0; grp < 4; ++grp) {
+          settle(d4[grp]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dpd[4 * grp + e] = sc[4 * grp + e] - __uint_as_float(d4[grp][e]);
+        }
+      };
+      static_for<2>([&](auto mqc) {
+        constexpr int mq = decltype(mqc)::value;
+        if constexpr (ROLE_A) {
+          if (act_cur || act_prev) run_a(mqc);
+        } else {
+          const bool act1 = mq == 0 ? act_prev : act_cur;
+          if (act1 || act_cur) run_b(mqc, act1);
+        }
+        if constexpr (mq == 1) {
+          if (t + 1 < NT) publish(b_next);
+          // this wavefront's part of the next tile is in LDS.  Unconditional, so that no fetch counts as pending at
+          // the top of the loop (where the next one is issued and every wait would be for both).
+          FGRPO_WAIT_VMCNT(0);
+        }
+        barrier();
+      });
+      const int bb = b_prev;
+      b_prev = b_cur, b_cur = b_next, b_next = bb;
+      act_prev = act_cur;
+      qb_cur += kAttnBK;
+      if (qb_cur >= q_end) qb_cur = q_begin;
+    }
+  };
+  if (role_a) pipeline(std::true_type{}); else pipeline(std::false_type{});
+  // result lane = column d, rows = keys of this pair
+#pragma unroll
+  for (int nb = 0; nb < DH; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kk = k0 + 32 * pw + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (kk < p.T) {
+        const long long o = ((long long)kk * p.Hkv + hkv) * kHD + 32 * (dh + nb) + (lane & 31);
+        p.dk[o] = f32_to_bf16_rn(acc_k[nb][r] * p.scale);
+        p.dv[o] = f32_to_bf16_rn(acc_v[nb][r]);
+      }
+    }
+}
+
 // seg_start[t], seg_end[t] from cu_seqlens (tokens outside every segment stand alone)
 __global__ void segment_bounds_kernel(const int* cu, int nseq, int T, int* seg_start, int* seg_end) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;

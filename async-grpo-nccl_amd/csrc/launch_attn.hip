@@ -143,8 +143,18 @@ int fgrpo_varlen_attn_bwd(const void* dout, const void* q, const void* k, const 
   rc = launch_query_side<DqLauncher>(D, attn_heads_per_group(Hq / Hkv, T, n_seq), p, T, Hq, Hkv, bounds_ws, st);
   if (rc) return rc;
   const dim3 grid_k(Hkv, (T + kAttnBQ - 1) / kAttnBQ);
-  if (D == 128) hipLaunchKernelGGL(varlen_attn_dkv_kernel<128>, grid_k, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL(varlen_attn_dkv_kernel<64>, grid_k, dim3(256), 0, st, p);
+  if (g_tune.attn_dkv == 1) {
+    if (D == 128) hipLaunchKernelGGL(varlen_attn_dkv_kernel<128>, grid_k, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(varlen_attn_dkv_kernel<64>, grid_k, dim3(256), 0, st, p);
+  } else if (D == 128) {
+    rc = raise_lds<varlen_attn_dkv2_kernel<128>>(kAttnDkv2Lds<128>);
+    if (rc) return rc;
+    hipLaunchKernelGGL(varlen_attn_dkv2_kernel<128>, grid_k, dim3(512), kAttnDkv2Lds<128>, st, p);
+  } else {
+    rc = raise_lds<varlen_attn_dkv2_kernel<64>>(kAttnDkv2Lds<64>);
+    if (rc) return rc;
+    hipLaunchKernelGGL(varlen_attn_dkv2_kernel<64>, grid_k, dim3(512), kAttnDkv2Lds<64>, st, p);
+  }
   HIP_TRY(hipGetLastError());
   return 0;
 }

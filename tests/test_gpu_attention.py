@@ -393,3 +393,44 @@ def test_shared_segment_scratch_gives_identical_results(dev):
         assert all(torch.equal(a, b) for a, b in zip(g1, g2))
     with pytest.raises(RuntimeError, match="bounds"):
         ops.varlen_attn_fwd(q, k, v, cu, None, True, bounds=bounds[:-1])
+
+
+def test_both_key_side_kernels_give_identical_gradients(dev):
+    """dK/dV comes in two kernels: one wavefront per 32 keys, and a pair of wavefronts per 32 keys (the default: one
+    computes S and P, the other dP and dS, each accumulates half of the head dimension).  Same products in the same
+    order: bit-identical dK and dV over short and long segments, tile-edge token counts, both masks, both head
+    dimensions, grouped heads; the single-wavefront kernel also against the oracle.  Twice, so that a result that
+    depended on timing would show."""
+    import random
+    from fgrpo import _lib, ops
+    cases = [(200, [0, 5, 6, 70, 71, 72, 200], 4, 2, True, 128), (200, [0, 5, 6, 70, 71, 72, 200], 4, 2, False, 128),
+             (1000, [0, 130, 385, 390, 900, 1000], 4, 4, True, 128), (1000, [0, 130, 385, 390, 900, 1000], 14, 2, False, 64),
+             (777, [0, 777], 2, 1, True, 128), (4096, [0, 1000, 1001, 3000, 4096], 12, 2, True, 128),
+             (4096, [0, 1000, 1001, 3000, 4096], 12, 2, False, 128), (3000, [0, 3000], 6, 2, True, 64),
+             (1, [0, 1], 2, 2, True, 128), (129, [0, 64, 129], 3, 1, True, 64)]
+    rnd = random.Random(5)
+    for _ in range(10):
+        T = rnd.randint(2, 2500)
+        cuts = sorted(rnd.sample(range(1, T), min(rnd.randint(0, 7), T - 1)))
+        cases.append((T, [0] + cuts + [T], rnd.choice([2, 4, 6]), 2, rnd.random() < 0.7, rnd.choice([64, 128])))
+    try:
+        for i, (T, cu, Hq, Hkv, causal, D) in enumerate(cases):
+            print(f"[attention case] key-side kernels #{i}: T={T} segments={len(cu) - 1} Hq={Hq} Hkv={Hkv} causal={causal} D={D}", flush=True)
+            q, k, v, do = (x.to(dev) for x in make(T, Hq, Hkv, 500 + i, D=D))
+            cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+            out, lse = ops.varlen_attn_fwd(q, k, v, cu_t, None, causal)
+            got = {}
+            for variant in (1, 2, 2):
+                _lib.set_tuning(attn_dkv=variant)
+                g = ops.varlen_attn_bwd(do, q, k, v, out, lse, cu_t, None, causal)
+                torch.cuda.synchronize()
+                if variant in got:
+                    assert all(torch.equal(a, b) for a, b in zip(got[variant], g)), f"case {i}: the paired kernel is not reproducible"
+                got[variant] = g
+            for nm, a, b in zip(("dq", "dk", "dv"), got[1], got[2]):
+                assert torch.equal(a, b), f"case {i}: {nm} differs between the two kernels"
+        _lib.set_tuning(attn_dkv=1)
+        check(dev, "single-wavefront key-side kernel", 1000, [0, 130, 385, 390, 900, 1000], 4, 4, True, seed=2)
+        check(dev, "single-wavefront key-side kernel, head dim 64", 1000, [0, 130, 385, 390, 900, 1000], 14, 2, False, seed=22, D=64)
+    finally:
+        _lib.set_tuning(attn_dkv=0)
