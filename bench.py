@@ -411,11 +411,18 @@ def main():
     ap.add_argument("--attention-shape", choices=["cfg1", "long"], default="cfg1")
     ap.add_argument("--hbm-kernels", action="store_true",
                     help="time the bandwidth-bound kernels of the path instead (prints their own JSON line)")
+    ap.add_argument("--tuning", action="append", default=[], metavar="KEY=VALUE",
+                    help="set a tuning key of the library before anything runs (e.g. attn_dkv=1: the single-wavefront "
+                         "dK/dV kernel); may be given several times")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path shards by micro-batch, one per GPU); "
               "--gpus must be 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.tuning:
+        from fgrpo import _lib
+        _lib.set_tuning(**{k: int(v) for k, v in (kv.split("=", 1) for kv in args.tuning)})
 
     if args.attention:
         return attention_line(args)
