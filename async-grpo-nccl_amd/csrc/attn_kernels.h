@@ -1137,6 +1137,248 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Query-side kernels, second form: the same walk and the same arithmetic in the same order as
+// varlen_attn_fwd_kernel / varlen_attn_dq_kernel (bit-identical results), with the memory side done by hand:
+//  * K / V tiles travel global -> LDS directly (buffer_load ... lds; rows past the end of the keys read as zero) into
+//    two buffers, a step ahead: no staging registers, one barrier per 64-key step instead of two;
+//  * every LDS fragment read is inline assembly, requested in groups a group ahead of the matrix instructions that
+//    use it, with counted waits (left to the compiler, each matrix instruction waits for a fragment requested one
+//    instruction earlier: an LDS round trip per 32-cycle instruction); the dO^T / V^T fragments of the second
+//    product are on their way while the softmax arithmetic runs.
+// Every value an asm read delivers passes through attn_settle() right after its wait (see varlen_attn_dkv2_kernel).
+// ---------------------------------------------------------------------------------------------------------
+struct AttnTr {
+  u32x2_t lo, hi;
+};
+template <int OFF>
+__device__ __forceinline__ AttnTr attn_rd_tr_asm(uint32_t a0, uint32_t a1) {
+  static_assert(OFF >= 0 && OFF < 65536, "DS offset field");
+  AttnTr f;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(f.lo) : "v"(a0), "i"(OFF));
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(f.hi) : "v"(a1), "i"(OFF));
+  return f;
+}
+__device__ __forceinline__ u32x4_t attn_settle_tr(AttnTr& f) {
+  asm volatile("" : "+v"(f.lo), "+v"(f.hi));
+  return u32x4_t{f.lo.x, f.lo.y, f.hi.x, f.hi.y};
+}
+__device__ __forceinline__ void attn_settle(u32x4_t& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ f32x16_t attn_mfma(u32x4_t a, u32x4_t b, f32x16_t acc) {
+  return FGRPO_MFMA(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc);
+}
+
+// Direct-to-LDS fetch of 64-row tiles by a 256-thread work-group: instruction i of wavefront w fills the KiB
+// (4 i + w) of the tile, i.e. rows (4 i + w) * RPI .. with RPI = 1024 / (2 HD); lane l lands at 16 l of that KiB - row
+// l / (HD/8), chunk slot l % (HD/8) - and therefore fetches the chunk the swizzle puts there.  The swizzle of a row
+// depends on the lane and the wavefront only (not on i), so one per-lane byte offset serves every instruction and
+// the step from one to the next is a scalar.
+template <int HD>
+__device__ __forceinline__ uint32_t attn_dma_lane_offset(int wave, int lane, long long st) {
+  constexpr int RPI = 1024 / (HD * 2);
+  const int row = wave * RPI + lane / (HD / 8), ch = (lane % (HD / 8)) ^ attn_swz<HD>(row);
+  return (uint32_t)(((long long)row * st + ch * 8) * 2);
+}
+template <int HD>
+__device__ __forceinline__ void attn_dma_tile(const bf16_t* base, long long st, int row0, int row_end, uint32_t lane_off,
+                                              char* tile_w /* tile + wave * 1024 */) {
+  constexpr int RPI = 1024 / (HD * 2), NLD = kAttnBK / RPI / 4;
+  const long long rows = (long long)row_end - row0;
+  long long bytes = rows > 0 ? (rows - 1) * st * 2 + HD * 2 : 0;
+  if (bytes > 0xffffffffLL) bytes = 0xffffffffLL;
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(base + (long long)row0 * st, (uint32_t)bytes);
+#pragma unroll
+  for (int i = 0; i < NLD; ++i)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, FGRPO_LDS_PTR(tile_w + i * 4096), 16, (int)lane_off, (int)(i * 4 * RPI * st * 2), 0, 0);
+}
+
+template <int HD, int HB>
+__global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) {
+  constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD, G4 = KS / 2;
+  __shared__ __attribute__((aligned(16))) char smem[4 * kAttnTile];      // [buffer][K | V]
+  const uint32_t lds0 = lds_addr(smem);
+  const int lane = threadIdx.x & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const AttnLane<HD> L = attn_lane<HD>(lane);
+  // work-group -> (tile, K/V head, query heads): as in varlen_attn_fwd_kernel
+  constexpr int WPH = 4 / HB, RB = 32 * WPH;
+  const int G = p.Hq / p.Hkv, NB = (G + HB - 1) / HB;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int unit = (slot / NB) * 8 + xcd;
+  const int ntile = (p.T + RB - 1) / RB;
+  if (unit >= ntile * p.Hkv) return;
+  const int hkv = unit % p.Hkv;
+  const int head_g = (slot % NB) * HB + wave / WPH;
+  const bool head_ok = head_g < G;
+  const int hq = hkv * G + (head_ok ? head_g : G - 1);
+  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * RB;
+  const int tq = q0 + 32 * (wave % WPH) + (lane & 31);
+  const bool valid = head_ok && tq < p.T;
+  const int lo = valid ? p.seg_start[tq] : 1;
+  const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
+  const int last = (q0 + RB - 1 < p.T ? q0 + RB - 1 : p.T - 1);
+  const int k_begin = max(__builtin_amdgcn_readfirstlane(p.seg_start[q0]), 0);
+  const int k_end = min(__builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]), p.T);
+  const int wfirst = q0 + 32 * (wave % WPH), wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = head_ok && wfirst < p.T;
+  const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
+  const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
+  const bool wave_full = wave_on && wfirst + 31 < p.T;
+  const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
+  const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
+
+  bf16x8_t qf[KS];
+  attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
+#pragma unroll
+  for (int st = 0; st < KS; ++st) asm volatile("" : "+v"(qf[st]));     // complete before the loop: nothing in it waits for them behind a tile load
+
+  f32x16_t acc_o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_o[db][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale * kLog2e;
+
+  const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
+  const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
+  const uint32_t fko = attn_dma_lane_offset<HD>(wave, lane, p.k_st), fvo = attn_dma_lane_offset<HD>(wave, lane, p.v_st);
+  auto fetch = [&](int kb, int buf) {
+    char* t = smem + buf * 2 * kAttnTile + wave * 1024;
+    attn_dma_tile<HD>(kbase, p.k_st, kb, k_end, fko, t);
+    attn_dma_tile<HD>(vbase, p.v_st, kb, k_end, fvo, t + kAttnTile);
+  };
+  if (k_begin < k_end) fetch(k_begin, 0);
+  FGRPO_WAIT_VMCNT(0);
+  wg_barrier();
+  int cur = 0;
+  for (int kb = k_begin; kb < k_end; kb += kAttnBK, cur ^= 1) {
+    if (kb + kAttnBK < k_end) fetch(kb + kAttnBK, cur ^ 1);     // that buffer was last read a step ago, before the barrier
+    if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
+      const uint32_t kt = lds0 + cur * 2 * kAttnTile, vt = kt + kAttnTile;
+      // ---- S^T = K Q^T: four groups of G4 K fragments (key block mb = g / 2, k steps G4 (g % 2) ..), two groups in flight
+      u32x4_t kf[2][G4];
+      AttnTr vq[2][DB];
+      f32x16_t s[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[mb][r] = 0.f;
+      auto req_k = [&](auto gc) {
+        constexpr int g = decltype(gc)::value;
+        static_for<G4>([&](auto ic) {
+          constexpr int i = decltype(ic)::value, st = G4 * (g % 2) + i;
+          kf[g % 2][i] = lds_read_u128_asm<(g / 2) * 32 * HD * 2>(kt + L.rowc[st]);
+        });
+      };
+      auto req_v = [&](auto qc) {          // V^T fragments of keys 16 q .. 16 q + 15, every 32-column block
+        constexpr int q = decltype(qc)::value;
+        static_for<DB>([&](auto dc) {
+          constexpr int db = decltype(dc)::value;
+          vq[q % 2][db] = attn_rd_tr_asm<16 * q * HD * 2>(vt + L.tr[db][0], vt + L.tr[db][1]);
+        });
+      };
+      auto mma_k = [&](auto gc) {
+        constexpr int g = decltype(gc)::value;
+#pragma unroll
+        for (int i = 0; i < G4; ++i) {
+          attn_settle(kf[g % 2][i]);
+          s[g / 2] = attn_mfma(kf[g % 2][i], __builtin_bit_cast(u32x4_t, qf[G4 * (g % 2) + i]), s[g / 2]);
+        }
+      };
+      using I0 = std::integral_constant<int, 0>;
+      using I1 = std::integral_constant<int, 1>;
+      using I2 = std::integral_constant<int, 2>;
+      using I3 = std::integral_constant<int, 3>;
+      req_k(I0{});
+      req_k(I1{});
+      wait_lgkm<G4>();
+      __builtin_amdgcn_sched_barrier(0);
+      mma_k(I0{});
+      __builtin_amdgcn_sched_barrier(0);
+      req_k(I2{});
+      wait_lgkm<G4>();
+      __builtin_amdgcn_sched_barrier(0);
+      mma_k(I1{});
+      __builtin_amdgcn_sched_barrier(0);
+      req_k(I3{});
+      req_v(I0{});                          // on its way while the softmax arithmetic runs
+      wait_lgkm<G4 + 2 * DB>();
+      __builtin_amdgcn_sched_barrier(0);
+      mma_k(I2{});
+      __builtin_amdgcn_sched_barrier(0);
+      wait_lgkm<2 * DB>();
+      __builtin_amdgcn_sched_barrier(0);
+      mma_k(I3{});
+      __builtin_amdgcn_sched_barrier(0);
+
+      float mx = -INFINITY;
+      if (kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min) {   // every pair of this step is visible
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[mb][r]);
+      } else {
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
+            const float x = (key >= lo && key <= hi) ? s[mb][r] : -INFINITY;
+            s[mb][r] = x;
+            mx = fmaxf(mx, x);
+          }
+      }
+      mx = fmaxf(mx, attn_swap32(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2((m_run - m_use) * c);
+      const float mc = m_use * c;
+      float sum = 0.f;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = fast_exp2(__builtin_fmaf(s[mb][r], c, -mc));
+          s[mb][r] = e;
+          sum += e;
+        }
+      l_run = l_run * alpha + sum;
+      m_run = m_new;
+      if (__any(alpha != 1.f)) {      // once the running maxima have settled no lane rescales any more
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc_o[db][r] *= alpha;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- O^T += V^T P^T: four groups of 16 keys, the next group's fragments requested before this one's products
+      static_for<4>([&](auto qc) {
+        constexpr int q = decltype(qc)::value, mb = q / 2, s2 = q % 2;
+        if constexpr (q < 3) req_v(std::integral_constant<int, q + 1>{});
+        wait_lgkm<(q < 3 ? 2 * DB : 0)>();
+        __builtin_amdgcn_sched_barrier(0);
+        float tmp[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tmp[j] = s[mb][8 * s2 + j];
+        const u32x4_t pf = __builtin_bit_cast(u32x4_t, attn_pack8(tmp));
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc_o[db] = attn_mfma(attn_settle_tr(vq[q % 2][db]), pf, acc_o[db]);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    }
+    FGRPO_WAIT_VMCNT(0);            // this wavefront's part of the next tile is in LDS
+    wait_lgkm<0>();
+    wg_barrier();
+  }
+  const float l = l_run + attn_swap32(l_run);
+  if (valid) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    attn_store_rowmajor(acc_o, inv, p.out + ((long long)tq * p.Hq + hq) * kHD, h);
+    if (h == 0) p.lse[(long long)hq * p.T + tq] = l > 0.f ? m_run * p.scale + __logf(l) : -INFINITY;
+  }
+}
+
 // seg_start[t], seg_end[t] from cu_seqlens (tokens outside every segment stand alone)
 __global__ void segment_bounds_kernel(const int* cu, int nseq, int T, int* seg_start, int* seg_end) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;

@@ -107,6 +107,7 @@ int* tuning_slot(const char* key) {
   if (!strcmp(key, "bwd_kmajor")) return &g_tune.bwd_kmajor;
   if (!strcmp(key, "attn_heads")) return &g_tune.attn_heads;
   if (!strcmp(key, "attn_dkv")) return &g_tune.attn_dkv;
+  if (!strcmp(key, "attn_qside")) return &g_tune.attn_qside;
   if (!strcmp(key, "wide_stores")) return &g_tune.wide_stores;
   if (!strcmp(key, "keep_panels")) return &g_tune.keep_panels;
   if (!strcmp(key, "keep_skip_dead")) return &g_tune.keep_skip_dead;

@@ -39,7 +39,8 @@ int launch_query_side(int D, int hb, AttnParams& p, int T, int Hq, int Hkv, int3
 template <int HD, int HB>
 struct FwdLauncher {
   static void run(dim3 grid, hipStream_t st, const AttnParams& p) {
-    hipLaunchKernelGGL((varlen_attn_fwd_kernel<HD, HB>), grid, dim3(256), 0, st, p);
+    if (g_tune.attn_qside == 1) hipLaunchKernelGGL((varlen_attn_fwd_kernel<HD, HB>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((varlen_attn_fwd2_kernel<HD, HB>), grid, dim3(256), 0, st, p);
   }
 };
 template <int HD, int HB>

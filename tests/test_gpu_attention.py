@@ -434,3 +434,41 @@ def test_both_key_side_kernels_give_identical_gradients(dev):
         check(dev, "single-wavefront key-side kernel, head dim 64", 1000, [0, 130, 385, 390, 900, 1000], 14, 2, False, seed=22, D=64)
     finally:
         _lib.set_tuning(attn_dkv=0)
+
+
+def test_both_forward_kernels_give_identical_results(dev):
+    """The forward comes in two kernels: tiles staged through registers with compiler-scheduled LDS reads, and the
+    default with tiles loaded direct to LDS and hand-scheduled fragment reads.  Same products in the same order:
+    bit-identical out and lse (and therefore gradients) for every heads-per-work-group shape, both head dimensions,
+    both masks, tile-edge token counts; the register-staged kernel also against the oracle.  The default runs twice."""
+    import random
+    from fgrpo import _lib, ops
+    rnd = random.Random(11)
+    cases = [(200, [0, 5, 6, 70, 71, 72, 200], 4, 2, True, 128, 0), (1000, [0, 130, 385, 390, 900, 1000], 14, 2, False, 64, 0),
+             (777, [0, 777], 2, 1, True, 128, 1), (4096, [0, 1000, 1001, 3000, 4096], 12, 2, True, 128, 2),
+             (4096, [0, 1000, 1001, 3000, 4096], 12, 2, False, 128, 4), (3000, [0, 3000], 6, 2, True, 64, 4),
+             (1, [0, 1], 2, 2, True, 128, 0), (129, [0, 64, 129], 3, 1, True, 64, 2), (97, [0, 32, 33, 97], 10, 2, True, 128, 4)]
+    for _ in range(10):
+        T = rnd.randint(2, 2500)
+        cuts = sorted(rnd.sample(range(1, T), min(rnd.randint(0, 7), T - 1)))
+        cases.append((T, [0] + cuts + [T], rnd.choice([2, 4, 6, 14]), 2, rnd.random() < 0.7, rnd.choice([64, 128]), rnd.choice([0, 1, 2, 4])))
+    try:
+        for i, (T, cu, Hq, Hkv, causal, D, hb) in enumerate(cases):
+            print(f"[attention case] forward kernels #{i}: T={T} segments={len(cu) - 1} Hq={Hq} Hkv={Hkv} causal={causal} D={D} heads/wg={hb}", flush=True)
+            q, k, v, do = (x.to(dev) for x in make(T, Hq, Hkv, 700 + i, D=D))
+            cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+            got = {}
+            for variant in (1, 2, 2):
+                _lib.set_tuning(attn_qside=variant, attn_heads=hb)
+                r = ops.varlen_attn_fwd(q, k, v, cu_t, None, causal)
+                torch.cuda.synchronize()
+                if variant in got:
+                    assert all(torch.equal(a, b) for a, b in zip(got[variant], r)), f"case {i}: the default forward is not reproducible"
+                got[variant] = r
+            for nm, a, b in zip(("out", "lse"), got[1], got[2]):
+                assert torch.equal(a, b), f"case {i}: {nm} differs between the two forward kernels"
+        _lib.set_tuning(attn_qside=1, attn_heads=0)
+        check(dev, "register-staged forward", 1000, [0, 130, 385, 390, 900, 1000], 4, 4, True, seed=2, backward=False)
+        check(dev, "register-staged forward, head dim 64", 1000, [0, 130, 385, 390, 900, 1000], 14, 2, False, seed=22, D=64, backward=False)
+    finally:
+        _lib.set_tuning(attn_qside=0, attn_heads=0)
