@@ -22,13 +22,17 @@
 //    dV = P^T dO and dK = dS^T Q products from registers in the same way.
 // LDS tiles are [row][HD] bf16 with the 16-byte chunk index XOR-swizzled by the row (attn_swz): conflict-free both
 // for 16-byte row reads (16 consecutive rows, one chunk) and for the transposing reads (4 consecutive rows x 64 B).
-// Tiles travel global -> registers (bounds-checked buffer loads, issued one step ahead) -> LDS; masks are applied
-// only on steps that can hold a masked pair, and without branches (select before the exponential).
-// Registers: the forward and dQ kernels fit 256 registers and run two wavefronts per SIMD, which is what overlaps
-// one wavefront's softmax arithmetic with the other's MFMAs.  The dK/dV kernel holds two accumulator sets
-// (128 registers) plus its K and V operands and runs one wavefront per SIMD, so its step is software-pipelined
-// by hand (one MFMA per softmax element); splitting it into a dV and a dK launch (two wavefronts per SIMD each,
-// S computed twice) measured slower, as did a second LDS buffer.
+// Masks are applied only on steps that can hold a masked pair, and without branches (select before the exponential).
+// Each of the three kernels exists in two forms with bit-identical results.  The first forms (varlen_attn_fwd_kernel,
+// varlen_attn_dq_kernel, varlen_attn_dkv_kernel) move tiles global -> registers (bounds-checked buffer loads, issued
+// one step ahead) -> LDS and leave the LDS reads to the compiler; the forward and dQ kernels fit 256 registers and
+// run two wavefronts per SIMD, which is what overlaps one wavefront's softmax arithmetic with the other's MFMAs,
+// while the dK/dV kernel holds two accumulator sets (128 registers) plus its K and V operands, runs one wavefront per
+// SIMD and has its step software-pipelined by hand (one MFMA per softmax element); splitting it into a dV and a dK
+// launch (two wavefronts per SIMD each, S computed twice) measured slower, as did a second LDS buffer.  The second
+// forms, the defaults for the forward and for dK/dV (varlen_attn_fwd2_kernel, varlen_attn_dkv2_kernel, further
+// down), move tiles global -> LDS directly and schedule every LDS access by hand; the dK/dV one deals a
+// wavefront's work to a pair so that it, too, runs two wavefronts per SIMD.
 // Launch order: work-groups start in the order of a device-built list, tiles with the most steps first (a third of
 // a launch was tail before), and in the query-side kernels the query heads of one K/V group share an XCD.
 #pragma once
