@@ -30,9 +30,9 @@
 // while the dK/dV kernel holds two accumulator sets (128 registers) plus its K and V operands, runs one wavefront per
 // SIMD and has its step software-pipelined by hand (one MFMA per softmax element); splitting it into a dV and a dK
 // launch (two wavefronts per SIMD each, S computed twice) measured slower, as did a second LDS buffer.  The second
-// forms, the defaults for the forward and for dK/dV (varlen_attn_fwd2_kernel, varlen_attn_dkv2_kernel, further
-// down), move tiles global -> LDS directly and schedule every LDS access by hand; the dK/dV one deals a
-// wavefront's work to a pair so that it, too, runs two wavefronts per SIMD.
+// forms, the defaults (varlen_attn_fwd2_kernel, varlen_attn_dq2_kernel, varlen_attn_dkv2_kernel, further down),
+// move tiles global -> LDS directly and schedule every LDS access by hand; the dK/dV one deals a wavefront's
+// work to a pair so that it, too, runs two wavefronts per SIMD.
 // Launch order: work-groups start in the order of a device-built list, tiles with the most steps first (a third of
 // a launch was tail before), and in the query-side kernels the query heads of one K/V group share an XCD.
 #pragma once
@@ -1203,7 +1203,11 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
   const uint32_t lds0 = lds_addr(smem);
   const int lane = threadIdx.x & 63, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const AttnLane<HD> L = attn_lane<HD>(lane);
+  AttnLane<HD> L = attn_lane<HD>(lane);      // + the LDS base: a fragment address is one of these plus a constant
+#pragma unroll
+  for (int st = 0; st < KS; ++st) L.rowc[st] += (int)lds0;
+#pragma unroll
+  for (int db = 0; db < DB; ++db) L.tr[db][0] += (int)lds0, L.tr[db][1] += (int)lds0;
   // work-group -> (tile, K/V head, query heads): as in varlen_attn_fwd_kernel
   constexpr int WPH = 4 / HB, RB = 32 * WPH;
   const int G = p.Hq / p.Hkv, NB = (G + HB - 1) / HB;
@@ -1255,11 +1259,11 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
   if (k_begin < k_end) fetch(k_begin, 0);
   FGRPO_WAIT_VMCNT(0);
   wg_barrier();
-  int cur = 0;
-  for (int kb = k_begin; kb < k_end; kb += kAttnBK, cur ^= 1) {
+  // a step on LDS buffer `cur`, a compile-time constant: buffer, tile and block are the instruction's offset field
+  auto step = [&](auto curc, int kb) {
+    constexpr int cur = decltype(curc)::value, kt = cur * 2 * kAttnTile, vt = kt + kAttnTile;
     if (kb + kAttnBK < k_end) fetch(kb + kAttnBK, cur ^ 1);     // that buffer was last read a step ago, before the barrier
     if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
-      const uint32_t kt = lds0 + cur * 2 * kAttnTile, vt = kt + kAttnTile;
       // ---- S^T = K Q^T: four groups of G4 K fragments (key block mb = g / 2, k steps G4 (g % 2) ..), two groups in flight
       u32x4_t kf[2][G4];
       AttnTr vq[2][DB];
@@ -1272,14 +1276,14 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
         constexpr int g = decltype(gc)::value;
         static_for<G4>([&](auto ic) {
           constexpr int i = decltype(ic)::value, st = G4 * (g % 2) + i;
-          kf[g % 2][i] = lds_read_u128_asm<(g / 2) * 32 * HD * 2>(kt + L.rowc[st]);
+          kf[g % 2][i] = lds_read_u128_asm<kt + (g / 2) * 32 * HD * 2>((uint32_t)L.rowc[st]);
         });
       };
       auto req_v = [&](auto qc) {          // V^T fragments of keys 16 q .. 16 q + 15, every 32-column block
         constexpr int q = decltype(qc)::value;
         static_for<DB>([&](auto dc) {
           constexpr int db = decltype(dc)::value;
-          vq[q % 2][db] = attn_rd_tr_asm<16 * q * HD * 2>(vt + L.tr[db][0], vt + L.tr[db][1]);
+          vq[q % 2][db] = attn_rd_tr_asm<vt + 16 * q * HD * 2>((uint32_t)L.tr[db][0], (uint32_t)L.tr[db][1]);
         });
       };
       auto mma_k = [&](auto gc) {
@@ -1374,6 +1378,10 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
     FGRPO_WAIT_VMCNT(0);            // this wavefront's part of the next tile is in LDS
     wait_lgkm<0>();
     wg_barrier();
+  };
+  for (int kb = k_begin; kb < k_end; kb += 2 * kAttnBK) {
+    step(std::integral_constant<int, 0>{}, kb);
+    if (kb + kAttnBK < k_end) step(std::integral_constant<int, 1>{}, kb + kAttnBK);
   }
   const float l = l_run + attn_swap32(l_run);
   if (valid) {
@@ -1381,6 +1389,193 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
     attn_store_rowmajor(acc_o, inv, p.out + ((long long)tq * p.Hq + hq) * kHD, h);
     if (h == 0) p.lse[(long long)hq * p.T + tq] = l > 0.f ? m_run * p.scale + __logf(l) : -INFINITY;
   }
+}
+
+// dQ in the same form (see varlen_attn_fwd2_kernel): per 32-key block the K and V row fragments of the two score
+// products arrive in two groups of four k steps each, the K^T fragments of the dQ product are requested while the
+// second group and the softmax arithmetic run.
+template <int HD, int HB>
+__global__ __launch_bounds__(256, 2) void varlen_attn_dq2_kernel(AttnParams p) {
+  constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD, G4 = KS / 2;
+  __shared__ __attribute__((aligned(16))) char smem[4 * kAttnTile];      // [buffer][K | V]
+  const uint32_t lds0 = lds_addr(smem);
+  const int lane = threadIdx.x & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  AttnLane<HD> L = attn_lane<HD>(lane);      // + the LDS base: a fragment address is one of these plus a constant
+#pragma unroll
+  for (int st = 0; st < KS; ++st) L.rowc[st] += (int)lds0;
+#pragma unroll
+  for (int db = 0; db < DB; ++db) L.tr[db][0] += (int)lds0, L.tr[db][1] += (int)lds0;
+  // work-group -> (tile, K/V head, query heads): as in varlen_attn_dq_kernel
+  constexpr int WPH = 4 / HB, RB = 32 * WPH;
+  const int G = p.Hq / p.Hkv, NB = (G + HB - 1) / HB;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int unit = (slot / NB) * 8 + xcd;
+  const int ntile = (p.T + RB - 1) / RB;
+  if (unit >= ntile * p.Hkv) return;
+  const int hkv = unit % p.Hkv;
+  const int head_g = (slot % NB) * HB + wave / WPH;
+  const bool head_ok = head_g < G;
+  const int hq = hkv * G + (head_ok ? head_g : G - 1);
+  const int q0 = min(max(p.order_q[unit / p.Hkv], 0), ntile - 1) * RB;
+  const int tq = q0 + 32 * (wave % WPH) + (lane & 31);
+  const bool valid = head_ok && tq < p.T;
+  const int lo = valid ? p.seg_start[tq] : 1;
+  const int hi = valid ? (p.causal ? tq : p.seg_end[tq] - 1) : 0;
+  const int last = (q0 + RB - 1 < p.T ? q0 + RB - 1 : p.T - 1);
+  const int k_begin = max(__builtin_amdgcn_readfirstlane(p.seg_start[q0]), 0);
+  const int k_end = min(__builtin_amdgcn_readfirstlane(p.causal ? last + 1 : p.seg_end[last]), p.T);
+  const int wfirst = q0 + 32 * (wave % WPH), wlast = (wfirst + 31 < p.T ? wfirst + 31 : p.T - 1);
+  const bool wave_on = head_ok && wfirst < p.T;
+  const int w_lo = wave_on ? p.seg_start[wfirst] : 1;
+  const int w_hi = wave_on ? (p.causal ? wlast : p.seg_end[wlast] - 1) : 0;
+  const bool wave_full = wave_on && wfirst + 31 < p.T;
+  const int w_lo_max = wave_full ? p.seg_start[wlast] : 0x7fffffff;
+  const int w_hi_min = wave_full ? (p.causal ? wfirst : p.seg_end[wfirst] - 1) : -1;
+
+  bf16x8_t qf[KS], dof[KS];
+  attn_row_operand(qf, p.q + (long long)(valid ? tq : 0) * p.q_st + (long long)hq * p.q_sh, valid, h);
+  attn_row_operand(dof, p.dout + ((long long)(valid ? tq : 0) * p.Hq + hq) * kHD, valid, h);
+  const float lse2 = valid ? p.lse[(long long)hq * p.T + tq] * kLog2e : 0.f;
+  // delta = rowsum(dO * O) of the lane's query: each lane half holds alternate 8-element pieces of the row
+  float dl = 0.f;
+  {
+    bf16x8_t of[KS];
+    attn_row_operand(of, p.out_fwd + ((long long)(valid ? tq : 0) * p.Hq + hq) * kHD, valid, h);
+#pragma unroll
+    for (int st = 0; st < KS; ++st) {
+      const u32x4_t x = __builtin_bit_cast(u32x4_t, dof[st]), y = __builtin_bit_cast(u32x4_t, of[st]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        dl += __uint_as_float(x[i] << 16) * __uint_as_float(y[i] << 16);
+        dl += __uint_as_float(x[i] & 0xffff0000u) * __uint_as_float(y[i] & 0xffff0000u);
+      }
+    }
+    dl += attn_swap32(dl);
+    if (valid && h == 0) p.delta[(long long)hq * p.T + tq] = dl;    // for the dK/dV kernel, launched after this one
+  }
+  const float c = p.scale * kLog2e;
+#pragma unroll
+  for (int st = 0; st < KS; ++st) asm volatile("" : "+v"(qf[st]), "+v"(dof[st]));     // complete before the loop
+  float lse2_v = lse2;
+  asm volatile("" : "+v"(lse2_v));
+
+  f32x16_t acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+
+  const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
+  const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
+  const uint32_t fko = attn_dma_lane_offset<HD>(wave, lane, p.k_st), fvo = attn_dma_lane_offset<HD>(wave, lane, p.v_st);
+  auto fetch = [&](int kb, int buf) {
+    char* t = smem + buf * 2 * kAttnTile + wave * 1024;
+    attn_dma_tile<HD>(kbase, p.k_st, kb, k_end, fko, t);
+    attn_dma_tile<HD>(vbase, p.v_st, kb, k_end, fvo, t + kAttnTile);
+  };
+  if (k_begin < k_end) fetch(k_begin, 0);
+  FGRPO_WAIT_VMCNT(0);
+  wg_barrier();
+  // a step on LDS buffer `cur`, a compile-time constant: buffer, tile and block are the instruction's offset field
+  auto step = [&](auto curc, int kb) {
+    constexpr int cur = decltype(curc)::value, kt = cur * 2 * kAttnTile, vt = kt + kAttnTile;
+    if (kb + kAttnBK < k_end) fetch(kb + kAttnBK, cur ^ 1);     // that buffer was last read a step ago, before the barrier
+    if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
+      const bool all_vis = kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min;       // every pair of this step is visible
+      static_for<2>([&](auto mbc) {
+        constexpr int mb = decltype(mbc)::value;
+        constexpr int GQ = KS / 4;            // k steps of a group of row fragments (K and V: 2 GQ reads), four groups, two in flight
+        u32x4_t kf[2][GQ], vf[2][GQ];
+        AttnTr kq[2][DB];
+        f32x16_t sc, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = dp[r] = 0.f;
+        auto req_r = [&](auto gc) {
+          constexpr int g = decltype(gc)::value;
+          static_for<GQ>([&](auto ic) {
+            constexpr int i = decltype(ic)::value, st = GQ * g + i;
+            kf[g % 2][i] = lds_read_u128_asm<kt + mb * 32 * HD * 2>((uint32_t)L.rowc[st]);
+            vf[g % 2][i] = lds_read_u128_asm<vt + mb * 32 * HD * 2>((uint32_t)L.rowc[st]);
+          });
+        };
+        auto mma_r = [&](auto gc) {
+          constexpr int g = decltype(gc)::value;
+#pragma unroll
+          for (int i = 0; i < GQ; ++i) {
+            attn_settle(kf[g % 2][i]);
+            attn_settle(vf[g % 2][i]);
+            sc = attn_mfma(kf[g % 2][i], __builtin_bit_cast(u32x4_t, qf[GQ * g + i]), sc);
+            dp = attn_mfma(vf[g % 2][i], __builtin_bit_cast(u32x4_t, dof[GQ * g + i]), dp);
+          }
+        };
+        auto req_t = [&](auto s2c) {          // K^T fragments of keys 32 mb + 16 s2 .., every 32-column block
+          constexpr int s2 = decltype(s2c)::value;
+          static_for<DB>([&](auto dc) {
+            constexpr int db = decltype(dc)::value;
+            kq[s2][db] = attn_rd_tr_asm<kt + (32 * mb + 16 * s2) * HD * 2>((uint32_t)L.tr[db][0], (uint32_t)L.tr[db][1]);
+          });
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        req_r(I0{});
+        req_r(I1{});
+        wait_lgkm<2 * GQ>();
+        __builtin_amdgcn_sched_barrier(0);
+        mma_r(I0{});
+        __builtin_amdgcn_sched_barrier(0);
+        req_r(I2{});
+        wait_lgkm<2 * GQ>();
+        __builtin_amdgcn_sched_barrier(0);
+        mma_r(I1{});
+        __builtin_amdgcn_sched_barrier(0);
+        req_r(I3{});
+        wait_lgkm<2 * GQ>();
+        __builtin_amdgcn_sched_barrier(0);
+        mma_r(I2{});
+        __builtin_amdgcn_sched_barrier(0);
+        wait_lgkm<0>();
+        __builtin_amdgcn_sched_barrier(0);
+        mma_r(I3{});
+        __builtin_amdgcn_sched_barrier(0);
+        req_t(I0{});                          // on their way while the softmax arithmetic runs
+        req_t(I1{});
+        float ds[16];
+        if (all_vis) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(__builtin_fmaf(sc[r], c, -lse2_v)) * (dp[r] - dl);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int vis = (int)(key >= lo) & (int)(key <= hi);
+            const float pr = fast_exp2(vis ? __builtin_fmaf(sc[r], c, -lse2_v) : -INFINITY);
+            ds[r] = pr * (dp[r] - dl);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<2>([&](auto s2c) {
+          constexpr int s2 = decltype(s2c)::value;
+          wait_lgkm<(s2 == 0 ? 2 * DB : 0)>();
+          __builtin_amdgcn_sched_barrier(0);
+          const u32x4_t dsf = __builtin_bit_cast(u32x4_t, attn_pack8(ds + 8 * s2));
+#pragma unroll
+          for (int db = 0; db < DB; ++db) acc[db] = attn_mfma(attn_settle_tr(kq[s2][db]), dsf, acc[db]);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      });
+    }
+    FGRPO_WAIT_VMCNT(0);            // this wavefront's part of the next tile is in LDS
+    wait_lgkm<0>();
+    wg_barrier();
+  };
+  for (int kb = k_begin; kb < k_end; kb += 2 * kAttnBK) {
+    step(std::integral_constant<int, 0>{}, kb);
+    if (kb + kAttnBK < k_end) step(std::integral_constant<int, 1>{}, kb + kAttnBK);
+  }
+  if (valid) attn_store_rowmajor(acc, p.scale, p.dq + ((long long)tq * p.Hq + hq) * kHD, h);   // dS was kept / scale
 }
 
 // seg_start[t], seg_end[t] from cu_seqlens (tokens outside every segment stand alone)

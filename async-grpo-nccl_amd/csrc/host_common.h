@@ -87,7 +87,7 @@ struct Tuning {
   int small_variant = 4;   // used when a problem has fewer than small_tiles tiles of the big variant
   int bwd_kmajor = 2;      // 0: transposed copies; 1: the dW GEMM reads dLogits and hidden in place; 2: the dH GEMM reads W in place too
   int attn_heads = 0;      // query heads per work-group of the attention forward / dQ kernels (1, 2, 4); 0 = heuristic
-  int attn_qside = 0;      // forward / dQ kernels: 1 = tiles staged through registers, compiler-scheduled LDS reads; 0, 2 = the hand-scheduled form
+  int attn_qside = 0;      // forward / dQ kernels: 1 = tiles staged through registers, compiler-scheduled LDS reads (3: dQ only); 0, 2 = the hand-scheduled forms
   int attn_dkv = 0;        // dK/dV kernel: 1 = one wavefront per 32 keys, 2 = a pair of wavefronts per 32 keys; 0 = default
   int wide_stores = 1;     // GEMM epilogues write 16-byte pieces through an LDS patch where alignment allows
   int keep_skip_dead = 1;  // kept-path backward skips stretches of tokens that carry no gradient

@@ -46,7 +46,8 @@ struct FwdLauncher {
 template <int HD, int HB>
 struct DqLauncher {
   static void run(dim3 grid, hipStream_t st, const AttnParams& p) {
-    hipLaunchKernelGGL((varlen_attn_dq_kernel<HD, HB>), grid, dim3(256), 0, st, p);
+    if (g_tune.attn_qside == 1 || g_tune.attn_qside == 3) hipLaunchKernelGGL((varlen_attn_dq_kernel<HD, HB>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((varlen_attn_dq2_kernel<HD, HB>), grid, dim3(256), 0, st, p);
   }
 };
 }  // namespace

@@ -436,11 +436,11 @@ def test_both_key_side_kernels_give_identical_gradients(dev):
         _lib.set_tuning(attn_dkv=0)
 
 
-def test_both_forward_kernels_give_identical_results(dev):
-    """The forward comes in two kernels: tiles staged through registers with compiler-scheduled LDS reads, and the
-    default with tiles loaded direct to LDS and hand-scheduled fragment reads.  Same products in the same order:
-    bit-identical out and lse (and therefore gradients) for every heads-per-work-group shape, both head dimensions,
-    both masks, tile-edge token counts; the register-staged kernel also against the oracle.  The default runs twice."""
+def test_both_query_side_kernels_give_identical_results(dev):
+    """The forward and the dQ kernel come in two forms: tiles staged through registers with compiler-scheduled LDS
+    reads, and the default with tiles loaded direct to LDS and hand-scheduled fragment reads.  Same products in the
+    same order: bit-identical out, lse and gradients for every heads-per-work-group shape, both head dimensions,
+    both masks, tile-edge token counts; the register-staged kernels also against the oracle.  The default runs twice."""
     import random
     from fgrpo import _lib, ops
     rnd = random.Random(11)
@@ -460,15 +460,16 @@ def test_both_forward_kernels_give_identical_results(dev):
             got = {}
             for variant in (1, 2, 2):
                 _lib.set_tuning(attn_qside=variant, attn_heads=hb)
-                r = ops.varlen_attn_fwd(q, k, v, cu_t, None, causal)
+                out, lse = ops.varlen_attn_fwd(q, k, v, cu_t, None, causal)
+                r = (out, lse) + tuple(ops.varlen_attn_bwd(do, q, k, v, out, lse, cu_t, None, causal))
                 torch.cuda.synchronize()
                 if variant in got:
-                    assert all(torch.equal(a, b) for a, b in zip(got[variant], r)), f"case {i}: the default forward is not reproducible"
+                    assert all(torch.equal(a, b) for a, b in zip(got[variant], r)), f"case {i}: the default kernels are not reproducible"
                 got[variant] = r
-            for nm, a, b in zip(("out", "lse"), got[1], got[2]):
-                assert torch.equal(a, b), f"case {i}: {nm} differs between the two forward kernels"
+            for nm, a, b in zip(("out", "lse", "dq", "dk", "dv"), got[1], got[2]):
+                assert torch.equal(a, b), f"case {i}: {nm} differs between the two forms"
         _lib.set_tuning(attn_qside=1, attn_heads=0)
-        check(dev, "register-staged forward", 1000, [0, 130, 385, 390, 900, 1000], 4, 4, True, seed=2, backward=False)
-        check(dev, "register-staged forward, head dim 64", 1000, [0, 130, 385, 390, 900, 1000], 14, 2, False, seed=22, D=64, backward=False)
+        check(dev, "register-staged query-side kernels", 1000, [0, 130, 385, 390, 900, 1000], 4, 4, True, seed=2)
+        check(dev, "register-staged query-side kernels, head dim 64", 1000, [0, 130, 385, 390, 900, 1000], 14, 2, False, seed=22, D=64)
     finally:
         _lib.set_tuning(attn_qside=0, attn_heads=0)
