@@ -43,8 +43,11 @@ TILE_KERNELS = ("lmhead_fwd_kernel", "lmhead_ds_kernel", "gemm_store_kernel")
 TWO_PER_SIMD = ("TileCfgILi256ELi256ELi64ELi2ELi4ELi2ELi2ELb1EE",      # id 8
                 "TileCfgILi256ELi128ELi32ELi2ELi2ELi2ELi3ELb1EE",      # id 7
                 "TileCfgILi128ELi128ELi64ELi2ELi2ELi2ELi2ELb0EE",      # id 4
-                "varlen_attn_fwd_kernel", "varlen_attn_dq_kernel")
-MUST_EXIST = TILE_KERNELS + ("varlen_attn_fwd_kernel", "varlen_attn_dq_kernel", "varlen_attn_dkv_kernel")
+                "varlen_attn_fwd_kernel", "varlen_attn_dq_kernel",
+                "varlen_attn_fwd2_kernel", "varlen_attn_dq2_kernel", "varlen_attn_dkv2_kernel")
+# attention kernels whose LDS reads are inline assembly: a spilled register could be one whose data is still on its way
+ASM_READ_ATTN = ("varlen_attn_fwd2_kernel", "varlen_attn_dq2_kernel", "varlen_attn_dkv2_kernel")
+MUST_EXIST = TILE_KERNELS + ("varlen_attn_fwd_kernel", "varlen_attn_dq_kernel", "varlen_attn_dkv_kernel") + ASM_READ_ATTN
 
 _FIELDS = {
     "TotalSGPRs": "sgprs", "VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch",
@@ -78,6 +81,9 @@ def check_resource_usage(usage: dict) -> list:
                 seen[key] += 1
         tile = any(k in name for k in TILE_KERNELS)
         if tile and ASM_READ_CFG.search(name) and (u.get("scratch", 0) or u.get("vgpr_spill", 0)):
+            bad.append(f"{name}: inline-assembly fragment reads with {u.get('vgpr_spill')} spilled VGPRs "
+                       f"({u.get('scratch')} B/lane of scratch)")
+        if any(k in name for k in ASM_READ_ATTN) and (u.get("scratch", 0) or u.get("vgpr_spill", 0)):
             bad.append(f"{name}: inline-assembly fragment reads with {u.get('vgpr_spill')} spilled VGPRs "
                        f"({u.get('scratch')} B/lane of scratch)")
         if any(k in name for k in TWO_PER_SIMD) and (tile or "varlen" in name):

@@ -37,7 +37,8 @@ def full_report(**over):
     """A report that names every guarded family once (so that only the kernel under test can trip the guard)."""
     text = remarks(ASM_KERNEL, **over)
     for other in ("lmhead_ds_kernelI_plain", "gemm_store_kernelI_plain", "varlen_attn_fwd_kernelILi128ELi1EE",
-                  "varlen_attn_dq_kernelILi128ELi1EE", "varlen_attn_dkv_kernelILi128EE"):
+                  "varlen_attn_dq_kernelILi128ELi1EE", "varlen_attn_dkv_kernelILi128EE", "varlen_attn_fwd2_kernelILi128ELi1EE",
+                  "varlen_attn_dq2_kernelILi128ELi1EE", "varlen_attn_dkv2_kernelILi128EE"):
         text += "\n" + remarks("_ZN5fgrpo" + other)
     return B.parse_resource_usage(text)
 
@@ -82,3 +83,16 @@ def test_built_library_passed_the_guard():
     for family in B.MUST_EXIST:
         assert any(family in n for n in names)
     assert os.path.getmtime(B.USAGE_PATH) >= os.path.getmtime(B.LIB_PATH) - 5
+
+
+def test_guard_covers_the_hand_scheduled_attention_kernels():
+    """Their LDS reads are inline assembly too: a spill fails the build."""
+    base = full_report()
+    name = "_ZN5fgrpo23varlen_attn_dkv2_kernelILi128EE"
+    assert name in base
+    spilled = dict(base)
+    spilled[name] = dict(base[name], vgpr_spill=3, scratch=12)
+    problems = B.check_resource_usage(spilled)
+    assert problems and any("varlen_attn_dkv2_kernel" in x for x in problems)
+    gone = {k: v for k, v in base.items() if "varlen_attn_dq2_kernel" not in k}
+    assert any("varlen_attn_dq2_kernel" in x for x in B.check_resource_usage(gone))
