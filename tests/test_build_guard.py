@@ -88,7 +88,7 @@ def test_built_library_passed_the_guard():
 def test_guard_covers_the_hand_scheduled_attention_kernels():
     """Their LDS reads are inline assembly too: a spill fails the build."""
     base = full_report()
-    name = "_ZN5fgrpo23varlen_attn_dkv2_kernelILi128EE"
+    name = "_ZN5fgrpovarlen_attn_dkv2_kernelILi128EE"
     assert name in base
     spilled = dict(base)
     spilled[name] = dict(base[name], vgpr_spill=3, scratch=12)
