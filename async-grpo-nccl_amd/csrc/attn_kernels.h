@@ -937,6 +937,9 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
         });
         wait_lgkm<2 + kTr>();                               // the Q rows are there (requested first; LDS returns in order)
         fence();
+        // a wavefront in a run of matrix instructions goes first at the SIMD's issue port: its partner's vector
+        // arithmetic fills the cycles the matrix pipe leaves, not the other way round (-4 % on the kernel)
+        __builtin_amdgcn_s_setprio(2);
 #pragma unroll
         for (int st = 0; st < KS; ++st) settle(fa[st]);
 #pragma unroll
@@ -967,6 +970,7 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
           if constexpr (i < 2 * DH) acc_k[i % DH] = mfma(dsf[i / DH], fqk[i / DH][i % DH], acc_k[i % DH]);
         });
         fence();
+        __builtin_amdgcn_s_setprio(0);
         wait_lgkm<0>();                                     // the dO^T fragments and lse are there
         fence();
         u32x4_t fdo[2][DH];
@@ -1060,6 +1064,7 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
         }
         wait_lgkm<2 + KS / 2 + kTr>();                      // the first transposed fragments are there
         fence();
+        __builtin_amdgcn_s_setprio(2);
 #pragma unroll
         for (int nb = 0; nb < DH; ++nb) acc_v[nb] = mfma(pf[0], settle_tr(fdo1_[0][nb]), acc_v[nb]);
 #pragma unroll
@@ -1094,6 +1099,7 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
           sc = mfma(fa[st], __builtin_bit_cast(u32x4_t, of[st]), sc);
         }
         fence();
+        __builtin_amdgcn_s_setprio(0);
         wait_lgkm<0>();
         fence();
 #pragma unroll
