@@ -180,6 +180,13 @@ __device__ __forceinline__ void attn_row_operand(bf16x8_t (&f)[KS], const bf16_t
 }
 
 __device__ __forceinline__ float attn_swap32(float x) { return __shfl_xor(x, 32, 64); }
+// The same exchange without the LDS round trip of a bpermute: on return `lo` holds, in every lane, the value lane % 32
+// had and `hi` the value lane % 32 + 32 had (v_permlane32_swap: lanes 32..63 of the first operand <-> lanes 0..31 of
+// the second).  fmaxf(lo, hi) and lo + hi are then what fmaxf(x, attn_swap32(x)) and x + attn_swap32(x) give.
+__device__ __forceinline__ void attn_halves(float x, float& lo, float& hi) {
+  lo = x, hi = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lo), "+v"(hi));
+}
 
 // transposed accumulator (4 blocks of 32 d x 32 tokens, the lane's token = its column) -> [token][head][128] bf16
 template <int DB>
@@ -1343,7 +1350,11 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
             mx = fmaxf(mx, x);
           }
       }
-      mx = fmaxf(mx, attn_swap32(mx));
+      {
+        float mlo, mhi;
+        attn_halves(mx, mlo, mhi);
+        mx = fmaxf(mlo, mhi);
+      }
       const float m_new = fmaxf(m_run, mx);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = fast_exp2((m_run - m_use) * c);
@@ -1389,7 +1400,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
     step(std::integral_constant<int, 0>{}, kb);
     if (kb + kAttnBK < k_end) step(std::integral_constant<int, 1>{}, kb + kAttnBK);
   }
-  const float l = l_run + attn_swap32(l_run);
+  float l_lo, l_hi;
+  attn_halves(l_run, l_lo, l_hi);
+  const float l = l_lo + l_hi;
   if (valid) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
     attn_store_rowmajor(acc_o, inv, p.out + ((long long)tq * p.Hq + hq) * kHD, h);
@@ -1397,12 +1410,13 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
   }
 }
 
-// dQ in the same form (see varlen_attn_fwd2_kernel): per 32-key block the K and V row fragments of the two score
-// products arrive in two groups of four k steps each, the K^T fragments of the dQ product are requested while the
-// second group and the softmax arithmetic run.
+// dQ in the same form (see varlen_attn_fwd2_kernel).  A 64-key step runs as six phases of eight matrix instructions
+// with the vector arithmetic of one 32-key half placed behind the matrix instructions of the other (see the step);
+// row fragments arrive in groups of four k steps, two groups in flight, the K^T fragments of the dQ products a
+// phase ahead.
 template <int HD, int HB>
 __global__ __launch_bounds__(256, 2) void varlen_attn_dq2_kernel(AttnParams p) {
-  constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD, G4 = KS / 2;
+  constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD;
   __shared__ __attribute__((aligned(16))) char smem[4 * kAttnTile];      // [buffer][K | V]
   const uint32_t lds0 = lds_addr(smem);
   const int lane = threadIdx.x & 63, h = lane >> 5;
@@ -1463,7 +1477,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq2_kernel(AttnParams p) {
   const float c = p.scale * kLog2e;
 #pragma unroll
   for (int st = 0; st < KS; ++st) asm volatile("" : "+v"(qf[st]), "+v"(dof[st]));     // complete before the loop
-  float lse2_v = lse2;
+  // finite also for a query that sees no key at all (lse = -inf; every pair of such a query is hidden and gets its
+  // zero from the score, see hide() below): -inf * c + inf would be a NaN
+  float lse2_v = lse2 == -INFINITY ? 0.f : lse2;
   asm volatile("" : "+v"(lse2_v));
 
   f32x16_t acc[DB];
@@ -1489,89 +1505,163 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq2_kernel(AttnParams p) {
     if (kb + kAttnBK < k_end) fetch(kb + kAttnBK, cur ^ 1);     // that buffer was last read a step ago, before the barrier
     if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
       const bool all_vis = kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min;       // every pair of this step is visible
-      static_for<2>([&](auto mbc) {
-        constexpr int mb = decltype(mbc)::value;
-        constexpr int GQ = KS / 4;            // k steps of a group of row fragments (K and V: 2 GQ reads), four groups, two in flight
-        u32x4_t kf[2][GQ], vf[2][GQ];
+      // The two 32-key halves of the step as a software pipeline in which the vector arithmetic of a half runs in
+      // the shadow of matrix instructions (a 32x32x16 instruction keeps the matrix pipe busy for 32 cycles and the
+      // issue port for about 8: four or five vector instructions fit behind each one for free, whereas a wavefront
+      // that alternates long runs of the two kinds leaves the pipe idle during its arithmetic).  Eight matrix
+      // instructions a phase:
+      //   S(0) | dP(0) + E(0) | S(1) + F(0) | dP(1) + E(1) | Z(0) + F(1) | Z(1)
+      // S, dP = the score products of a half, E = P = exp2(S c - lse) of its 16 elements, F = dS = P (dP - delta)
+      // and the bf16 operand, Z = dQ += dS K.  Every product and every sum is the one the half-by-half order
+      // computes, in the same order.
+      {
+        constexpr int GR = KS / 2;            // k steps (= LDS reads) of a group of row fragments: two groups a product, two in flight
+        u32x4_t fr[2][GR];
         AttnTr kq[2][DB];
-        f32x16_t sc, dp;
+        f32x16_t sc[2], dp[2];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] = dp[r] = 0.f;
-        auto req_r = [&](auto gc) {
-          constexpr int g = decltype(gc)::value;
-          static_for<GQ>([&](auto ic) {
-            constexpr int i = decltype(ic)::value, st = GQ * g + i;
-            kf[g % 2][i] = lds_read_u128_asm<kt + mb * 32 * HD * 2>((uint32_t)L.rowc[st]);
-            vf[g % 2][i] = lds_read_u128_asm<vt + mb * 32 * HD * 2>((uint32_t)L.rowc[st]);
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[mb][r] = dp[mb][r] = 0.f;
+        auto fence = []() { __builtin_amdgcn_sched_barrier(0); };
+        // group n = 0 .. 7 of the row fragments: product n / 2 (S(0), dP(0), S(1), dP(1)), k steps GR (n % 2) ..
+        auto req_g = [&](auto nc) {
+          constexpr int n = decltype(nc)::value, prod = n / 2, mb = prod / 2, tile = (prod % 2 == 0 ? kt : vt);
+          static_for<GR>([&](auto ic) {
+            constexpr int i = decltype(ic)::value, st = GR * (n % 2) + i;
+            fr[n % 2][i] = lds_read_u128_asm<tile + mb * 32 * HD * 2>((uint32_t)L.rowc[st]);
           });
         };
-        auto mma_r = [&](auto gc) {
-          constexpr int g = decltype(gc)::value;
-#pragma unroll
-          for (int i = 0; i < GQ; ++i) {
-            attn_settle(kf[g % 2][i]);
-            attn_settle(vf[g % 2][i]);
-            sc = attn_mfma(kf[g % 2][i], __builtin_bit_cast(u32x4_t, qf[GQ * g + i]), sc);
-            dp = attn_mfma(vf[g % 2][i], __builtin_bit_cast(u32x4_t, dof[GQ * g + i]), dp);
-          }
-        };
-        auto req_t = [&](auto s2c) {          // K^T fragments of keys 32 mb + 16 s2 .., every 32-column block
-          constexpr int s2 = decltype(s2c)::value;
+        auto req_t = [&](auto mbc, auto s2c) {          // K^T fragments of keys 32 mb + 16 s2 .., every 32-column block
+          constexpr int mb = decltype(mbc)::value, s2 = decltype(s2c)::value;
           static_for<DB>([&](auto dc) {
             constexpr int db = decltype(dc)::value;
             kq[s2][db] = attn_rd_tr_asm<kt + (32 * mb + 16 * s2) * HD * 2>((uint32_t)L.tr[db][0], (uint32_t)L.tr[db][1]);
           });
         };
-        using I0 = std::integral_constant<int, 0>;
-        using I1 = std::integral_constant<int, 1>;
-        using I2 = std::integral_constant<int, 2>;
-        using I3 = std::integral_constant<int, 3>;
-        req_r(I0{});
-        req_r(I1{});
-        wait_lgkm<2 * GQ>();
-        __builtin_amdgcn_sched_barrier(0);
-        mma_r(I0{});
-        __builtin_amdgcn_sched_barrier(0);
-        req_r(I2{});
-        wait_lgkm<2 * GQ>();
-        __builtin_amdgcn_sched_barrier(0);
-        mma_r(I1{});
-        __builtin_amdgcn_sched_barrier(0);
-        req_r(I3{});
-        wait_lgkm<2 * GQ>();
-        __builtin_amdgcn_sched_barrier(0);
-        mma_r(I2{});
-        __builtin_amdgcn_sched_barrier(0);
-        wait_lgkm<0>();
-        __builtin_amdgcn_sched_barrier(0);
-        mma_r(I3{});
-        __builtin_amdgcn_sched_barrier(0);
-        req_t(I0{});                          // on their way while the softmax arithmetic runs
-        req_t(I1{});
-        float ds[16];
-        if (all_vis) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(__builtin_fmaf(sc[r], c, -lse2_v)) * (dp[r] - dl);
-        } else {
+        auto e_el = [&](auto mbc, auto rc) {             // P in place of S
+          constexpr int mb = decltype(mbc)::value, r = decltype(rc)::value;
+          sc[mb][r] = fast_exp2(__builtin_fmaf(sc[mb][r], c, -lse2_v));
+          asm volatile("" : "+v"(sc[mb][r]));      // computed here, behind its matrix instruction: not where the value is next used
+        };
+        // a step with hidden pairs: their scores become -inf between the S and the E phase (exp2 then gives the
+        // exact zero the select in front of the exponential gives; lse2_v is finite).  A branch of its own around
+        // sixteen selects: one around a whole phase costs copies of the accumulators it merges.
+        auto hide = [&](auto mbc) {
+          constexpr int mb = decltype(mbc)::value;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int key = kb + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
-            const int vis = (int)(key >= lo) & (int)(key <= hi);
-            const float pr = fast_exp2(vis ? __builtin_fmaf(sc[r], c, -lse2_v) : -INFINITY);
-            ds[r] = pr * (dp[r] - dl);
+            sc[mb][r] = ((int)(key >= lo) & (int)(key <= hi)) ? sc[mb][r] : -INFINITY;
           }
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        };
+        auto f_el = [&](auto mbc, auto rc) {             // dS in place of P
+          constexpr int mb = decltype(mbc)::value, r = decltype(rc)::value;
+          sc[mb][r] = sc[mb][r] * (dp[mb][r] - dl);
+          asm volatile("" : "+v"(sc[mb][r]));
+        };
+        u32x4_t dsf[2][2];
+        auto pack = [&](auto mbc, auto s2c) {
+          constexpr int mb = decltype(mbc)::value, s2 = decltype(s2c)::value;
+          float tmp[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) tmp[j] = sc[mb][8 * s2 + j];
+          dsf[mb][s2] = __builtin_bit_cast(u32x4_t, attn_pack8(tmp));
+        };
+        // the GR matrix instructions of group n; behind instruction i the vector work side(i)
+        auto mma_g = [&](auto nc, auto&& side) {
+          constexpr int n = decltype(nc)::value, prod = n / 2, mb = prod / 2;
+          static_for<GR>([&](auto ic) {
+            constexpr int i = decltype(ic)::value, st = GR * (n % 2) + i;
+            attn_settle(fr[n % 2][i]);
+            if constexpr (prod % 2 == 0) sc[mb] = attn_mfma(fr[n % 2][i], __builtin_bit_cast(u32x4_t, qf[st]), sc[mb]);
+            else dp[mb] = attn_mfma(fr[n % 2][i], __builtin_bit_cast(u32x4_t, dof[st]), dp[mb]);
+            fence();       // the matrix instruction first: the vector work then runs while the pipe is busy
+            side(ic);
+            fence();
+          });
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        constexpr int EPI = 8 / GR;            // elements behind one matrix instruction: a group covers eight
+        auto none = [](auto) {};
+        auto side_e = [&](auto mbc, auto halfc) {        // E of elements 8 half .. 8 half + 7
+          return [&, mbc, halfc](auto ic) {
+            static_for<EPI>([&](auto jc) { e_el(mbc, std::integral_constant<int, 8 * decltype(halfc)::value + EPI * decltype(ic)::value + decltype(jc)::value>{}); });
+          };
+        };
+        auto side_f = [&](auto mbc, auto halfc) {
+          return [&, mbc, halfc](auto ic) {
+            static_for<EPI>([&](auto jc) { f_el(mbc, std::integral_constant<int, 8 * decltype(halfc)::value + EPI * decltype(ic)::value + decltype(jc)::value>{}); });
+          };
+        };
+        // ---- S(0)
+        req_g(std::integral_constant<int, 0>{});
+        req_g(std::integral_constant<int, 1>{});
+        wait_lgkm<GR>();
+        fence();
+        mma_g(std::integral_constant<int, 0>{}, none);
+        req_g(std::integral_constant<int, 2>{});
+        wait_lgkm<GR>();
+        fence();
+        mma_g(std::integral_constant<int, 1>{}, none);
+        // ---- dP(0) + E(0)
+        req_g(std::integral_constant<int, 3>{});
+        if (!all_vis) hide(I0{});
+        wait_lgkm<GR>();
+        fence();
+        mma_g(std::integral_constant<int, 2>{}, side_e(I0{}, I0{}));
+        req_g(std::integral_constant<int, 4>{});
+        wait_lgkm<GR>();
+        fence();
+        mma_g(std::integral_constant<int, 3>{}, side_e(I0{}, I1{}));
+        // ---- S(1) + F(0)
+        req_g(std::integral_constant<int, 5>{});
+        wait_lgkm<GR>();
+        fence();
+        mma_g(std::integral_constant<int, 4>{}, side_f(I0{}, I0{}));
+        pack(I0{}, I0{});
+        req_g(std::integral_constant<int, 6>{});
+        wait_lgkm<GR>();
+        fence();
+        mma_g(std::integral_constant<int, 5>{}, side_f(I0{}, I1{}));
+        pack(I0{}, I1{});
+        // ---- dP(1) + E(1)
+        req_g(std::integral_constant<int, 7>{});
+        if (!all_vis) hide(I1{});
+        wait_lgkm<GR>();
+        fence();
+        mma_g(std::integral_constant<int, 6>{}, side_e(I1{}, I0{}));
+        req_t(I0{}, I0{});
+        wait_lgkm<2 * DB>();
+        fence();
+        mma_g(std::integral_constant<int, 7>{}, side_e(I1{}, I1{}));
+        // ---- Z(0) + F(1): two elements behind each matrix instruction
+        req_t(I0{}, I1{});
         static_for<2>([&](auto s2c) {
           constexpr int s2 = decltype(s2c)::value;
           wait_lgkm<(s2 == 0 ? 2 * DB : 0)>();
-          __builtin_amdgcn_sched_barrier(0);
-          const u32x4_t dsf = __builtin_bit_cast(u32x4_t, attn_pack8(ds + 8 * s2));
-#pragma unroll
-          for (int db = 0; db < DB; ++db) acc[db] = attn_mfma(attn_settle_tr(kq[s2][db]), dsf, acc[db]);
-          __builtin_amdgcn_sched_barrier(0);
+          fence();
+          static_for<DB>([&](auto dc) {
+            constexpr int db = decltype(dc)::value;
+            acc[db] = attn_mfma(attn_settle_tr(kq[s2][db]), dsf[0][s2], acc[db]);
+            fence();
+            static_for<8 / DB>([&](auto jc) { f_el(I1{}, std::integral_constant<int, 8 * s2 + (8 / DB) * db + decltype(jc)::value>{}); });
+            fence();
+          });
+          pack(I1{}, s2c);
+          req_t(I1{}, s2c);
         });
-      });
+        // ---- Z(1)
+        static_for<2>([&](auto s2c) {
+          constexpr int s2 = decltype(s2c)::value;
+          wait_lgkm<(s2 == 0 ? 2 * DB : 0)>();
+          fence();
+#pragma unroll
+          for (int db = 0; db < DB; ++db) acc[db] = attn_mfma(attn_settle_tr(kq[s2][db]), dsf[1][s2], acc[db]);
+          fence();
+        });
+      }
     }
     FGRPO_WAIT_VMCNT(0);            // this wavefront's part of the next tile is in LDS
     wait_lgkm<0>();
