@@ -1545,7 +1545,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq2_kernel(AttnParams p) {
           asm volatile("" : "+v"(sc[mb][r]));      // computed here, behind its matrix instruction: not where the value is next used
         };
         // a step with hidden pairs: their scores become -inf between the S and the E phase (exp2 then gives the
-        // exact zero the select in front of the exponential gives; lse2_v is finite).  A branch of its own around
+        // exact zero the select in front of the exponential gives: lse2_v is finite and the scale positive, which the
+        // host checks).  A branch of its own around
         // sixteen selects: one around a whole phase costs copies of the accumulators it merges.
         auto hide = [&](auto mbc) {
           constexpr int mb = decltype(mbc)::value;
