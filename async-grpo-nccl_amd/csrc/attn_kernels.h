@@ -815,16 +815,29 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
   // instruction that touches them would wait for the tile loads issued before them too - the memory counter retires in order)
   float r_lse = 0.f, r_dl = 0.f;
   int r_lo = 0, r_end = 0, r_t = 0;
-  auto fetch_next = [&](int buf) {             // tile -> LDS buffer buf (in flight until publish()), its scalars -> registers
+  // The descriptors of the next tile move by additions (down a head's queries 64 at a time) and are formed from
+  // scratch only when the walk starts the next head: every wavefront does this scalar work at the same moment, at the
+  // top of a tile's first interval, before its first LDS request.
+  const char *f_qp = nullptr, *f_dp = nullptr;                   // first row of the next tile
+  long long f_qbytes = 0, f_dbytes = 0;                          // from there to the end of the head's last query row
+  const float *f_lse = nullptr, *f_delta = nullptr;              // the head's per-query scalars
+  const long long f_qstep = (long long)kAttnBK * p.q_st * 2, f_dstep = (long long)kAttnBK * do_st * 2;
+  auto fetch_head = [&]() {                    // the walk is at the first tile of head f_g
     const int hq = hkv * G + f_g;
-    const bf16_t* qbase = p.q + (long long)hq * p.q_sh;
-    const bf16_t* dobase = p.dout + (long long)hq * kHD;
-    const long long rows = (long long)q_end - f_qb;
-    long long bq = rows > 0 ? (rows - 1) * p.q_st * 2 + HD * 2 : 0, bd = rows > 0 ? (rows - 1) * do_st * 2 + HD * 2 : 0;
+    f_qp = (const char*)(p.q + (long long)hq * p.q_sh + (long long)q_begin * p.q_st);
+    f_dp = (const char*)(p.dout + (long long)hq * kHD + (long long)q_begin * do_st);
+    f_qbytes = ((long long)q_end - q_begin - 1) * p.q_st * 2 + HD * 2;      // strides >= HD: not positive past the end
+    f_dbytes = ((long long)q_end - q_begin - 1) * do_st * 2 + HD * 2;
+    f_lse = p.lse + (long long)hq * p.T;
+    f_delta = p.delta + (long long)hq * p.T;
+  };
+  auto fetch_next = [&](int buf) {             // tile -> LDS buffer buf (in flight until publish()), its scalars -> registers
+    if (f_qb == q_begin) fetch_head();
+    long long bq = f_qbytes > 0 ? f_qbytes : 0, bd = f_dbytes > 0 ? f_dbytes : 0;
     if (bq > 0xffffffffLL) bq = 0xffffffffLL;
     if (bd > 0xffffffffLL) bd = 0xffffffffLL;
-    const __amdgpu_buffer_rsrc_t rsq = make_rsrc(qbase + (long long)f_qb * p.q_st, (uint32_t)bq);
-    const __amdgpu_buffer_rsrc_t rsd = make_rsrc(dobase + (long long)f_qb * do_st, (uint32_t)bd);
+    const __amdgpu_buffer_rsrc_t rsq = make_rsrc(f_qp, (uint32_t)bq);
+    const __amdgpu_buffer_rsrc_t rsd = make_rsrc(f_dp, (uint32_t)bd);
     char* qt = smem + buf * 2 * kAttnTile + wave * 1024;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
@@ -834,12 +847,13 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
     if (threadIdx.x < kAttnBK) {
       r_t = f_qb + threadIdx.x;
       const int tc = r_t < q_end ? r_t : q_end - 1;       // q_end > q_begin here: a row that exists
-      r_lse = p.lse[(long long)hq * p.T + tc];
-      r_dl = p.delta[(long long)hq * p.T + tc];
+      r_lse = f_lse[tc];
+      r_dl = f_delta[tc];
       r_lo = p.seg_start[tc];
       r_end = p.seg_end[tc];
     }
     f_qb += kAttnBK;
+    f_qp += f_qstep, f_dp += f_dstep, f_qbytes -= f_qstep, f_dbytes -= f_dstep;
     if (f_qb >= q_end) f_qb = q_begin, ++f_g;
   };
   auto publish = [&](int buf) {                // before the barrier that opens the tile's first interval
@@ -1209,6 +1223,33 @@ __device__ __forceinline__ void attn_dma_tile(const bf16_t* base, long long st, 
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, FGRPO_LDS_PTR(tile_w + i * 4096), 16, (int)lane_off, (int)(i * 4 * RPI * st * 2), 0, 0);
 }
 
+// The descriptor of the next 64-row tile, kept up to date by additions: the walk goes down the rows 64 at a time,
+// and forming `base + row0 * st` and the byte count from scratch costs four 64-bit multiplications a tile - scalar
+// work at the top of a step, which every wavefront of the work-group does at the same moment, right behind the
+// barrier, before its first LDS request.  bytes = distance from the tile's first row to the end of the last row there
+// is (row_end - 1); zero or less when the walk has passed the end: the loads then write zeros.
+template <int HD>
+struct AttnTileCursor {
+  const char* ptr;
+  long long bytes, step;
+  __device__ __forceinline__ void init(const bf16_t* base, long long st, int row0, int row_end) {
+    ptr = (const char*)(base + (long long)row0 * st);
+    bytes = ((long long)row_end - row0 - 1) * st * 2 + HD * 2;      // st >= HD: not positive from row0 = row_end on
+    step = (long long)kAttnBK * st * 2;
+  }
+  __device__ __forceinline__ void next() { ptr += step, bytes -= step; }
+  // loads of the tile at the cursor, by a 256-thread work-group (see attn_dma_tile)
+  __device__ __forceinline__ void load(long long st, uint32_t lane_off, char* tile_w) const {
+    constexpr int RPI = 1024 / (HD * 2), NLD = kAttnBK / RPI / 4;
+    long long b = bytes > 0 ? bytes : 0;
+    if (b > 0xffffffffLL) b = 0xffffffffLL;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(ptr, (uint32_t)b);
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, FGRPO_LDS_PTR(tile_w + i * 4096), 16, (int)lane_off, (int)(i * 4 * RPI * st * 2), 0, 0);
+  }
+};
+
 template <int HD, int HB>
 __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) {
   constexpr int KS = HD / 16, DB = HD / 32, kAttnTile = kAttnBK * HD * 2, kHD = HD, G4 = KS / 2;
@@ -1264,18 +1305,23 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_fwd2_kernel(AttnParams p) 
   const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
   const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
   const uint32_t fko = attn_dma_lane_offset<HD>(wave, lane, p.k_st), fvo = attn_dma_lane_offset<HD>(wave, lane, p.v_st);
-  auto fetch = [&](int kb, int buf) {
+  AttnTileCursor<HD> ck, cv;               // the tile the next fetch brings: the steps are fetched in order
+  ck.init(kbase, p.k_st, k_begin, k_end);
+  cv.init(vbase, p.v_st, k_begin, k_end);
+  auto fetch = [&](int buf) {
     char* t = smem + buf * 2 * kAttnTile + wave * 1024;
-    attn_dma_tile<HD>(kbase, p.k_st, kb, k_end, fko, t);
-    attn_dma_tile<HD>(vbase, p.v_st, kb, k_end, fvo, t + kAttnTile);
+    ck.load(p.k_st, fko, t);
+    cv.load(p.v_st, fvo, t + kAttnTile);
+    ck.next();
+    cv.next();
   };
-  if (k_begin < k_end) fetch(k_begin, 0);
+  if (k_begin < k_end) fetch(0);
   FGRPO_WAIT_VMCNT(0);
   wg_barrier();
   // a step on LDS buffer `cur`, a compile-time constant: buffer, tile and block are the instruction's offset field
   auto step = [&](auto curc, int kb) {
     constexpr int cur = decltype(curc)::value, kt = cur * 2 * kAttnTile, vt = kt + kAttnTile;
-    if (kb + kAttnBK < k_end) fetch(kb + kAttnBK, cur ^ 1);     // that buffer was last read a step ago, before the barrier
+    if (kb + kAttnBK < k_end) fetch(cur ^ 1);     // the next step's tiles; that buffer was last read a step ago, before the barrier
     if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
       // ---- S^T = K Q^T: four groups of G4 K fragments (key block mb = g / 2, k steps G4 (g % 2) ..), two groups in flight
       u32x4_t kf[2][G4];
@@ -1491,18 +1537,23 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dq2_kernel(AttnParams p) {
   const bf16_t* kbase = p.k + (long long)hkv * p.k_sh;
   const bf16_t* vbase = p.v + (long long)hkv * p.v_sh;
   const uint32_t fko = attn_dma_lane_offset<HD>(wave, lane, p.k_st), fvo = attn_dma_lane_offset<HD>(wave, lane, p.v_st);
-  auto fetch = [&](int kb, int buf) {
+  AttnTileCursor<HD> ck, cv;               // the tile the next fetch brings: the steps are fetched in order
+  ck.init(kbase, p.k_st, k_begin, k_end);
+  cv.init(vbase, p.v_st, k_begin, k_end);
+  auto fetch = [&](int buf) {
     char* t = smem + buf * 2 * kAttnTile + wave * 1024;
-    attn_dma_tile<HD>(kbase, p.k_st, kb, k_end, fko, t);
-    attn_dma_tile<HD>(vbase, p.v_st, kb, k_end, fvo, t + kAttnTile);
+    ck.load(p.k_st, fko, t);
+    cv.load(p.v_st, fvo, t + kAttnTile);
+    ck.next();
+    cv.next();
   };
-  if (k_begin < k_end) fetch(k_begin, 0);
+  if (k_begin < k_end) fetch(0);
   FGRPO_WAIT_VMCNT(0);
   wg_barrier();
   // a step on LDS buffer `cur`, a compile-time constant: buffer, tile and block are the instruction's offset field
   auto step = [&](auto curc, int kb) {
     constexpr int cur = decltype(curc)::value, kt = cur * 2 * kAttnTile, vt = kt + kAttnTile;
-    if (kb + kAttnBK < k_end) fetch(kb + kAttnBK, cur ^ 1);     // that buffer was last read a step ago, before the barrier
+    if (kb + kAttnBK < k_end) fetch(cur ^ 1);     // the next step's tiles; that buffer was last read a step ago, before the barrier
     if (wave_on && kb <= w_hi && kb + kAttnBK > w_lo) {
       const bool all_vis = kb >= w_lo_max && kb + kAttnBK - 1 <= w_hi_min;       // every pair of this step is visible
       // The two 32-key halves of the step as a software pipeline in which the vector arithmetic of a half runs in
