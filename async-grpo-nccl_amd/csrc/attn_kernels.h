@@ -941,7 +941,11 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
         all_visible = wfirst + 31 < p.T && qb_cur + kAttnBK <= q_end && __builtin_amdgcn_readfirstlane(lo_last) <= wfirst &&
                       __builtin_amdgcn_readfirstlane(hi_first) >= wlast;
       }
-      if (t + 1 < NT) fetch_next(b_next);        // b_next was last read two intervals ago (as the tile before the previous one)
+      // The next tile is fetched (descriptors, loads, wave 0's scalars) from inside the tile's first interval, behind
+      // the first run of matrix instructions: at the top of the loop every wavefront would do that work at the same
+      // moment, right behind the barrier, before its first LDS request.  b_next was last read two intervals ago (as
+      // the tile before the previous one).
+      const bool do_fetch = t + 1 < NT;
 
       // ---- role A: [Q rows | dS, Q^T of the tile before] S(first half) [dO^T, lse] S(second half) x dK; exp; P out; dV
       auto run_a = [&](auto mqc) {
@@ -968,6 +972,10 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
 #pragma unroll
         for (int st = 0; st < KS / 2; ++st) sc = mfma(fa[st], __builtin_bit_cast(u32x4_t, of[st]), sc);
         fence();
+        if constexpr (mq == 0) {
+          if (do_fetch) fetch_next(b_next);
+          fence();
+        }
         static_for<2>([&](auto s2c) {
           constexpr int s2 = decltype(s2c)::value;
 #pragma unroll
@@ -1091,6 +1099,10 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
 #pragma unroll
         for (int nb = 0; nb < DH; ++nb) acc_k[nb] = mfma(dsf[0], settle_tr(fq1_[0][nb]), acc_k[nb]);
         fence();
+        if constexpr (mq == 0) {
+          if (do_fetch) fetch_next(b_next);
+          fence();
+        }
         static_for<KS / 2>([&](auto stc) {
           fa[KS / 2 + decltype(stc)::value] = lds_read_u128_asm<mq * 32 * HD * 2>(dot + rowc[KS / 2 + decltype(stc)::value]);
         });
@@ -1134,9 +1146,11 @@ __global__ __launch_bounds__(512) void varlen_attn_dkv2_kernel(AttnParams p) {
         constexpr int mq = decltype(mqc)::value;
         if constexpr (ROLE_A) {
           if (act_cur || act_prev) run_a(mqc);
+          else if (mq == 0 && do_fetch) fetch_next(b_next);
         } else {
           const bool act1 = mq == 0 ? act_prev : act_cur;
           if (act1 || act_cur) run_b(mqc, act1);
+          else if (mq == 0 && do_fetch) fetch_next(b_next);
         }
         if constexpr (mq == 1) {
           if (t + 1 < NT) publish(b_next);
